@@ -1,0 +1,211 @@
+/*
+ * libmmsim -- MI355X (gfx950) evaluation of candidate model placements with
+ * AlpaServe's approximate serving simulator.
+ *
+ * Plain C ABI: opaque handles, plain pointers and sizes, integer status codes.
+ * Every entry point returns MMSIM_OK (0) or a negative MMSIM_E_* code; a
+ * human-readable message for the last failure on the calling thread is
+ * available from mmsim_last_error().  No entry point retains a host pointer
+ * after it returns.  A context and the objects made from it must be used by
+ * one thread at a time.  There is no CPU fallback: without a usable HIP
+ * device mmsim_ctx_create fails.
+ *
+ * What each entry point stands in for in the reference (alpa-projects/mms):
+ *
+ *   mmsim_simulate_requests_mixed
+ *       the numba kernel simulate_requests_mixed, same argument list
+ *       (alpa_serve/simulator/controller.py:561-628; called at :491-494).
+ *   mmsim_simulate_requests_mixed_batching
+ *       simulate_requests_mixed_batching, same argument list
+ *       (alpa_serve/simulator/controller.py:631-798; called at :486-489).
+ *   mmsim_workload_create
+ *       the per-workload arrays approximate_one_case derives once and caches:
+ *       arrivals, model_ids (int32) and slos (float32)
+ *       (alpa_serve/simulator/controller.py:321-339).
+ *   mmsim_batch_create / _run / _sync / _fetch, mmsim_eval_batch
+ *       the loop "for sol in sols: approximate_one_case(...)" of
+ *       PlacementEvaluator.get_scores / get_stats
+ *       (alpa_serve/placement_policy/base_policy.py:175-189, 191-264), i.e.
+ *       approximate_one_case_one_placement's table build
+ *       (controller.py:412-476) plus the request loop for every placement
+ *       of the list, and the reductions of the fast-stats epilogue
+ *       (controller.py:393-403: number of good requests, sum of latencies).
+ */
+#ifndef MMSIM_H_
+#define MMSIM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MMSIM_ABI_VERSION 1
+
+enum {
+    MMSIM_OK = 0,
+    MMSIM_E_INVALID = -1,     /* bad argument (null pointer, negative size, index out of range) */
+    MMSIM_E_UNSUPPORTED = -2, /* shape outside the compiled kernel buckets                      */
+    MMSIM_E_HIP = -3,         /* a HIP runtime call failed                                      */
+    MMSIM_E_NOMEM = -4,       /* host or device allocation failed                               */
+    MMSIM_E_OVERFLOW = -5     /* a lane ran out of idle-event slots (batching); see status[]    */
+};
+
+/* Limits of the compiled kernels. */
+#define MMSIM_MAX_STAGES 32        /* pipeline stages of one group                */
+#define MMSIM_MAX_REPLICAS 64      /* groups hosting one model in one placement   */
+#define MMSIM_MAX_GROUPS 255       /* groups of one placement                     */
+#define MMSIM_MAX_SLOTS 255        /* sum of pipeline stages over a placement     */
+#define MMSIM_MAX_CONFIGS 255      /* distinct parallel configurations            */
+
+typedef struct mmsim_ctx mmsim_ctx;
+typedef struct mmsim_workload mmsim_workload;
+typedef struct mmsim_batch mmsim_batch;
+
+int mmsim_abi_version(void);
+const char *mmsim_last_error(void);
+
+/* Binds a context to HIP device `device` and creates its stream. */
+int mmsim_ctx_create(int device, mmsim_ctx **out);
+void mmsim_ctx_destroy(mmsim_ctx *ctx);
+
+typedef struct {
+    char name[128];
+    char arch[64];
+    int32_t compute_units;
+    int32_t clock_khz;
+    int32_t lds_bytes_per_block;
+    int64_t hbm_bytes;
+} mmsim_device_info;
+int mmsim_ctx_device_info(mmsim_ctx *ctx, mmsim_device_info *out);
+
+/*
+ * One request stream (one arrival seed), copied to device memory.
+ *   tstamps   [R] arrival times in the order the requests are to be processed
+ *   model_ids [R] model index in [0, M) or negative for "not registered"
+ *   slos      [R] float32 seconds; +inf = never dropped, NaN = always dropped
+ */
+int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M,
+                          const double *tstamps, const int32_t *model_ids,
+                          const float *slos, mmsim_workload **out);
+void mmsim_workload_destroy(mmsim_workload *wl);
+
+/*
+ * Latency table shared by all placements of a batch: what
+ * approximate_one_case_one_placement computes per (model, group) depends only
+ * on the group's parallel configuration, so it is given once per distinct
+ * configuration.
+ *   cfg_lat [M][C][Smax][NB]  float32( stage latency * (1 + 0.009*pp) ), or
+ *                             +inf for a configuration the model has no
+ *                             profile for; entries k >= cfg_pp[c] are ignored
+ *   cfg_pp  [C]               pipeline stages of configuration c (1..Smax)
+ *   batch_sizes [NB]          batch sizes, batch_sizes[0] == 1; only column 0
+ *                             is used without MMSIM_BATCHING
+ */
+typedef struct {
+    int32_t M, C, Smax, NB;
+    const float *cfg_lat;
+    const int32_t *cfg_pp;
+    const int32_t *batch_sizes;
+    double fixed_overhead; /* 0.011 in the reference */
+} mmsim_tables;
+
+/*
+ * B candidate placements.  Placement b has num_groups[b] groups; group g uses
+ * configuration group_cfg[b*Gmax+g] and hosts the models
+ *   gm_idx[ gm_off[b*(Gmax+1)+g] .. gm_off[b*(Gmax+1)+g+1] )
+ * in the order given (the order of ModelPlacement.group_models[g]).
+ */
+typedef struct {
+    int32_t B, Gmax;
+    const int32_t *num_groups;
+    const int32_t *group_cfg;
+    const int64_t *gm_off;
+    const int32_t *gm_idx;
+} mmsim_placements;
+
+/* flags */
+#define MMSIM_BATCHING 1u          /* batching simulator instead of the plain one */
+#define MMSIM_WANT_MODEL_COUNTS 2u /* fill model_num_requests / model_num_good     */
+#define MMSIM_WANT_GROUP_COUNTS 4u /* fill group_num_requests / group_num_good     */
+#define MMSIM_WANT_PER_REQUEST 8u  /* fill finish / good for every request         */
+#define MMSIM_WANT_OP_COUNT 16u    /* fill fp_ops (plain simulator only)            */
+
+/*
+ * Results, caller-allocated.  Simulation ("lane") l = seed * B + b.
+ * Pointers not asked for by the flags may be null.
+ */
+typedef struct {
+    int64_t *n_good;             /* [L]        accepted requests                                    */
+    double *latency_sum;         /* [L]        sum of (finish - arrival) over requests in arrival order */
+    int32_t *model_num_requests; /* [L][M]     */
+    int32_t *model_num_good;     /* [L][M]     */
+    int32_t *group_num_requests; /* [L][Gmax]  */
+    int32_t *group_num_good;     /* [L][Gmax]  */
+    double *finish;              /* [L][Rmax]  Rmax = longest stream of the batch; row tail unspecified */
+    uint8_t *good;               /* [L][Rmax]  */
+    int32_t *status;             /* [L]        0, or MMSIM_E_OVERFLOW for a lane whose results are invalid */
+    int64_t *fp_ops;             /* [L]        sum over dispatched requests of 2*stages + replicas + 3:
+                                               the fp64 max/add/compare operations the reference's loop
+                                               performs (controller.py:590-613) */
+} mmsim_result;
+
+/* Packs the placements, uploads them and allocates device result buffers. */
+int mmsim_batch_create(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                       const mmsim_tables *tables, const mmsim_placements *placements,
+                       uint32_t flags, mmsim_batch **out);
+/* Enqueues the simulation kernels on the context's stream (asynchronous). */
+int mmsim_batch_run(mmsim_batch *batch);
+/* Waits for the last run.  kernel_ms (optional) receives the time between HIP
+ * events recorded on the stream right before and after the simulation kernel. */
+int mmsim_batch_sync(mmsim_batch *batch, float *kernel_ms);
+/* Copies results of the last completed run into caller memory. */
+int mmsim_batch_fetch(mmsim_batch *batch, mmsim_result *out);
+void mmsim_batch_destroy(mmsim_batch *batch);
+
+typedef struct {
+    int32_t lanes, waves, n_seeds, B;
+    int32_t smax_bucket, rmax_bucket, slots, lds_bytes;
+    int64_t requests_total;   /* sum of stream lengths over seeds                     */
+    int64_t table_bytes;      /* device bytes of the packed placement tables          */
+    int64_t stream_bytes;     /* device bytes of the request streams                  */
+} mmsim_batch_info;
+int mmsim_batch_get_info(const mmsim_batch *batch, mmsim_batch_info *out);
+
+/* create + run + sync + fetch + destroy */
+int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                     const mmsim_tables *tables, const mmsim_placements *placements,
+                     uint32_t flags, mmsim_result *out);
+
+/*
+ * Single-placement calls with the argument lists of the reference's kernels.
+ * finish [R] and good [R] are written for every request; the four count
+ * arrays are zeroed and filled.  Layouts:
+ *   m_id2g_id     [M][G]  replica groups of each model, -1 terminated
+ *   g_id2m_id     [G][M]  models of each group, -1 terminated (batching only)
+ *   num_stages    [G]
+ *   stage_latency [M][G][Smax]        (plain)   float32
+ *                 [M][G][Smax][NB]    (batching)
+ */
+int mmsim_simulate_requests_mixed(
+    mmsim_ctx *ctx, double *finish, uint8_t *good, const double *tstamps,
+    const int32_t *model_ids, const float *slos, const int32_t *m_id2g_id,
+    const int32_t *num_stages, const float *stage_latency, int64_t num_requests,
+    int32_t M, int32_t G, int32_t Smax, double fixed_overhead,
+    int32_t *model_num_requests, int32_t *model_num_good_requests,
+    int32_t *group_num_requests, int32_t *group_num_good_requests);
+
+int mmsim_simulate_requests_mixed_batching(
+    mmsim_ctx *ctx, double *finish, uint8_t *good, const double *tstamps,
+    const int32_t *model_ids, const float *slos, const int32_t *m_id2g_id,
+    const int32_t *g_id2m_id, const int32_t *num_stages, const float *stage_latency,
+    const int32_t *batch_sizes, int64_t num_requests,
+    int32_t M, int32_t G, int32_t Smax, int32_t NB, double fixed_overhead,
+    int32_t *model_num_requests, int32_t *model_num_good_requests,
+    int32_t *group_num_requests, int32_t *group_num_good_requests);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MMSIM_H_ */

@@ -1,0 +1,58 @@
+"""Builds libmmsim.so (HIP, gfx950 only) into the package folder.
+
+    python -m mms_amd.csrc.build        # or: from mms_amd.csrc.build import build; build()
+
+Every translation unit is compiled by hipcc for gfx950 with fp contraction
+off, then linked into one shared library next to the Python package, where
+``mms_amd._lib`` looks for it.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.dirname(HERE)
+OUT = os.path.join(PKG, "libmmsim.so")
+OBJ_DIR = os.path.join(HERE, "build")
+
+SOURCES = ["mmsim_api.hip", "sim_mixed.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    "-ffp-contract=off", "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+]
+
+
+def _compile(src, extra):
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(HERE, src), "-o", obj]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{proc.stdout}\n{proc.stderr}")
+    noise = "packed-fp32-ops' is not a recognized feature"
+    warn = [l for l in proc.stderr.splitlines() if l.strip() and noise not in l]
+    return obj, "\n".join(warn)
+
+
+def build(verbose=False, extra_flags=()):
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+        results = list(pool.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
+    objs = [o for o, _ in results]
+    if verbose:
+        for _, w in results:
+            if w:
+                print(w, file=sys.stderr)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", OUT]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

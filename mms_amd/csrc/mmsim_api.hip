@@ -1,0 +1,637 @@
+// Host side of libmmsim: handles, validation, packing of placements into the
+// device layout the kernels read, launches, result unpacking.
+//
+// The packing restates the table build of approximate_one_case_one_placement
+// (alpa_serve/simulator/controller.py:412-476) in the factored form the
+// kernels use: instead of stage_latency[M][G][Smax] per placement, one latency
+// table per distinct parallel configuration plus, per (placement, model), the
+// ordered list of replica groups (m_id2g_id, :418-422).
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <new>
+
+#include "mmsim_internal.h"
+
+using namespace mmsim;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string &msg) {
+    g_last_error = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    return fail(e == hipErrorOutOfMemory ? MMSIM_E_NOMEM : MMSIM_E_HIP,
+                std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                      \
+    do {                                                   \
+        hipError_t e__ = (expr);                           \
+        if (e__ != hipSuccess) return hip_fail(e__, #expr); \
+    } while (0)
+
+template <typename T>
+struct DevBuf {
+    T *p = nullptr;
+    size_t n = 0;
+    DevBuf() = default;
+    DevBuf(const DevBuf &) = delete;
+    DevBuf &operator=(const DevBuf &) = delete;
+    ~DevBuf() { release(); }
+    void release() {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        n = 0;
+    }
+    hipError_t alloc(size_t count) {
+        release();
+        n = count;
+        return hipMalloc(reinterpret_cast<void **>(&p), std::max<size_t>(count, 1) * sizeof(T));
+    }
+    size_t bytes() const { return n * sizeof(T); }
+};
+
+}  // namespace
+
+struct mmsim_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t prop{};
+    int max_lds = 0;
+};
+
+struct mmsim_workload {
+    mmsim_ctx *ctx = nullptr;
+    int64_t R = 0;
+    int32_t M = 0;
+    DevBuf<Req> reqs;
+    std::vector<int32_t> model_num_requests;  // requests per model id (placement independent)
+};
+
+// Ordered replica lists per (placement, model): the rows of m_id2g_id.
+struct RepLists {
+    int32_t B = 0, M = 0, Gmax = 0;
+    std::vector<int32_t> num_groups;  // [B]
+    std::vector<int32_t> group_cfg;   // [B][Gmax]
+    std::vector<int64_t> off;         // [B*M+1]
+    std::vector<int32_t> grp;         // group index per replica
+};
+
+struct mmsim_batch {
+    mmsim_ctx *ctx = nullptr;
+    uint32_t flags = 0;
+    int32_t n_seeds = 0, B = 0, M = 0, Gmax = 0, tiles = 0, waves = 0;
+    int32_t smax_bucket = 0, rmax_bucket = 0, nslots = 0;
+    size_t lds_bytes = 0;
+    int64_t Rmax = 0, Rtotal = 0;
+    std::vector<const mmsim_workload *> wl;
+
+    DevBuf<Req> streams;
+    DevBuf<int64_t> stream_off;
+    DevBuf<uint32_t> rep;
+    DevBuf<int32_t> rmax;
+    DevBuf<float> lat;
+    DevBuf<int32_t> n_good;
+    DevBuf<double> lat_sum;
+    DevBuf<int32_t> model_good, group_req, group_good;
+    DevBuf<double> finish;
+    DevBuf<uint8_t> good;
+    DevBuf<int64_t> fp_ops;
+
+    MixedArgs args{};
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    bool ran = false;
+
+    ~mmsim_batch() {
+        if (ev_start) (void)hipEventDestroy(ev_start);
+        if (ev_stop) (void)hipEventDestroy(ev_stop);
+    }
+};
+
+namespace {
+
+int check_tables(const mmsim_tables *t) {
+    if (!t || !t->cfg_lat || !t->cfg_pp) return fail(MMSIM_E_INVALID, "tables: null pointer");
+    if (t->M < 1 || t->C < 1 || t->Smax < 1 || t->NB < 1) return fail(MMSIM_E_INVALID, "tables: M, C, Smax, NB must be >= 1");
+    if (t->C > 255) return fail(MMSIM_E_UNSUPPORTED, "tables: more than 255 parallel configurations");
+    if (t->Smax > MMSIM_MAX_STAGES) return fail(MMSIM_E_UNSUPPORTED, "tables: more than 32 pipeline stages");
+    for (int c = 0; c < t->C; ++c)
+        if (t->cfg_pp[c] < 1 || t->cfg_pp[c] > t->Smax)
+            return fail(MMSIM_E_INVALID, "tables: cfg_pp[c] outside 1..Smax");
+    if (t->NB > 1 && (!t->batch_sizes || t->batch_sizes[0] != 1))
+        return fail(MMSIM_E_INVALID, "tables: batch_sizes[0] must be 1");
+    if (!(t->fixed_overhead == t->fixed_overhead)) return fail(MMSIM_E_INVALID, "tables: fixed_overhead is NaN");
+    return MMSIM_OK;
+}
+
+// group -> models CSR of the C ABI into ordered per-(placement, model) replica lists
+int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLists *out) {
+    if (!p || !p->num_groups || !p->group_cfg || !p->gm_off) return fail(MMSIM_E_INVALID, "placements: null pointer");
+    if (p->B < 1 || p->Gmax < 1) return fail(MMSIM_E_INVALID, "placements: B and Gmax must be >= 1");
+    if (p->Gmax > MMSIM_MAX_GROUPS) return fail(MMSIM_E_UNSUPPORTED, "placements: more than 255 groups");
+    out->B = p->B;
+    out->M = M;
+    out->Gmax = p->Gmax;
+    out->num_groups.assign(p->num_groups, p->num_groups + p->B);
+    out->group_cfg.assign(p->group_cfg, p->group_cfg + (size_t)p->B * p->Gmax);
+    out->off.assign((size_t)p->B * M + 1, 0);
+    for (int32_t b = 0; b < p->B; ++b) {
+        const int32_t G = p->num_groups[b];
+        if (G < 0 || G > p->Gmax) return fail(MMSIM_E_INVALID, "placements: num_groups[b] outside 0..Gmax");
+        const int64_t *off = p->gm_off + (size_t)b * (p->Gmax + 1);
+        for (int32_t g = 0; g < G; ++g) {
+            const int32_t c = p->group_cfg[(size_t)b * p->Gmax + g];
+            if (c < 0 || c >= C) return fail(MMSIM_E_INVALID, "placements: group_cfg outside 0..C-1");
+            if (off[g + 1] < off[g]) return fail(MMSIM_E_INVALID, "placements: gm_off not monotone");
+            if (off[g + 1] > off[g] && !p->gm_idx) return fail(MMSIM_E_INVALID, "placements: gm_idx is null");
+            for (int64_t x = off[g]; x < off[g + 1]; ++x) {
+                const int32_t m = p->gm_idx[x];
+                if (m < 0 || m >= M) return fail(MMSIM_E_INVALID, "placements: model index outside 0..M-1");
+                out->off[(size_t)b * M + m + 1] += 1;
+            }
+        }
+    }
+    for (size_t i = 1; i < out->off.size(); ++i) out->off[i] += out->off[i - 1];
+    out->grp.assign((size_t)out->off.back(), 0);
+    std::vector<int64_t> fill(out->off.begin(), out->off.end() - 1);
+    for (int32_t b = 0; b < p->B; ++b) {
+        const int64_t *off = p->gm_off + (size_t)b * (p->Gmax + 1);
+        for (int32_t g = 0; g < p->num_groups[b]; ++g)  // ascending group index = reference order (:419-422)
+            for (int64_t x = off[g]; x < off[g + 1]; ++x) out->grp[(size_t)fill[(size_t)b * M + p->gm_idx[x]]++] = g;
+    }
+    return MMSIM_OK;
+}
+
+// Builds every device table of a batch from replica lists and launches nothing.
+int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seeds, const mmsim_tables *t,
+                const RepLists &rl, uint32_t flags, mmsim_batch **out) {
+    if (flags & MMSIM_BATCHING) return fail(MMSIM_E_UNSUPPORTED, "batching simulator is not available in this build");
+    const int32_t M = t->M, C = t->C, B = rl.B, Gmax = rl.Gmax;
+    if (n_seeds < 1 || !wls) return fail(MMSIM_E_INVALID, "need at least one workload");
+    for (int s = 0; s < n_seeds; ++s) {
+        if (!wls[s]) return fail(MMSIM_E_INVALID, "null workload");
+        if (wls[s]->ctx != ctx) return fail(MMSIM_E_INVALID, "workload belongs to another context");
+        if (wls[s]->M != M) return fail(MMSIM_E_INVALID, "workload and tables disagree on the number of models");
+    }
+    std::unique_ptr<mmsim_batch> b(new (std::nothrow) mmsim_batch);
+    if (!b) return fail(MMSIM_E_NOMEM, "host allocation failed");
+    b->ctx = ctx;
+    b->flags = flags;
+    b->n_seeds = n_seeds;
+    b->B = B;
+    b->M = M;
+    b->Gmax = Gmax;
+    b->tiles = (B + kWave - 1) / kWave;
+    b->waves = b->tiles * n_seeds;
+    b->wl.assign(wls, wls + n_seeds);
+
+    // ---- per placement: slot layout; per (placement, model): replica count
+    int smax = 1, rmax_all = 1, nslots = 1;
+    std::vector<uint8_t> slot0((size_t)B * Gmax, 0);
+    for (int32_t p = 0; p < B; ++p) {
+        int s = 0;
+        for (int32_t g = 0; g < rl.num_groups[p]; ++g) {
+            const int pp = t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]];
+            if (s + pp > MMSIM_MAX_SLOTS)
+                return fail(MMSIM_E_UNSUPPORTED, "placement has more than 255 pipeline stages in total");
+            slot0[(size_t)p * Gmax + g] = (uint8_t)s;
+            s += pp;
+            smax = std::max(smax, pp);
+        }
+        nslots = std::max(nslots, s);
+        for (int32_t m = 0; m < M; ++m)
+            rmax_all = std::max<int64_t>(rmax_all, rl.off[(size_t)p * M + m + 1] - rl.off[(size_t)p * M + m]);
+    }
+    if (rmax_all > MMSIM_MAX_REPLICAS) return fail(MMSIM_E_UNSUPPORTED, "a model has more than 64 replicas in one placement");
+    b->smax_bucket = smax_bucket_for(smax);
+    b->rmax_bucket = rmax_bucket_for(rmax_all);
+    if (b->smax_bucket < 0 || b->rmax_bucket < 0) return fail(MMSIM_E_UNSUPPORTED, "no kernel bucket for this shape");
+    b->nslots = nslots;
+    b->lds_bytes = (size_t)nslots * kWave * sizeof(double) +
+                   ((flags & MMSIM_WANT_GROUP_COUNTS) ? (size_t)2 * Gmax * kWave * sizeof(uint32_t) : 0);
+    if (b->lds_bytes > (size_t)ctx->max_lds)
+        return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups)");
+
+    // ---- replica descriptors [tiles][M][RB][64] and per-tile replica maxima
+    const int RB = b->rmax_bucket;
+    std::vector<uint32_t> rep((size_t)b->tiles * M * RB * kWave, kEmpty);
+    std::vector<int32_t> rmax((size_t)b->tiles * M, 0);
+    for (int32_t p = 0; p < B; ++p) {
+        const int tile = p / kWave, lane = p % kWave;
+        for (int32_t m = 0; m < M; ++m) {
+            const int64_t lo = rl.off[(size_t)p * M + m], hi = rl.off[(size_t)p * M + m + 1];
+            int32_t &rm = rmax[(size_t)tile * M + m];
+            rm = std::max<int32_t>(rm, (int32_t)(hi - lo));
+            for (int64_t x = lo; x < hi; ++x) {
+                const int32_t g = rl.grp[(size_t)x];
+                if (g < 0 || g >= rl.num_groups[p]) return fail(MMSIM_E_INVALID, "replica list names a group that does not exist");
+                const int32_t c = rl.group_cfg[(size_t)p * Gmax + g];
+                rep[(((size_t)tile * M + m) * RB + (size_t)(x - lo)) * kWave + lane] =
+                    pack_desc(slot0[(size_t)p * Gmax + g], (uint32_t)t->cfg_pp[c], (uint32_t)c, (uint32_t)g);
+            }
+        }
+    }
+    // ---- batch-size-1 latency table [M][C][Smax]
+    std::vector<float> lat((size_t)M * C * t->Smax);
+    for (size_t i = 0; i < lat.size(); ++i) lat[i] = t->cfg_lat[i * (size_t)t->NB];
+
+    // ---- request streams back to back
+    std::vector<int64_t> soff(n_seeds + 1, 0);
+    for (int s = 0; s < n_seeds; ++s) {
+        soff[s + 1] = soff[s] + wls[s]->R;
+        b->Rmax = std::max(b->Rmax, wls[s]->R);
+    }
+    b->Rtotal = soff[n_seeds];
+
+    hipStream_t st = ctx->stream;
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(b->streams.alloc((size_t)b->Rtotal));
+    for (int s = 0; s < n_seeds; ++s)
+        if (wls[s]->R > 0)
+            HIP_TRY(hipMemcpyAsync(b->streams.p + soff[s], wls[s]->reqs.p, sizeof(Req) * (size_t)wls[s]->R,
+                                   hipMemcpyDeviceToDevice, st));
+    HIP_TRY(b->stream_off.alloc(soff.size()));
+    HIP_TRY(hipMemcpyAsync(b->stream_off.p, soff.data(), sizeof(int64_t) * soff.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(b->rep.alloc(rep.size()));
+    HIP_TRY(hipMemcpyAsync(b->rep.p, rep.data(), sizeof(uint32_t) * rep.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(b->rmax.alloc(rmax.size()));
+    HIP_TRY(hipMemcpyAsync(b->rmax.p, rmax.data(), sizeof(int32_t) * rmax.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(b->lat.alloc(lat.size()));
+    HIP_TRY(hipMemcpyAsync(b->lat.p, lat.data(), sizeof(float) * lat.size(), hipMemcpyHostToDevice, st));
+
+    const size_t lanes_padded = (size_t)b->waves * kWave;
+    HIP_TRY(b->n_good.alloc(lanes_padded));
+    HIP_TRY(b->lat_sum.alloc(lanes_padded));
+    if (flags & MMSIM_WANT_MODEL_COUNTS) HIP_TRY(b->model_good.alloc(lanes_padded * M));
+    if (flags & MMSIM_WANT_GROUP_COUNTS) {
+        HIP_TRY(b->group_req.alloc(lanes_padded * Gmax));
+        HIP_TRY(b->group_good.alloc(lanes_padded * Gmax));
+    }
+    if (flags & MMSIM_WANT_PER_REQUEST) {
+        HIP_TRY(b->finish.alloc(lanes_padded * (size_t)b->Rmax));
+        HIP_TRY(b->good.alloc(lanes_padded * (size_t)b->Rmax));
+    }
+    if (flags & MMSIM_WANT_OP_COUNT) HIP_TRY(b->fp_ops.alloc(lanes_padded));
+    HIP_TRY(hipEventCreate(&b->ev_start));
+    HIP_TRY(hipEventCreate(&b->ev_stop));
+    HIP_TRY(hipStreamSynchronize(st));  // host staging vectors go out of scope below
+
+    MixedArgs &a = b->args;
+    a.streams = b->streams.p;
+    a.stream_off = b->stream_off.p;
+    a.rep = b->rep.p;
+    a.rmax = b->rmax.p;
+    a.lat = b->lat.p;
+    a.M = M;
+    a.C = C;
+    a.lat_stride = t->Smax;
+    a.n_seeds = n_seeds;
+    a.B = B;
+    a.tiles = b->tiles;
+    a.nslots = nslots;
+    a.Gmax = Gmax;
+    a.Rmax = b->Rmax;
+    a.fixed_overhead = t->fixed_overhead;
+    a.flags = flags;
+    a.n_good = b->n_good.p;
+    a.lat_sum = b->lat_sum.p;
+    a.model_good = b->model_good.p;
+    a.group_req = b->group_req.p;
+    a.group_good = b->group_good.p;
+    a.finish = b->finish.p;
+    a.good = b->good.p;
+    a.fp_ops = b->fp_ops.p;
+    *out = b.release();
+    return MMSIM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mmsim_abi_version(void) { return MMSIM_ABI_VERSION; }
+
+const char *mmsim_last_error(void) { return g_last_error.c_str(); }
+
+int mmsim_ctx_create(int device, mmsim_ctx **out) {
+    if (!out) return fail(MMSIM_E_INVALID, "ctx_create: out is null");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count < 1)
+        return fail(MMSIM_E_HIP, std::string("no usable HIP device: ") + (e != hipSuccess ? hipGetErrorString(e) : "device count is 0"));
+    if (device < 0 || device >= count) return fail(MMSIM_E_INVALID, "ctx_create: device ordinal out of range");
+    std::unique_ptr<mmsim_ctx> c(new (std::nothrow) mmsim_ctx);
+    if (!c) return fail(MMSIM_E_NOMEM, "host allocation failed");
+    c->device = device;
+    HIP_TRY(hipSetDevice(device));
+    HIP_TRY(hipGetDeviceProperties(&c->prop, device));
+    if (std::strncmp(c->prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(MMSIM_E_UNSUPPORTED, std::string("libmmsim is built for gfx950 only, device is ") + c->prop.gcnArchName);
+    int lds = 0;
+    if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess || lds <= 0)
+        lds = (int)c->prop.sharedMemPerBlock;
+    c->max_lds = lds;
+    HIP_TRY(hipStreamCreate(&c->stream));  // default priority
+    *out = c.release();
+    return MMSIM_OK;
+}
+
+void mmsim_ctx_destroy(mmsim_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipStreamDestroy(ctx->stream);
+    }
+    delete ctx;
+}
+
+int mmsim_ctx_device_info(mmsim_ctx *ctx, mmsim_device_info *out) {
+    if (!ctx || !out) return fail(MMSIM_E_INVALID, "device_info: null pointer");
+    std::memset(out, 0, sizeof(*out));
+    std::snprintf(out->name, sizeof(out->name), "%s", ctx->prop.name);
+    std::snprintf(out->arch, sizeof(out->arch), "%s", ctx->prop.gcnArchName);
+    out->compute_units = ctx->prop.multiProcessorCount;
+    out->clock_khz = ctx->prop.clockRate;
+    out->lds_bytes_per_block = ctx->max_lds;
+    out->hbm_bytes = (int64_t)ctx->prop.totalGlobalMem;
+    return MMSIM_OK;
+}
+
+int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *tstamps, const int32_t *model_ids,
+                          const float *slos, mmsim_workload **out) {
+    if (!ctx || !out) return fail(MMSIM_E_INVALID, "workload_create: null pointer");
+    *out = nullptr;
+    if (R < 0 || M < 1) return fail(MMSIM_E_INVALID, "workload_create: R must be >= 0 and M >= 1");
+    if (R > 0 && (!tstamps || !model_ids || !slos)) return fail(MMSIM_E_INVALID, "workload_create: null array");
+    std::unique_ptr<mmsim_workload> w(new (std::nothrow) mmsim_workload);
+    if (!w) return fail(MMSIM_E_NOMEM, "host allocation failed");
+    w->ctx = ctx;
+    w->R = R;
+    w->M = M;
+    w->model_num_requests.assign(M, 0);
+    std::vector<Req> host((size_t)R);
+    for (int64_t i = 0; i < R; ++i) {
+        if (model_ids[i] >= M) return fail(MMSIM_E_INVALID, "workload_create: model id >= M");
+        host[i].t = tstamps[i];
+        host[i].m = model_ids[i] < 0 ? -1 : model_ids[i];
+        host[i].slo = slos[i];
+        if (model_ids[i] >= 0) w->model_num_requests[model_ids[i]] += 1;
+    }
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(w->reqs.alloc((size_t)R));
+    if (R > 0) {
+        HIP_TRY(hipMemcpyAsync(w->reqs.p, host.data(), sizeof(Req) * (size_t)R, hipMemcpyHostToDevice, ctx->stream));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+    }
+    *out = w.release();
+    return MMSIM_OK;
+}
+
+void mmsim_workload_destroy(mmsim_workload *wl) {
+    if (!wl) return;
+    if (wl->ctx) (void)hipSetDevice(wl->ctx->device);
+    delete wl;
+}
+
+int mmsim_batch_create(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                       const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
+                       mmsim_batch **out) {
+    if (!ctx || !out) return fail(MMSIM_E_INVALID, "batch_create: null pointer");
+    *out = nullptr;
+    int rc = check_tables(tables);
+    if (rc) return rc;
+    RepLists rl;
+    rc = lists_from_placements(placements, tables->M, tables->C, &rl);
+    if (rc) return rc;
+    return build_batch(ctx, workloads, n_seeds, tables, rl, flags, out);
+}
+
+int mmsim_batch_run(mmsim_batch *b) {
+    if (!b) return fail(MMSIM_E_INVALID, "batch_run: null batch");
+    mmsim_ctx *ctx = b->ctx;
+    HIP_TRY(hipSetDevice(ctx->device));
+    if (b->flags & MMSIM_WANT_MODEL_COUNTS)
+        HIP_TRY(hipMemsetAsync(b->model_good.p, 0, b->model_good.bytes(), ctx->stream));
+    HIP_TRY(hipEventRecord(b->ev_start, ctx->stream));
+    std::string err;
+    hipError_t e = launch_sim_mixed(b->args, b->smax_bucket, b->rmax_bucket, b->lds_bytes, ctx->stream, &err);
+    if (e != hipSuccess) return fail(MMSIM_E_HIP, err);
+    HIP_TRY(hipEventRecord(b->ev_stop, ctx->stream));
+    b->ran = true;
+    return MMSIM_OK;
+}
+
+int mmsim_batch_sync(mmsim_batch *b, float *kernel_ms) {
+    if (!b) return fail(MMSIM_E_INVALID, "batch_sync: null batch");
+    if (!b->ran) return fail(MMSIM_E_INVALID, "batch_sync: batch was never run");
+    HIP_TRY(hipSetDevice(b->ctx->device));
+    HIP_TRY(hipEventSynchronize(b->ev_stop));
+    if (kernel_ms) HIP_TRY(hipEventElapsedTime(kernel_ms, b->ev_start, b->ev_stop));
+    return MMSIM_OK;
+}
+
+int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
+    if (!b || !out) return fail(MMSIM_E_INVALID, "batch_fetch: null pointer");
+    if (!b->ran) return fail(MMSIM_E_INVALID, "batch_fetch: batch was never run");
+    if (!out->n_good || !out->latency_sum) return fail(MMSIM_E_INVALID, "batch_fetch: n_good and latency_sum are required");
+    const bool wm = b->flags & MMSIM_WANT_MODEL_COUNTS, wg = b->flags & MMSIM_WANT_GROUP_COUNTS,
+               wr = b->flags & MMSIM_WANT_PER_REQUEST;
+    if (wm && (!out->model_num_requests || !out->model_num_good)) return fail(MMSIM_E_INVALID, "batch_fetch: model count arrays missing");
+    if (wg && (!out->group_num_requests || !out->group_num_good)) return fail(MMSIM_E_INVALID, "batch_fetch: group count arrays missing");
+    if (wr && (!out->finish || !out->good)) return fail(MMSIM_E_INVALID, "batch_fetch: per-request arrays missing");
+    HIP_TRY(hipSetDevice(b->ctx->device));
+    HIP_TRY(hipStreamSynchronize(b->ctx->stream));
+
+    const int32_t B = b->B, M = b->M, Gmax = b->Gmax, tiles = b->tiles;
+    const size_t lanes_padded = (size_t)b->waves * kWave;
+    std::vector<int32_t> ng(lanes_padded);
+    std::vector<double> ls(lanes_padded);
+    HIP_TRY(hipMemcpy(ng.data(), b->n_good.p, sizeof(int32_t) * lanes_padded, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(ls.data(), b->lat_sum.p, sizeof(double) * lanes_padded, hipMemcpyDeviceToHost));
+    std::vector<int64_t> ops;
+    if (b->flags & MMSIM_WANT_OP_COUNT) {
+        if (!out->fp_ops) return fail(MMSIM_E_INVALID, "batch_fetch: fp_ops array missing");
+        ops.resize(lanes_padded);
+        HIP_TRY(hipMemcpy(ops.data(), b->fp_ops.p, sizeof(int64_t) * lanes_padded, hipMemcpyDeviceToHost));
+    }
+    for (int s = 0; s < b->n_seeds; ++s)
+        for (int32_t p = 0; p < B; ++p) {
+            const size_t src = (size_t)s * tiles * kWave + p;
+            out->n_good[(size_t)s * B + p] = ng[src];
+            out->latency_sum[(size_t)s * B + p] = ls[src];
+            if (out->status) out->status[(size_t)s * B + p] = 0;
+            if (!ops.empty()) out->fp_ops[(size_t)s * B + p] = ops[src];
+        }
+    // device rows are [wave][x][64] with wave = seed*tiles + tile; lane l of a seed is placement l
+    auto unpack_i32 = [&](const DevBuf<int32_t> &dev, int32_t width, int32_t *dst) -> int {
+        std::vector<int32_t> h(dev.n);
+        HIP_TRY(hipMemcpy(h.data(), dev.p, dev.bytes(), hipMemcpyDeviceToHost));
+        for (int s = 0; s < b->n_seeds; ++s)
+            for (int32_t p = 0; p < B; ++p) {
+                const size_t wave = (size_t)s * tiles + p / kWave;
+                for (int32_t x = 0; x < width; ++x)
+                    dst[((size_t)s * B + p) * width + x] = h[(wave * width + x) * kWave + p % kWave];
+            }
+        return MMSIM_OK;
+    };
+    if (wm) {
+        int rc = unpack_i32(b->model_good, M, out->model_num_good);
+        if (rc) return rc;
+        for (int s = 0; s < b->n_seeds; ++s)
+            for (int32_t p = 0; p < B; ++p)
+                std::memcpy(out->model_num_requests + ((size_t)s * B + p) * M, b->wl[s]->model_num_requests.data(),
+                            sizeof(int32_t) * (size_t)M);
+    }
+    if (wg) {
+        int rc = unpack_i32(b->group_req, Gmax, out->group_num_requests);
+        if (rc) return rc;
+        rc = unpack_i32(b->group_good, Gmax, out->group_num_good);
+        if (rc) return rc;
+    }
+    if (wr && b->Rmax > 0) {
+        const size_t Rm = (size_t)b->Rmax;
+        std::vector<double> hf(Rm * kWave);
+        std::vector<uint8_t> hg(Rm * kWave);
+        for (int s = 0; s < b->n_seeds; ++s)
+            for (int32_t tile = 0; tile < tiles; ++tile) {
+                const size_t wave = (size_t)s * tiles + tile;
+                HIP_TRY(hipMemcpy(hf.data(), b->finish.p + wave * Rm * kWave, sizeof(double) * Rm * kWave, hipMemcpyDeviceToHost));
+                HIP_TRY(hipMemcpy(hg.data(), b->good.p + wave * Rm * kWave, Rm * kWave, hipMemcpyDeviceToHost));
+                const size_t Rs = (size_t)b->wl[s]->R;
+                for (int l = 0; l < kWave && tile * kWave + l < B; ++l) {
+                    const size_t row = ((size_t)s * B + (size_t)tile * kWave + l) * Rm;
+                    for (size_t i = 0; i < Rs; ++i) {
+                        out->finish[row + i] = hf[i * kWave + l];
+                        out->good[row + i] = hg[i * kWave + l];
+                    }
+                }
+            }
+    }
+    return MMSIM_OK;
+}
+
+void mmsim_batch_destroy(mmsim_batch *b) {
+    if (!b) return;
+    if (b->ctx) {
+        (void)hipSetDevice(b->ctx->device);
+        (void)hipStreamSynchronize(b->ctx->stream);
+    }
+    delete b;
+}
+
+int mmsim_batch_get_info(const mmsim_batch *b, mmsim_batch_info *out) {
+    if (!b || !out) return fail(MMSIM_E_INVALID, "batch_get_info: null pointer");
+    out->lanes = b->B * b->n_seeds;
+    out->waves = b->waves;
+    out->n_seeds = b->n_seeds;
+    out->B = b->B;
+    out->smax_bucket = b->smax_bucket;
+    out->rmax_bucket = b->rmax_bucket;
+    out->slots = b->nslots;
+    out->lds_bytes = (int32_t)b->lds_bytes;
+    out->requests_total = b->Rtotal;
+    out->table_bytes = (int64_t)(b->rep.bytes() + b->rmax.bytes() + b->lat.bytes());
+    out->stream_bytes = (int64_t)b->streams.bytes();
+    return MMSIM_OK;
+}
+
+int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                     const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
+                     mmsim_result *out) {
+    if (!out) return fail(MMSIM_E_INVALID, "eval_batch: out is null");
+    mmsim_batch *b = nullptr;
+    int rc = mmsim_batch_create(ctx, workloads, n_seeds, tables, placements, flags, &b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
+    if (rc == MMSIM_OK) rc = mmsim_batch_fetch(b, out);
+    mmsim_batch_destroy(b);
+    return rc;
+}
+
+int mmsim_simulate_requests_mixed(mmsim_ctx *ctx, double *finish, uint8_t *good, const double *tstamps,
+                                  const int32_t *model_ids, const float *slos, const int32_t *m_id2g_id,
+                                  const int32_t *num_stages, const float *stage_latency, int64_t num_requests,
+                                  int32_t M, int32_t G, int32_t Smax, double fixed_overhead,
+                                  int32_t *model_num_requests, int32_t *model_num_good_requests,
+                                  int32_t *group_num_requests, int32_t *group_num_good_requests) {
+    if (!ctx) return fail(MMSIM_E_INVALID, "simulate_requests_mixed: null context");
+    if (M < 1 || G < 1 || Smax < 1 || num_requests < 0) return fail(MMSIM_E_INVALID, "simulate_requests_mixed: bad size");
+    if (!m_id2g_id || !num_stages || !stage_latency || !model_num_requests || !model_num_good_requests ||
+        !group_num_requests || !group_num_good_requests || (num_requests > 0 && (!finish || !good)))
+        return fail(MMSIM_E_INVALID, "simulate_requests_mixed: null pointer");
+    if (G > MMSIM_MAX_GROUPS) return fail(MMSIM_E_UNSUPPORTED, "simulate_requests_mixed: more than 255 groups");
+    // every group is its own latency-table column
+    mmsim_tables t{};
+    t.M = M;
+    t.C = G;
+    t.Smax = Smax;
+    t.NB = 1;
+    t.cfg_lat = stage_latency;
+    t.cfg_pp = num_stages;
+    t.batch_sizes = nullptr;
+    t.fixed_overhead = fixed_overhead;
+    int rc = check_tables(&t);
+    if (rc) return rc;
+    RepLists rl;
+    rl.B = 1;
+    rl.M = M;
+    rl.Gmax = G;
+    rl.num_groups.assign(1, G);
+    rl.group_cfg.resize(G);
+    for (int g = 0; g < G; ++g) rl.group_cfg[g] = g;
+    rl.off.assign((size_t)M + 1, 0);
+    for (int32_t m = 0; m < M; ++m)
+        for (int32_t j = 0; j < G; ++j) {
+            const int32_t g = m_id2g_id[(size_t)m * G + j];
+            if (g < 0) break;
+            if (g >= G) return fail(MMSIM_E_INVALID, "simulate_requests_mixed: m_id2g_id names a group >= G");
+            rl.grp.push_back(g);
+            rl.off[m + 1] += 1;
+        }
+    for (int32_t m = 0; m < M; ++m) rl.off[m + 1] += rl.off[m];
+
+    mmsim_workload *wl = nullptr;
+    rc = mmsim_workload_create(ctx, num_requests, M, tstamps, model_ids, slos, &wl);
+    if (rc) return rc;
+    mmsim_batch *b = nullptr;
+    const mmsim_workload *wls[1] = {wl};
+    const uint32_t flags = MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS | MMSIM_WANT_PER_REQUEST;
+    rc = build_batch(ctx, wls, 1, &t, rl, flags, &b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
+    if (rc == MMSIM_OK) {
+        int64_t ng = 0;
+        double ls = 0.0;
+        mmsim_result r{};
+        r.n_good = &ng;
+        r.latency_sum = &ls;
+        r.model_num_requests = model_num_requests;
+        r.model_num_good = model_num_good_requests;
+        r.group_num_requests = group_num_requests;
+        r.group_num_good = group_num_good_requests;
+        r.finish = finish;
+        r.good = good;
+        rc = mmsim_batch_fetch(b, &r);
+    }
+    mmsim_batch_destroy(b);
+    mmsim_workload_destroy(wl);
+    return rc;
+}
+
+int mmsim_simulate_requests_mixed_batching(mmsim_ctx *, double *, uint8_t *, const double *, const int32_t *,
+                                           const float *, const int32_t *, const int32_t *, const int32_t *,
+                                           const float *, const int32_t *, int64_t, int32_t, int32_t, int32_t, int32_t,
+                                           double, int32_t *, int32_t *, int32_t *, int32_t *) {
+    return fail(MMSIM_E_UNSUPPORTED, "batching simulator is not available in this build");
+}
+
+}  // extern "C"

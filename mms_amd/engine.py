@@ -1,0 +1,320 @@
+"""Python side of the C ABI: packs placements and profiles into the flat
+arrays ``libmmsim`` takes and turns its results back into numpy arrays.
+
+The packing is the batched form of the reference's per-placement table build
+(``approximate_one_case_one_placement``, alpa_serve/simulator/controller.py:
+412-476).  That code fills ``stage_latency[model][group][stage]`` for every
+placement; the value depends only on the group's ParallelConfig, so here a
+latency table is built once per distinct ParallelConfig (``LatencyTable``) and a
+placement is reduced to "which config does each group use, which models does
+it host".
+"""
+import ctypes as C
+from itertools import chain
+from typing import List, Sequence
+
+import numpy as np
+
+from mms_amd import _lib
+from mms_amd.util import FIXED_OVERHEAD, STAGE_PENALTY
+
+
+class Engine:
+    """One libmmsim context (one GPU, one stream)."""
+
+    _default = None
+
+    def __init__(self, device: int = 0):
+        self.lib = _lib.load()
+        self._h = C.c_void_p()
+        _lib.check(self.lib.mmsim_ctx_create(device, C.byref(self._h)))
+        self.device = device
+
+    @classmethod
+    def default(cls):
+        if cls._default is None:
+            cls._default = cls(0)
+        return cls._default
+
+    def device_info(self):
+        info = _lib.DeviceInfo()
+        _lib.check(self.lib.mmsim_ctx_device_info(self._h, C.byref(info)))
+        return {"name": info.name.decode(), "arch": info.arch.decode(),
+                "compute_units": info.compute_units, "clock_khz": info.clock_khz,
+                "lds_bytes_per_block": info.lds_bytes_per_block, "hbm_bytes": info.hbm_bytes}
+
+    def close(self):
+        if self._h:
+            self.lib.mmsim_ctx_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class DeviceWorkload:
+    """A request stream resident in HBM (arrivals f64, model ids i32, SLOs f32)."""
+
+    def __init__(self, engine: Engine, tstamps, model_ids, slos, num_models: int):
+        self.engine = engine
+        ts = _lib.carray(tstamps, np.float64)
+        mid = _lib.carray(model_ids, np.int32)
+        sl = _lib.carray(slos, np.float32)
+        assert len(ts) == len(mid) == len(sl)
+        self.R = len(ts)
+        self.M = int(num_models)
+        self._h = C.c_void_p()
+        _lib.check(engine.lib.mmsim_workload_create(
+            engine._h, self.R, self.M, _lib.ptr(ts, C.c_double), _lib.ptr(mid, C.c_int32),
+            _lib.ptr(sl, C.c_float), C.byref(self._h)))
+
+    def close(self):
+        if self._h:
+            self.engine.lib.mmsim_workload_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class LatencyTable:
+    """cfg_lat[M][C][Smax][NB] float32 for a growing set of ParallelConfigs.
+
+    Entry values follow controller.py:456-459 / :472-474 exactly: the Python
+    float product ``latency[bs][k] * (1 + 0.009 * len(latency[1]))`` rounded to
+    float32 on store; a config a model has no profile for gives +inf
+    (:461, :476).
+    """
+
+    def __init__(self, prof_ress: Sequence, batch_sizes: Sequence[int] = (1,)):
+        self.prof_ress = list(prof_ress)
+        self.batch_sizes = [int(b) for b in batch_sizes]
+        assert self.batch_sizes[0] == 1
+        self.configs = []
+        self.index = {}
+        self._arrays = None
+
+    def config_id(self, cfg) -> int:
+        i = self.index.get(cfg)
+        if i is None:
+            i = self.index[cfg] = len(self.configs)
+            self.configs.append(cfg)
+            self._arrays = None
+        return i
+
+    def arrays(self):
+        if self._arrays is None:
+            M, Cn, NB = len(self.prof_ress), max(len(self.configs), 1), len(self.batch_sizes)
+            smax = max([int(c.pp) for c in self.configs] or [1])
+            lat = np.zeros((M, Cn, smax, NB), np.float32)
+            pp = np.ones(Cn, np.int32)
+            with np.errstate(over="ignore"):
+                for c, cfg in enumerate(self.configs):
+                    pp[c] = cfg.pp
+                    for m, prof in enumerate(self.prof_ress):
+                        entry = prof.para_dict.get(cfg, None)
+                        if not entry:
+                            lat[m, c] = np.inf
+                            continue
+                        scale = 1 + STAGE_PENALTY * len(entry.latency[1])
+                        for k in range(cfg.pp):
+                            for b, bs in enumerate(self.batch_sizes):
+                                lat[m, c, k, b] = entry.latency[bs][k] * scale
+            self._arrays = (lat, pp)
+        return self._arrays
+
+
+def pack_placements(sols: Sequence, table: LatencyTable):
+    """ModelPlacement list -> (num_groups[B], group_cfg[B][Gmax], gm_off[B][Gmax+1], gm_idx)."""
+    B = len(sols)
+    num_groups = np.fromiter((len(s.group_configs) for s in sols), np.int32, B)
+    Gmax = max(int(num_groups.max()) if B else 1, 1)
+    group_cfg = np.zeros((B, Gmax), np.int32)
+    sizes = np.zeros((B, Gmax), np.int64)
+    cid = table.config_id
+    for b, s in enumerate(sols):
+        g = num_groups[b]
+        if g:
+            group_cfg[b, :g] = [cid(c) for c in s.group_configs]
+            sizes[b, :g] = [len(ms) for ms in s.group_models]
+    gm_off = np.zeros((B, Gmax + 1), np.int64)
+    np.cumsum(sizes, axis=1, out=gm_off[:, 1:])
+    per_sol = gm_off[:, -1].copy()
+    base = np.zeros(B, np.int64)
+    np.cumsum(per_sol[:-1], out=base[1:])
+    gm_off += base[:, None]
+    total = int(per_sol.sum())
+    gm_idx = np.fromiter(chain.from_iterable(chain.from_iterable(s.group_models) for s in sols),
+                         np.int32, total)
+    return num_groups, group_cfg, gm_off, gm_idx
+
+
+class Batch:
+    """Device-resident batch of placements x seeds; run() may be repeated."""
+
+    def __init__(self, engine: Engine, workloads: Sequence[DeviceWorkload], table: LatencyTable,
+                 packed, flags: int, fixed_overhead: float = FIXED_OVERHEAD):
+        self.engine = engine
+        self.workloads = list(workloads)
+        self.flags = int(flags)
+        num_groups, group_cfg, gm_off, gm_idx = packed
+        lat, pp = table.arrays()
+        bss = _lib.carray(table.batch_sizes, np.int32)
+        self.B, self.Gmax = group_cfg.shape
+        self.M = lat.shape[0]
+        self.n_seeds = len(self.workloads)
+        self.Rmax = max(w.R for w in self.workloads)
+        t = _lib.Tables(lat.shape[0], lat.shape[1], lat.shape[2], lat.shape[3],
+                        _lib.ptr(lat, C.c_float), _lib.ptr(pp, C.c_int32), _lib.ptr(bss, C.c_int32),
+                        float(fixed_overhead))
+        num_groups = _lib.carray(num_groups, np.int32)
+        group_cfg = _lib.carray(group_cfg, np.int32)
+        gm_off = _lib.carray(gm_off, np.int64)
+        gm_idx = _lib.carray(gm_idx, np.int32)
+        p = _lib.Placements(self.B, self.Gmax, _lib.ptr(num_groups, C.c_int32),
+                            _lib.ptr(group_cfg, C.c_int32), _lib.ptr(gm_off, C.c_int64),
+                            _lib.ptr(gm_idx, C.c_int32))
+        wl = (C.c_void_p * self.n_seeds)(*[w._h for w in self.workloads])
+        self._h = C.c_void_p()
+        _lib.check(engine.lib.mmsim_batch_create(engine._h, wl, self.n_seeds, C.byref(t), C.byref(p),
+                                                 self.flags, C.byref(self._h)))
+
+    def run(self):
+        _lib.check(self.engine.lib.mmsim_batch_run(self._h))
+
+    def sync(self) -> float:
+        """Waits for the run; returns the simulation kernel's time in ms (HIP events)."""
+        ms = C.c_float(0)
+        _lib.check(self.engine.lib.mmsim_batch_sync(self._h, C.byref(ms)))
+        return ms.value
+
+    def info(self):
+        bi = _lib.BatchInfo()
+        _lib.check(self.engine.lib.mmsim_batch_get_info(self._h, C.byref(bi)))
+        return {f[0]: getattr(bi, f[0]) for f in bi._fields_}
+
+    def fetch(self):
+        L = self.B * self.n_seeds
+        out = {"n_good": np.zeros(L, np.int64), "latency_sum": np.zeros(L, np.float64),
+               "status": np.zeros(L, np.int32)}
+        r = _lib.Result()
+        r.n_good = _lib.ptr(out["n_good"], C.c_int64)
+        r.latency_sum = _lib.ptr(out["latency_sum"], C.c_double)
+        r.status = _lib.ptr(out["status"], C.c_int32)
+        if self.flags & _lib.WANT_MODEL_COUNTS:
+            out["model_num_requests"] = np.zeros((L, self.M), np.int32)
+            out["model_num_good"] = np.zeros((L, self.M), np.int32)
+            r.model_num_requests = _lib.ptr(out["model_num_requests"], C.c_int32)
+            r.model_num_good = _lib.ptr(out["model_num_good"], C.c_int32)
+        if self.flags & _lib.WANT_GROUP_COUNTS:
+            out["group_num_requests"] = np.zeros((L, self.Gmax), np.int32)
+            out["group_num_good"] = np.zeros((L, self.Gmax), np.int32)
+            r.group_num_requests = _lib.ptr(out["group_num_requests"], C.c_int32)
+            r.group_num_good = _lib.ptr(out["group_num_good"], C.c_int32)
+        if self.flags & _lib.WANT_PER_REQUEST:
+            out["finish"] = np.zeros((L, self.Rmax), np.float64)
+            out["good"] = np.zeros((L, self.Rmax), np.uint8)
+            r.finish = _lib.ptr(out["finish"], C.c_double)
+            r.good = _lib.ptr(out["good"], C.c_uint8)
+        if self.flags & _lib.WANT_OP_COUNT:
+            out["fp_ops"] = np.zeros(L, np.int64)
+            r.fp_ops = _lib.ptr(out["fp_ops"], C.c_int64)
+        _lib.check(self.engine.lib.mmsim_batch_fetch(self._h, C.byref(r)))
+        if "good" in out:
+            out["good"] = out["good"].astype(bool)
+        for k in list(out):
+            if out[k].ndim >= 1 and out[k].shape[0] == L:
+                out[k] = out[k].reshape((self.n_seeds, self.B) + out[k].shape[1:])
+        return out
+
+    def close(self):
+        if self._h:
+            self.engine.lib.mmsim_batch_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def evaluate(engine: Engine, workloads: Sequence[DeviceWorkload], table: LatencyTable, sols: Sequence,
+             flags: int = 0, fixed_overhead: float = FIXED_OVERHEAD):
+    """One-shot: pack, upload, simulate, fetch.  Result arrays are [n_seeds][B][...]."""
+    packed = pack_placements(sols, table)
+    batch = Batch(engine, workloads, table, packed, flags, fixed_overhead)
+    try:
+        batch.run()
+        ms = batch.sync()
+        out = batch.fetch()
+        out["kernel_ms"] = ms
+        out["info"] = batch.info()
+    finally:
+        batch.close()
+    return out
+
+
+def simulate_requests_mixed(engine: Engine, finish, good, tstamps, model_ids, slos, m_id2g_id,
+                            num_stages, stage_latency, num_requests=None,
+                            fixed_overhead: float = FIXED_OVERHEAD):
+    """Same call as the reference's numba kernel (controller.py:561-628):
+    fills ``finish``/``good`` in place and returns the four count arrays."""
+    ts = _lib.carray(tstamps, np.float64)
+    R = len(ts) if num_requests is None else int(num_requests)
+    mid = _lib.carray(model_ids, np.int32)
+    sl = _lib.carray(slos, np.float32)
+    m2g = _lib.carray(m_id2g_id, np.int32)
+    ns = _lib.carray(num_stages, np.int32)
+    lat = _lib.carray(stage_latency, np.float32)
+    M, G = m2g.shape
+    assert lat.shape[:2] == (M, G)
+    S = lat.shape[2]
+    fin = np.empty(R, np.float64)
+    gd = np.empty(R, np.uint8)
+    counts = [np.zeros(M, np.int32), np.zeros(M, np.int32), np.zeros(G, np.int32), np.zeros(G, np.int32)]
+    _lib.check(engine.lib.mmsim_simulate_requests_mixed(
+        engine._h, _lib.ptr(fin, C.c_double), _lib.ptr(gd, C.c_uint8), _lib.ptr(ts, C.c_double),
+        _lib.ptr(mid, C.c_int32), _lib.ptr(sl, C.c_float), _lib.ptr(m2g, C.c_int32),
+        _lib.ptr(ns, C.c_int32), _lib.ptr(lat, C.c_float), R, M, G, S, float(fixed_overhead),
+        *[_lib.ptr(c, C.c_int32) for c in counts]))
+    finish[:R] = fin
+    good[:R] = gd.astype(bool)
+    return tuple(counts)
+
+
+def simulate_requests_mixed_batching(engine: Engine, finish, good, tstamps, model_ids, slos, m_id2g_id,
+                                     g_id2m_id, num_stages, stage_latency, batch_sizes,
+                                     num_requests=None, fixed_overhead: float = FIXED_OVERHEAD):
+    """Same call as the reference's batching loop (controller.py:631-798);
+    ``stage_latency`` is [M][G][Smax][NB] with one column per batch size."""
+    ts = _lib.carray(tstamps, np.float64)
+    R = len(ts) if num_requests is None else int(num_requests)
+    mid = _lib.carray(model_ids, np.int32)
+    sl = _lib.carray(slos, np.float32)
+    m2g = _lib.carray(m_id2g_id, np.int32)
+    g2m = _lib.carray(g_id2m_id, np.int32)
+    ns = _lib.carray(num_stages, np.int32)
+    lat = _lib.carray(stage_latency, np.float32)
+    bss = _lib.carray(batch_sizes, np.int32)
+    M, G = m2g.shape
+    assert lat.shape[:2] == (M, G) and lat.shape[3] == len(bss)
+    S = lat.shape[2]
+    fin = np.empty(R, np.float64)
+    gd = np.empty(R, np.uint8)
+    counts = [np.zeros(M, np.int32), np.zeros(M, np.int32), np.zeros(G, np.int32), np.zeros(G, np.int32)]
+    _lib.check(engine.lib.mmsim_simulate_requests_mixed_batching(
+        engine._h, _lib.ptr(fin, C.c_double), _lib.ptr(gd, C.c_uint8), _lib.ptr(ts, C.c_double),
+        _lib.ptr(mid, C.c_int32), _lib.ptr(sl, C.c_float), _lib.ptr(m2g, C.c_int32),
+        _lib.ptr(g2m, C.c_int32), _lib.ptr(ns, C.c_int32), _lib.ptr(lat, C.c_float),
+        _lib.ptr(bss, C.c_int32), R, M, G, S, len(bss), float(fixed_overhead),
+        *[_lib.ptr(c, C.c_int32) for c in counts]))
+    finish[:R] = fin
+    good[:R] = gd.astype(bool)
+    return tuple(counts)

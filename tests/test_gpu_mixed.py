@@ -1,0 +1,204 @@
+"""GPU parity of the plain (non-batching) simulator against the CPU oracle.
+
+Everything goes through the C ABI of libmmsim (ctypes).  Bars: served/dropped
+flags, all counts and finish times bit-exact (the tolerance the task states
+for latencies is 1e-12 relative; the same fp64 operation sequence gives
+identical bits, so identical bits are asserted).
+"""
+import numpy as np
+import pytest
+
+from mms_amd import _lib, engine as E
+from mms_amd.synthetic import make_config
+from oracle import oracle_c
+from randcase import random_case
+from helpers import assert_batch_matches, oracle_batch
+
+pytestmark = pytest.mark.gpu
+
+ALL = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS | _lib.WANT_PER_REQUEST | _lib.WANT_OP_COUNT
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return E.Engine.default()
+
+
+def test_library_reports_the_device(eng):
+    info = eng.device_info()
+    print(info, flush=True)
+    assert info["arch"].startswith("gfx950")
+    assert info["compute_units"] >= 1
+
+
+def test_single_placement_call_matches_oracle_on_random_cases(eng):
+    for seed in range(300):
+        c = random_case(seed, max_m=5, max_g=4, max_s=4, max_r=120)
+        lat = c["lat"][..., 0]
+        fin, good, cnt, _ = oracle_c.simulate_requests_mixed(
+            c["tstamps"], c["model_ids"], c["slos"], c["m2g"], c["num_stages"], lat)
+        f2 = np.empty(c["R"])
+        g2 = np.empty(c["R"], bool)
+        cnt2 = E.simulate_requests_mixed(eng, f2, g2, c["tstamps"], c["model_ids"], c["slos"], c["m2g"],
+                                         c["num_stages"], lat)
+        assert np.array_equal(g2, good), seed
+        assert np.array_equal(f2.view(np.uint64), fin.view(np.uint64)), seed
+        for a, b in zip(cnt, cnt2):
+            assert np.array_equal(a, b), seed
+
+
+def test_single_placement_call_keeps_the_listing_order_of_replicas(eng):
+    # m_id2g_id lists group 1 before group 0: ties must go to group 1
+    lat = np.full((1, 2, 1), 0.1, np.float32)
+    m2g = np.array([[1, 0]], np.int32)
+    f, g = np.empty(3), np.empty(3, bool)
+    cnt = E.simulate_requests_mixed(eng, f, g, np.zeros(3), np.zeros(3, np.int32),
+                                    np.full(3, np.inf, np.float32), m2g, np.array([1, 1], np.int32), lat)
+    assert cnt[2].tolist() == [1, 2]
+
+
+def _run_config(eng, cfg, sols, seeds, flags):
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(sols, table)
+    streams = [cfg.stream(s) for s in seeds]
+    dws = [E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models) for st in streams]
+    batch = E.Batch(eng, dws, table, packed, flags)
+    batch.run()
+    batch.sync()
+    out = batch.fetch()
+    info = batch.info()
+    batch.close()
+    return out, table, packed, streams, info
+
+
+def test_config1_sanity_case(eng):
+    cfg = make_config(1)
+    out, table, packed, streams, _ = _run_config(eng, cfg, cfg.placements, [0], ALL)
+    ref = oracle_batch(streams[0], table, packed, want_per_request=True)
+    assert_batch_matches(out, ref, 0, packed[0], per_request=True, where="cfg1")
+    assert out["fp_ops"][0, 0] == ref["fp_ops"]
+    assert 0 < ref["n_good"][0] <= len(streams[0].tstamps)
+
+
+def test_config2_all_placements_all_seeds_per_request(eng):
+    cfg = make_config(2)
+    out, table, packed, streams, info = _run_config(eng, cfg, cfg.placements, cfg.base_seeds, ALL)
+    assert info["lanes"] == 256
+    total_ops = 0
+    for s, st in enumerate(streams):
+        ref = oracle_batch(st, table, packed, want_per_request=True)
+        assert_batch_matches(out, ref, s, packed[0], per_request=True, where=f"cfg2 seed {s}")
+        total_ops += ref["fp_ops"]
+    assert out["fp_ops"].sum() == total_ops
+
+
+def test_config2_ragged_batch_sizes(eng):
+    # batch sizes that do not fill a wavefront, and one that spills into a second tile
+    cfg = make_config(2, 70)
+    for n in (1, 3, 63, 65, 70):
+        out, table, packed, streams, _ = _run_config(eng, cfg, cfg.placements[:n], [1], ALL)
+        ref = oracle_batch(streams[0], table, packed, want_per_request=True)
+        assert_batch_matches(out, ref, 0, packed[0], per_request=True, where=f"cfg2 B={n}")
+
+
+def test_config3_greedy_step_candidates(eng):
+    cfg = make_config(3)
+    picks = list(range(0, 4096, 13))[:256]      # spread over both base placements
+    sols = [cfg.placements[i] for i in picks]
+    out, table, packed, streams, _ = _run_config(
+        eng, cfg, sols, [0], _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
+    ref = oracle_batch(streams[0], table, packed)
+    assert_batch_matches(out, ref, 0, packed[0], where="cfg3")
+
+
+def test_config4_subsample_counts_and_a_few_full_traces(eng):
+    cfg = make_config(4, 96)
+    out, table, packed, streams, info = _run_config(
+        eng, cfg, cfg.placements, [0], _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS | _lib.WANT_OP_COUNT)
+    print(info, flush=True)
+    ref = oracle_batch(streams[0], table, packed)
+    assert_batch_matches(out, ref, 0, packed[0], where="cfg4")
+    assert out["fp_ops"].sum() == ref["fp_ops"]
+    # full per-request traces (1M requests each) for 4 placements
+    out, table, packed, streams, _ = _run_config(eng, cfg, cfg.placements[:4], [0], ALL)
+    ref = oracle_batch(streams[0], table, packed, want_per_request=True)
+    assert_batch_matches(out, ref, 0, packed[0], per_request=True, where="cfg4 traces")
+
+
+def test_scores_only_mode_equals_full_mode(eng):
+    cfg = make_config(2)
+    a, *_ = _run_config(eng, cfg, cfg.placements, [0, 1], 0)
+    b, *_ = _run_config(eng, cfg, cfg.placements, [0, 1], ALL)
+    assert np.array_equal(a["n_good"], b["n_good"])
+    assert np.array_equal(a["latency_sum"], b["latency_sum"])
+
+
+def test_rerunning_a_batch_gives_the_same_answer(eng):
+    cfg = make_config(2)
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(cfg.placements, table)
+    st = cfg.stream(0)
+    dw = E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models)
+    batch = E.Batch(eng, [dw], table, packed, _lib.WANT_MODEL_COUNTS)
+    res = []
+    for _ in range(3):
+        batch.run()
+        batch.sync()
+        res.append(batch.fetch())
+    for r in res[1:]:
+        assert np.array_equal(r["n_good"], res[0]["n_good"])
+        assert np.array_equal(r["model_num_good"], res[0]["model_num_good"])
+
+
+def test_edge_inputs(eng):
+    cfg = make_config(2, 8)
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(cfg.placements, table)
+    # empty stream
+    dw = E.DeviceWorkload(eng, np.zeros(0), np.zeros(0, np.int32), np.zeros(0, np.float32), cfg.num_models)
+    out = E.evaluate(eng, [dw], table, cfg.placements, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
+    assert out["n_good"].sum() == 0 and out["model_num_requests"].sum() == 0
+    # unknown models, NaN / inf SLOs, a placement with an empty group and one with no model at all
+    from mms_amd.placement_policy.base_policy import ModelPlacement
+    from mms_amd.profiling import ParallelConfig
+    st = cfg.stream(0)
+    mids = st.model_ids.copy()
+    mids[::7] = -1
+    slos = st.slos.copy()
+    slos[::11] = np.nan
+    slos[::13] = np.inf
+    sols = list(cfg.placements) + [ModelPlacement([ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 1)], [[], [3, 4]]),
+                                   ModelPlacement([ParallelConfig(1, 1, 4)], [[]])]
+    packed = E.pack_placements(sols, table)
+    dw = E.DeviceWorkload(eng, st.tstamps, mids, slos, cfg.num_models)
+    batch = E.Batch(eng, [dw], table, packed, ALL)
+    batch.run(); batch.sync()
+    out = batch.fetch()
+    batch.close()
+    from mms_amd.synthetic import Stream
+    ref = oracle_batch(Stream(st.tstamps, mids, slos), table, packed, want_per_request=True)
+    assert_batch_matches(out, ref, 0, packed[0], per_request=True, where="edge")
+
+
+def test_error_codes(eng):
+    cfg = make_config(2, 4)
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    st = cfg.stream(0)
+    with pytest.raises(_lib.MmsimError) as e:
+        E.DeviceWorkload(eng, st.tstamps, st.model_ids + 1000, st.slos, cfg.num_models)
+    assert e.value.code == _lib.E_INVALID
+    dw = E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models)
+    num_groups, group_cfg, gm_off, gm_idx = E.pack_placements(cfg.placements, table)
+    bad = gm_idx.copy()
+    bad[0] = cfg.num_models + 5
+    with pytest.raises(_lib.MmsimError) as e:
+        E.Batch(eng, [dw], table, (num_groups, group_cfg, gm_off, bad), 0)
+    assert e.value.code == _lib.E_INVALID
+    bad_cfg = group_cfg.copy()
+    bad_cfg[0, 0] = 99
+    with pytest.raises(_lib.MmsimError) as e:
+        E.Batch(eng, [dw], table, (num_groups, bad_cfg, gm_off, gm_idx), 0)
+    assert e.value.code == _lib.E_INVALID
+    with pytest.raises(_lib.MmsimError) as e:
+        E.Engine(device=99)
+    assert e.value.code == _lib.E_INVALID
