@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""Benchmark of the placement-evaluation hot path on one MI355X.
+
+A "step" is one pass of the approximate simulator over the whole batch of
+candidate placements x arrival seeds of the workload (default: configuration 4,
+16384 placements x 8 seeds x ~1M requests each), with request streams and
+placement tables already resident in HBM.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 4] [--placements N]
+
+The CPU oracle is used here only for the `cpu_baseline` leg (a bounded sample of
+the same workload, timed on the host cores) and to cross-check the GPU counts
+of that sample; it is never part of what `value` measures.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+FP64_VECTOR_PEAK_FMA_TFLOPS = 78.6   # MI355X published fp64 vector peak, FMA counted as 2
+FP64_NON_FMA_PEAK_TOPS = 39.3        # the path has only add/max/compare: half of the above
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(cfg, table, stream, sols, n_threads):
+    """Times the C oracle (single thread, then n_threads threads over placement
+    slices) on `sols` x one stream.  Returns (result dict of 1-thread run, evals/s 1T, evals/s MT)."""
+    from mms_amd import engine as E
+    from helpers import oracle_batch
+    packed = E.pack_placements(sols, table)
+    t0 = time.perf_counter()
+    ref = oracle_batch(stream, table, packed)
+    t1 = time.perf_counter() - t0
+    evals = len(sols) * len(stream.tstamps)
+
+    chunks = [sols[i::n_threads] for i in range(n_threads)]
+    chunks = [c for c in chunks if c]
+    packs = [E.pack_placements(c, table) for c in chunks]
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(len(chunks)) as pool:      # ctypes releases the GIL during the call
+        list(pool.map(lambda p: oracle_batch(stream, table, p), packs))
+    tm = time.perf_counter() - t0
+    return ref, packed, evals / t1, evals / tm, t1
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", type=int, default=4, help="synthetic configuration 2..4 (plain simulator)")
+    ap.add_argument("--placements", type=int, default=None, help="truncate the candidate list")
+    ap.add_argument("--seeds", type=int, default=None, help="use only the first N arrival seeds")
+    ap.add_argument("--cpu-sample", type=int, default=1024, help="placements timed on the CPU oracle")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--flags", type=str, default="scores", choices=["scores", "model", "stats"],
+                    help="scores: goodput+latency only; model: + per-model counts; stats: + per-group counts")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build evaluates placements on ONE GPU; --gpus must be 1 "
+              "(lanes are independent, a multi-GPU run would only split the batch).", file=sys.stderr)
+        sys.exit(2)
+
+    from mms_amd import _lib, engine as E
+    from mms_amd.synthetic import make_config
+
+    t0 = time.perf_counter()
+    cfg = make_config(args.config, args.placements)
+    if cfg.batching:
+        print("bench.py: configuration 5 (batching) is not a bench line of this build", file=sys.stderr)
+        sys.exit(2)
+    seeds = list(cfg.base_seeds if args.seeds is None else cfg.base_seeds[:args.seeds])
+    streams = [cfg.stream(s) for s in seeds]
+    B = len(cfg.placements)
+    R_total = sum(len(s.tstamps) for s in streams)
+    log(f"[bench] {cfg.name}: {B} placements x {len(seeds)} seeds, {R_total} requests over seeds, "
+        f"inputs generated in {time.perf_counter() - t0:.1f}s")
+
+    eng = E.Engine.default()
+    dev = eng.device_info()
+    log(f"[bench] device: {dev}")
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    t0 = time.perf_counter()
+    packed = E.pack_placements(cfg.placements, table)
+    t_pack = time.perf_counter() - t0
+    flags = {"scores": 0, "model": _lib.WANT_MODEL_COUNTS,
+             "stats": _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS}[args.flags]
+    t0 = time.perf_counter()
+    dws = [E.DeviceWorkload(eng, s.tstamps, s.model_ids, s.slos, cfg.num_models) for s in streams]
+    batch = E.Batch(eng, dws, table, packed, flags)
+    t_upload = time.perf_counter() - t0
+    info = batch.info()
+    log(f"[bench] batch: {info}; python pack {t_pack:.2f}s, library pack+upload {t_upload:.2f}s")
+
+    for _ in range(args.warmup):
+        batch.run()
+        batch.sync()
+    kernel_ms = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        batch.run()
+        kernel_ms.append(batch.sync())          # HIP events around the kernel, on its stream
+    wall = time.perf_counter() - t0
+    out = batch.fetch()
+    batch.close()
+
+    evals_per_step = R_total * B
+    lanes = B * len(seeds)
+    sec_per_step = wall / args.steps
+    kernel_s = float(np.mean(kernel_ms)) / 1e3
+    value = evals_per_step / sec_per_step
+
+    # exact operation count of the reference loop on these inputs: one untimed pass
+    ops_batch = E.Batch(eng, dws, table, packed, _lib.WANT_OP_COUNT)
+    ops_batch.run()
+    ops_batch.sync()
+    ops_out = ops_batch.fetch()
+    ops_batch.close()
+    total_ops = int(ops_out["fp_ops"].sum())
+    assert np.array_equal(ops_out["n_good"], out["n_good"])
+    achieved_tops = total_ops / kernel_s / 1e12
+
+    result = {
+        "metric": "simulated request x placement evals/sec",
+        "value": value,
+        "unit": "evals/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec_per_step * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64",
+        "data": "synthetic",
+        "config": {"workload": f"config {cfg.index} ({cfg.name}): {cfg.num_models} models, "
+                               f"{cfg.num_devices} devices, {B} candidate placements x {len(seeds)} seeds, "
+                               f"{R_total // len(seeds)} requests/seed",
+                   "placements": B, "seeds": len(seeds), "requests_per_seed": R_total // len(seeds),
+                   "lanes": lanes, "outputs": args.flags, "inputs_resident_in_hbm": True},
+        "placements_per_sec": lanes / sec_per_step,
+        "kernel_ms": kernel_s * 1e3,
+        "goodput_mean": float(out["n_good"].sum() / evals_per_step),
+        "roofline": {
+            "bound": "valu_fp64",
+            "achieved": achieved_tops,
+            "peak": FP64_NON_FMA_PEAK_TOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved_tops / FP64_NON_FMA_PEAK_TOPS,
+            "frac_of_published_fma_peak": achieved_tops / FP64_VECTOR_PEAK_FMA_TFLOPS,
+            "ops_per_launch": total_ops,
+            "ops_per_eval": total_ops / evals_per_step,
+            "traffic": None,
+            "hbm_algorithmic_GBps": (info["stream_bytes"] * info["waves"] / max(len(seeds), 1)
+                                     + info["table_bytes"] * len(seeds)) / kernel_s / 1e9,
+            "note": "fp64 add/max/compare only (no FMA): peak = published 78.6 TFLOP/s / 2; "
+                    "achieved counts 2*stages+replicas+3 per dispatched request",
+        },
+    }
+
+    if not args.no_cpu:
+        n_threads = min(16, os.cpu_count() or 1)
+        sample = cfg.placements[:min(args.cpu_sample, B)]
+        ref, spacked, c1, cm, t1 = cpu_baseline(cfg, table, streams[0], sample, n_threads)
+        same = np.array_equal(out["n_good"][0, :len(sample)], ref["n_good"])
+        result["cpu_baseline"] = {
+            "value": c1, "unit": "evals/s", "cores": 1, "kind": "port",
+            "sample": f"first {len(sample)} placements x seed {seeds[0]} "
+                      f"({len(sample) * len(streams[0].tstamps)} evals, {t1:.1f}s), C oracle -O2, request loop only",
+            "value_all_cores": cm, "cores_all": n_threads,
+            "gpu_over_cpu_1core": value / c1, "gpu_over_cpu_all_cores": value / cm,
+            "gpu_counts_match_cpu_on_sample": bool(same),
+        }
+        if not same:
+            log("[bench] WARNING: GPU and CPU goodput counts differ on the CPU sample")
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

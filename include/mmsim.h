@@ -55,7 +55,7 @@ enum {
 /* Limits of the compiled kernels. */
 #define MMSIM_MAX_STAGES 32        /* pipeline stages of one group                */
 #define MMSIM_MAX_REPLICAS 64      /* groups hosting one model in one placement   */
-#define MMSIM_MAX_GROUPS 255       /* groups of one placement                     */
+#define MMSIM_MAX_GROUPS 254       /* groups of one placement                     */
 #define MMSIM_MAX_SLOTS 255        /* sum of pipeline stages over a placement     */
 #define MMSIM_MAX_CONFIGS 255      /* distinct parallel configurations            */
 
@@ -166,7 +166,7 @@ void mmsim_batch_destroy(mmsim_batch *batch);
 
 typedef struct {
     int32_t lanes, waves, n_seeds, B;
-    int32_t smax_bucket, rmax_bucket, slots, lds_bytes;
+    int32_t smax_bucket, max_replicas, slots, lds_bytes;
     int64_t requests_total;   /* sum of stream lengths over seeds                     */
     int64_t table_bytes;      /* device bytes of the packed placement tables          */
     int64_t stream_bytes;     /* device bytes of the request streams                  */

@@ -10,7 +10,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmmsim.so")
+# MMSIM_LIBRARY overrides the location (e.g. to try a differently built library).
+LIB_PATH = os.environ.get("MMSIM_LIBRARY") or os.path.join(_HERE, "libmmsim.so")
 
 MMSIM_OK = 0
 E_INVALID, E_UNSUPPORTED, E_HIP, E_NOMEM, E_OVERFLOW = -1, -2, -3, -4, -5
@@ -54,7 +55,7 @@ class DeviceInfo(C.Structure):
 
 class BatchInfo(C.Structure):
     _fields_ = [("lanes", C.c_int32), ("waves", C.c_int32), ("n_seeds", C.c_int32), ("B", C.c_int32),
-                ("smax_bucket", C.c_int32), ("rmax_bucket", C.c_int32), ("slots", C.c_int32),
+                ("smax_bucket", C.c_int32), ("max_replicas", C.c_int32), ("slots", C.c_int32),
                 ("lds_bytes", C.c_int32), ("requests_total", C.c_int64), ("table_bytes", C.c_int64),
                 ("stream_bytes", C.c_int64)]
 

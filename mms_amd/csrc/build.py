@@ -27,9 +27,9 @@ FLAGS = [
 ]
 
 
-def _compile(src, extra):
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(HERE, src), "-o", obj]
+def _compile(src, extra, src_dir=HERE, obj_dir=OBJ_DIR):
+    obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(src_dir, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{proc.stdout}\n{proc.stderr}")
@@ -38,20 +38,22 @@ def _compile(src, extra):
     return obj, "\n".join(warn)
 
 
-def build(verbose=False, extra_flags=()):
-    os.makedirs(OBJ_DIR, exist_ok=True)
+def build(verbose=False, extra_flags=(), src_dir=HERE, out=OUT):
+    """Compiles SOURCES from `src_dir` and links them into `out`."""
+    obj_dir = os.path.join(src_dir, "build")
+    os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
-        results = list(pool.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
+        results = list(pool.map(lambda s: _compile(s, list(extra_flags), src_dir, obj_dir), SOURCES))
     objs = [o for o, _ in results]
     if verbose:
         for _, w in results:
             if w:
                 print(w, file=sys.stderr)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", OUT]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
-    return OUT
+    return out
 
 
 if __name__ == "__main__":

@@ -88,15 +88,18 @@ struct mmsim_batch {
     mmsim_ctx *ctx = nullptr;
     uint32_t flags = 0;
     int32_t n_seeds = 0, B = 0, M = 0, Gmax = 0, tiles = 0, waves = 0;
-    int32_t smax_bucket = 0, rmax_bucket = 0, nslots = 0;
+    int32_t smax_bucket = 0, rmax_all = 0, nslots = 0, waves_per_block = 1;
     size_t lds_bytes = 0;
     int64_t Rmax = 0, Rtotal = 0;
     std::vector<const mmsim_workload *> wl;
+    std::vector<int32_t> pos;  // pos[placement] = tile * 64 + lane it is simulated on
 
     DevBuf<Req> streams;
     DevBuf<int64_t> stream_off;
-    DevBuf<uint32_t> rep;
-    DevBuf<int32_t> rmax;
+    DevBuf<uint64_t> rep8;
+    DevBuf<uint8_t> repx;
+    DevBuf<uint8_t> rmax;
+    DevBuf<uint32_t> ginfo;
     DevBuf<float> lat;
     DevBuf<int32_t> n_good;
     DevBuf<double> lat_sum;
@@ -135,7 +138,7 @@ int check_tables(const mmsim_tables *t) {
 int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLists *out) {
     if (!p || !p->num_groups || !p->group_cfg || !p->gm_off) return fail(MMSIM_E_INVALID, "placements: null pointer");
     if (p->B < 1 || p->Gmax < 1) return fail(MMSIM_E_INVALID, "placements: B and Gmax must be >= 1");
-    if (p->Gmax > MMSIM_MAX_GROUPS) return fail(MMSIM_E_UNSUPPORTED, "placements: more than 255 groups");
+    if (p->Gmax > MMSIM_MAX_GROUPS) return fail(MMSIM_E_UNSUPPORTED, "placements: more than 254 groups");
     out->B = p->B;
     out->M = M;
     out->Gmax = p->Gmax;
@@ -211,36 +214,123 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
     if (rmax_all > MMSIM_MAX_REPLICAS) return fail(MMSIM_E_UNSUPPORTED, "a model has more than 64 replicas in one placement");
     b->smax_bucket = smax_bucket_for(smax);
-    b->rmax_bucket = rmax_bucket_for(rmax_all);
-    if (b->smax_bucket < 0 || b->rmax_bucket < 0) return fail(MMSIM_E_UNSUPPORTED, "no kernel bucket for this shape");
+    b->rmax_all = rmax_all;
+    if (b->smax_bucket < 0) return fail(MMSIM_E_UNSUPPORTED, "no kernel bucket for this many pipeline stages");
     b->nslots = nslots;
-    b->lds_bytes = (size_t)nslots * kWave * sizeof(double) +
-                   ((flags & MMSIM_WANT_GROUP_COUNTS) ? (size_t)2 * Gmax * kWave * sizeof(uint32_t) : 0);
-    if (b->lds_bytes > (size_t)ctx->max_lds)
-        return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups)");
 
-    // ---- replica descriptors [tiles][M][RB][64] and per-tile replica maxima
-    const int RB = b->rmax_bucket;
-    std::vector<uint32_t> rep((size_t)b->tiles * M * RB * kWave, kEmpty);
-    std::vector<int32_t> rmax((size_t)b->tiles * M, 0);
+    // ---- compact batch-size-1 latency table.  General form: row of model m = its stage
+    //      latencies for configuration 0, then configuration 1, ... (the cfg_pp[c] real
+    //      stages only).  When every (model, config) has one latency for all its stages the
+    //      row is just one value per configuration.
+    bool uniform_stages = true;
+    for (int32_t m = 0; m < M && uniform_stages; ++m)
+        for (int c = 0; c < C && uniform_stages; ++c) {
+            const float *row = t->cfg_lat + ((size_t)m * C + c) * t->Smax * t->NB;
+            for (int k = 1; k < t->cfg_pp[c]; ++k)
+                if (std::memcmp(&row[(size_t)k * t->NB], &row[0], sizeof(float)) != 0) uniform_stages = false;
+        }
+    std::vector<int32_t> lat_off(C + 1, 0);
+    for (int c = 0; c < C; ++c) lat_off[c + 1] = lat_off[c] + (uniform_stages ? 1 : t->cfg_pp[c]);
+    const int32_t lat_row = lat_off[C];
+    if (lat_row > kMaxLatRow) return fail(MMSIM_E_UNSUPPORTED, "configurations have more than 1023 pipeline stages in total");
+    std::vector<float> lat((size_t)M * lat_row);
+    for (int32_t m = 0; m < M; ++m)
+        for (int c = 0; c < C; ++c)
+            for (int k = 0; k < (uniform_stages ? 1 : t->cfg_pp[c]); ++k) {
+                const float v = t->cfg_lat[(((size_t)m * C + c) * t->Smax + k) * t->NB];
+                if (v != v) return fail(MMSIM_E_INVALID, "tables: a stage latency is NaN");
+                if (v < 0.0f) return fail(MMSIM_E_INVALID, "tables: a stage latency is negative");
+                lat[(size_t)m * lat_row + lat_off[c] + k] = v;
+            }
+
+    // ---- LDS budget: shared latency table + per-wavefront private region
+    const int32_t rmax_lds_bytes = (M + 15) & ~15;
+    const size_t wave_bytes = ((size_t)kStageBytes + rmax_lds_bytes + (size_t)(Gmax + 1) * kWave * sizeof(uint32_t) +
+                               (size_t)nslots * kWave * sizeof(double) +
+                               ((flags & MMSIM_WANT_GROUP_COUNTS) ? (size_t)2 * Gmax * kWave * sizeof(uint32_t) : 0) + 15) & ~(size_t)15;
+    const size_t lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
+    int lat_in_lds = 1;
+    int wpb = 0;
+    if (lat_bytes + wave_bytes <= (size_t)ctx->max_lds) wpb = (int)std::min<size_t>(kMaxWavesPerBlock, ((size_t)ctx->max_lds - lat_bytes) / wave_bytes);
+    if (wpb == 0) {
+        lat_in_lds = 0;
+        wpb = (int)std::min<size_t>(kMaxWavesPerBlock, (size_t)ctx->max_lds / wave_bytes);
+    }
+    if (wpb == 0) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
+    wpb = std::min(wpb, b->tiles);
+    b->waves_per_block = wpb;
+    b->lds_bytes = (lat_in_lds ? lat_bytes : 0) + (size_t)wpb * wave_bytes;
+
+    // ---- lane assignment.  A wavefront walks as many pipeline stages as its deepest
+    //      lane needs, so placements are ordered by depth before they are cut into
+    //      tiles of 64: first by their deepest group, then by the expected depth of a
+    //      request (request-count weighted depth of the deepest group hosting each model).
+    {
+        std::vector<double> weight(M, 0.0);
+        for (int s = 0; s < n_seeds; ++s)
+            for (int32_t m = 0; m < M; ++m) weight[m] += (double)wls[s]->model_num_requests[m];
+        std::vector<int32_t> deepest(B, 0);
+        std::vector<double> expected(B, 0.0);
+        std::vector<int32_t> depth_of(M);
+        for (int32_t p = 0; p < B; ++p) {
+            std::fill(depth_of.begin(), depth_of.end(), 0);
+            for (int32_t m = 0; m < M; ++m)
+                for (int64_t x = rl.off[(size_t)p * M + m]; x < rl.off[(size_t)p * M + m + 1]; ++x) {
+                    const int32_t g = rl.grp[(size_t)x];
+                    if (g < 0 || g >= rl.num_groups[p]) return fail(MMSIM_E_INVALID, "replica list names a group that does not exist");
+                    depth_of[m] = std::max(depth_of[m], t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]]);
+                }
+            for (int32_t m = 0; m < M; ++m) {
+                deepest[p] = std::max(deepest[p], depth_of[m]);
+                expected[p] += weight[m] * depth_of[m];
+            }
+        }
+        std::vector<int32_t> order(B);
+        for (int32_t p = 0; p < B; ++p) order[p] = p;
+        std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
+            if (deepest[x] != deepest[y]) return deepest[x] < deepest[y];
+            return expected[x] < expected[y];
+        });
+        b->pos.assign(B, 0);
+        for (int32_t i = 0; i < B; ++i) b->pos[order[i]] = i;
+    }
+
+    // ---- per lane group descriptors [tiles][Gmax+1][64]; row Gmax stays empty
+    std::vector<uint32_t> ginfo((size_t)b->tiles * (Gmax + 1) * kWave, kEmpty);
     for (int32_t p = 0; p < B; ++p) {
-        const int tile = p / kWave, lane = p % kWave;
+        const int tile = b->pos[p] / kWave, lane = b->pos[p] % kWave;
+        for (int32_t g = 0; g < rl.num_groups[p]; ++g) {
+            const int32_t c = rl.group_cfg[(size_t)p * Gmax + g];
+            ginfo[((size_t)tile * (Gmax + 1) + g) * kWave + lane] =
+                pack_desc(slot0[(size_t)p * Gmax + g], (uint32_t)t->cfg_pp[c], (uint32_t)lat_off[c], (uint32_t)g);
+        }
+    }
+    // ---- replica lists as group indices: first 8 packed [tiles][M][64] x u64, the rest
+    //      [tiles][M][RX][64] x u8; missing entries name the empty row Gmax
+    const int RX = std::max(rmax_all - kPackedReplicas, 0);
+    const uint64_t none8 = 0x0101010101010101ull * (uint64_t)Gmax;
+    std::vector<uint64_t> rep8((size_t)b->tiles * M * kWave, none8);
+    std::vector<uint8_t> repx((size_t)b->tiles * M * RX * kWave, (uint8_t)Gmax);
+    std::vector<uint8_t> rmax((size_t)b->tiles * M, 0);
+    for (int32_t p = 0; p < B; ++p) {
+        const int tile = b->pos[p] / kWave, lane = b->pos[p] % kWave;
         for (int32_t m = 0; m < M; ++m) {
             const int64_t lo = rl.off[(size_t)p * M + m], hi = rl.off[(size_t)p * M + m + 1];
-            int32_t &rm = rmax[(size_t)tile * M + m];
-            rm = std::max<int32_t>(rm, (int32_t)(hi - lo));
+            uint8_t &rm = rmax[(size_t)tile * M + m];
+            rm = std::max<uint8_t>(rm, (uint8_t)(hi - lo));
+            uint64_t word = none8;
             for (int64_t x = lo; x < hi; ++x) {
                 const int32_t g = rl.grp[(size_t)x];
                 if (g < 0 || g >= rl.num_groups[p]) return fail(MMSIM_E_INVALID, "replica list names a group that does not exist");
-                const int32_t c = rl.group_cfg[(size_t)p * Gmax + g];
-                rep[(((size_t)tile * M + m) * RB + (size_t)(x - lo)) * kWave + lane] =
-                    pack_desc(slot0[(size_t)p * Gmax + g], (uint32_t)t->cfg_pp[c], (uint32_t)c, (uint32_t)g);
+                const int j = (int)(x - lo);
+                if (j < kPackedReplicas)
+                    word = (word & ~(0xFFull << (8 * j))) | ((uint64_t)g << (8 * j));
+                else
+                    repx[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = (uint8_t)g;
             }
+            rep8[((size_t)tile * M + m) * kWave + lane] = word;
         }
     }
-    // ---- batch-size-1 latency table [M][C][Smax]
-    std::vector<float> lat((size_t)M * C * t->Smax);
-    for (size_t i = 0; i < lat.size(); ++i) lat[i] = t->cfg_lat[i * (size_t)t->NB];
 
     // ---- request streams back to back
     std::vector<int64_t> soff(n_seeds + 1, 0);
@@ -259,10 +349,14 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                                    hipMemcpyDeviceToDevice, st));
     HIP_TRY(b->stream_off.alloc(soff.size()));
     HIP_TRY(hipMemcpyAsync(b->stream_off.p, soff.data(), sizeof(int64_t) * soff.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(b->rep.alloc(rep.size()));
-    HIP_TRY(hipMemcpyAsync(b->rep.p, rep.data(), sizeof(uint32_t) * rep.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(b->rep8.alloc(rep8.size()));
+    HIP_TRY(hipMemcpyAsync(b->rep8.p, rep8.data(), sizeof(uint64_t) * rep8.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(b->repx.alloc(repx.size()));
+    if (!repx.empty()) HIP_TRY(hipMemcpyAsync(b->repx.p, repx.data(), repx.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(b->ginfo.alloc(ginfo.size()));
+    HIP_TRY(hipMemcpyAsync(b->ginfo.p, ginfo.data(), sizeof(uint32_t) * ginfo.size(), hipMemcpyHostToDevice, st));
     HIP_TRY(b->rmax.alloc(rmax.size()));
-    HIP_TRY(hipMemcpyAsync(b->rmax.p, rmax.data(), sizeof(int32_t) * rmax.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(b->rmax.p, rmax.data(), rmax.size(), hipMemcpyHostToDevice, st));
     HIP_TRY(b->lat.alloc(lat.size()));
     HIP_TRY(hipMemcpyAsync(b->lat.p, lat.data(), sizeof(float) * lat.size(), hipMemcpyHostToDevice, st));
 
@@ -286,12 +380,18 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     MixedArgs &a = b->args;
     a.streams = b->streams.p;
     a.stream_off = b->stream_off.p;
-    a.rep = b->rep.p;
+    a.rep8 = b->rep8.p;
+    a.repx = b->repx.p;
     a.rmax = b->rmax.p;
+    a.ginfo = b->ginfo.p;
     a.lat = b->lat.p;
     a.M = M;
-    a.C = C;
-    a.lat_stride = t->Smax;
+    a.lat_row = lat_row;
+    a.rep_extra = RX;
+    a.lat_in_lds = lat_in_lds;
+    a.uniform_stages = uniform_stages ? 1 : 0;
+    a.wave_lds_bytes = (int32_t)wave_bytes;
+    a.rmax_lds_bytes = rmax_lds_bytes;
     a.n_seeds = n_seeds;
     a.B = B;
     a.tiles = b->tiles;
@@ -381,6 +481,7 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
     std::vector<Req> host((size_t)R);
     for (int64_t i = 0; i < R; ++i) {
         if (model_ids[i] >= M) return fail(MMSIM_E_INVALID, "workload_create: model id >= M");
+        if (tstamps[i] != tstamps[i]) return fail(MMSIM_E_INVALID, "workload_create: arrival time is NaN");
         host[i].t = tstamps[i];
         host[i].m = model_ids[i] < 0 ? -1 : model_ids[i];
         host[i].slo = slos[i];
@@ -423,7 +524,7 @@ int mmsim_batch_run(mmsim_batch *b) {
         HIP_TRY(hipMemsetAsync(b->model_good.p, 0, b->model_good.bytes(), ctx->stream));
     HIP_TRY(hipEventRecord(b->ev_start, ctx->stream));
     std::string err;
-    hipError_t e = launch_sim_mixed(b->args, b->smax_bucket, b->rmax_bucket, b->lds_bytes, ctx->stream, &err);
+    hipError_t e = launch_sim_mixed(b->args, b->smax_bucket, b->waves_per_block, b->lds_bytes, ctx->stream, &err);
     if (e != hipSuccess) return fail(MMSIM_E_HIP, err);
     HIP_TRY(hipEventRecord(b->ev_stop, ctx->stream));
     b->ran = true;
@@ -465,7 +566,7 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
     }
     for (int s = 0; s < b->n_seeds; ++s)
         for (int32_t p = 0; p < B; ++p) {
-            const size_t src = (size_t)s * tiles * kWave + p;
+            const size_t src = (size_t)s * tiles * kWave + b->pos[p];
             out->n_good[(size_t)s * B + p] = ng[src];
             out->latency_sum[(size_t)s * B + p] = ls[src];
             if (out->status) out->status[(size_t)s * B + p] = 0;
@@ -477,9 +578,9 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
         HIP_TRY(hipMemcpy(h.data(), dev.p, dev.bytes(), hipMemcpyDeviceToHost));
         for (int s = 0; s < b->n_seeds; ++s)
             for (int32_t p = 0; p < B; ++p) {
-                const size_t wave = (size_t)s * tiles + p / kWave;
+                const size_t wave = (size_t)s * tiles + b->pos[p] / kWave;
                 for (int32_t x = 0; x < width; ++x)
-                    dst[((size_t)s * B + p) * width + x] = h[(wave * width + x) * kWave + p % kWave];
+                    dst[((size_t)s * B + p) * width + x] = h[(wave * width + x) * kWave + b->pos[p] % kWave];
             }
         return MMSIM_OK;
     };
@@ -501,14 +602,18 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
         const size_t Rm = (size_t)b->Rmax;
         std::vector<double> hf(Rm * kWave);
         std::vector<uint8_t> hg(Rm * kWave);
+        std::vector<int32_t> owner((size_t)tiles * kWave, -1);  // placement simulated on each lane
+        for (int32_t p = 0; p < B; ++p) owner[b->pos[p]] = p;
         for (int s = 0; s < b->n_seeds; ++s)
             for (int32_t tile = 0; tile < tiles; ++tile) {
                 const size_t wave = (size_t)s * tiles + tile;
                 HIP_TRY(hipMemcpy(hf.data(), b->finish.p + wave * Rm * kWave, sizeof(double) * Rm * kWave, hipMemcpyDeviceToHost));
                 HIP_TRY(hipMemcpy(hg.data(), b->good.p + wave * Rm * kWave, Rm * kWave, hipMemcpyDeviceToHost));
                 const size_t Rs = (size_t)b->wl[s]->R;
-                for (int l = 0; l < kWave && tile * kWave + l < B; ++l) {
-                    const size_t row = ((size_t)s * B + (size_t)tile * kWave + l) * Rm;
+                for (int l = 0; l < kWave; ++l) {
+                    const int32_t p = owner[(size_t)tile * kWave + l];
+                    if (p < 0) continue;
+                    const size_t row = ((size_t)s * B + (size_t)p) * Rm;
                     for (size_t i = 0; i < Rs; ++i) {
                         out->finish[row + i] = hf[i * kWave + l];
                         out->good[row + i] = hg[i * kWave + l];
@@ -535,11 +640,11 @@ int mmsim_batch_get_info(const mmsim_batch *b, mmsim_batch_info *out) {
     out->n_seeds = b->n_seeds;
     out->B = b->B;
     out->smax_bucket = b->smax_bucket;
-    out->rmax_bucket = b->rmax_bucket;
+    out->max_replicas = b->rmax_all;
     out->slots = b->nslots;
     out->lds_bytes = (int32_t)b->lds_bytes;
     out->requests_total = b->Rtotal;
-    out->table_bytes = (int64_t)(b->rep.bytes() + b->rmax.bytes() + b->lat.bytes());
+    out->table_bytes = (int64_t)(b->rep8.bytes() + b->repx.bytes() + b->ginfo.bytes() + b->rmax.bytes() + b->lat.bytes());
     out->stream_bytes = (int64_t)b->streams.bytes();
     return MMSIM_OK;
 }
@@ -568,7 +673,7 @@ int mmsim_simulate_requests_mixed(mmsim_ctx *ctx, double *finish, uint8_t *good,
     if (!m_id2g_id || !num_stages || !stage_latency || !model_num_requests || !model_num_good_requests ||
         !group_num_requests || !group_num_good_requests || (num_requests > 0 && (!finish || !good)))
         return fail(MMSIM_E_INVALID, "simulate_requests_mixed: null pointer");
-    if (G > MMSIM_MAX_GROUPS) return fail(MMSIM_E_UNSUPPORTED, "simulate_requests_mixed: more than 255 groups");
+    if (G > MMSIM_MAX_GROUPS) return fail(MMSIM_E_UNSUPPORTED, "simulate_requests_mixed: more than 254 groups");
     // every group is its own latency-table column
     mmsim_tables t{};
     t.M = M;

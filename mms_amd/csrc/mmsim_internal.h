@@ -11,8 +11,8 @@
 
 namespace mmsim {
 
-// One request as the kernels read it: 16 bytes, so a wavefront fetches a
-// request with one scalar 128-bit load.
+// One request as the kernels read it: 16 bytes, so a block of 64 requests is
+// one coalesced 1 KiB load per wavefront.
 struct __attribute__((aligned(16))) Req {
     double t;
     int32_t m;
@@ -20,33 +20,47 @@ struct __attribute__((aligned(16))) Req {
 };
 static_assert(sizeof(Req) == 16, "Req must be 16 bytes");
 
-// Replica descriptor: one 32-bit word per (placement, model, replica).
-//   bits  0..7   first clock slot of the group (slots are the placement's
-//                pipeline stages laid end to end)
+// Group descriptor: one 32-bit word per (placement, group), kept per lane in LDS.
+//   bits  0..7   clock slot of the group's LAST pipeline stage (slots are the
+//                placement's pipeline stages laid end to end)
 //   bits  8..12  stages of the group minus one
-//   bits 13..20  configuration index (column of the latency table)
-//   bits 21..28  group index within the placement
-// kEmpty marks "no such replica".
-constexpr uint32_t kEmpty = 0xFFFFFFFFu;
-__host__ __device__ inline uint32_t pack_desc(uint32_t slot0, uint32_t stages, uint32_t cfg, uint32_t group) {
-    return slot0 | ((stages - 1u) << 8) | (cfg << 13) | (group << 21);
+//   bits 13..22  offset of the group's configuration inside a model's row of
+//                the compact latency table
+//   bits 23..30  group index within the placement
+// kEmpty (sign bit set, slot field 0) marks "no such group".
+//
+// The replicas of a model are listed as group indices, one byte each, eight to
+// a 64-bit word per (placement, model); unused bytes hold the index of the
+// extra, empty descriptor row (num_groups_max).
+constexpr uint32_t kEmpty = 0x80000000u;
+__host__ __device__ inline uint32_t pack_desc(uint32_t slot0, uint32_t stages, uint32_t lat_off, uint32_t group) {
+    return (slot0 + stages - 1u) | ((stages - 1u) << 8) | (lat_off << 13) | (group << 23);
 }
-__host__ __device__ inline uint32_t desc_slot0(uint32_t d) { return d & 0xFFu; }
-__host__ __device__ inline uint32_t desc_stages(uint32_t d) { return ((d >> 8) & 0x1Fu) + 1u; }
-__host__ __device__ inline uint32_t desc_cfg(uint32_t d) { return (d >> 13) & 0xFFu; }
-__host__ __device__ inline uint32_t desc_group(uint32_t d) { return (d >> 21) & 0xFFu; }
+__host__ __device__ inline uint32_t desc_last_slot(uint32_t d) { return d & 0xFFu; }
+__host__ __device__ inline uint32_t desc_stages_m1(uint32_t d) { return (d >> 8) & 0x1Fu; }
+__host__ __device__ inline uint32_t desc_lat_off(uint32_t d) { return (d >> 13) & 0x3FFu; }
+__host__ __device__ inline uint32_t desc_group(uint32_t d) { return (d >> 23) & 0xFFu; }
+constexpr int kMaxLatRow = 1023;  // floats per model in the compact latency table
+constexpr int kPackedReplicas = 8;
 
 constexpr int kWave = 64;
+constexpr int kStageBytes = kWave * (int)sizeof(Req);  // one staged block of requests
 
 // Arguments of the plain (non-batching) simulation kernel.
 struct MixedArgs {
     const Req *streams;          // all seeds' requests, back to back
     const int64_t *stream_off;   // [n_seeds+1] element offsets into streams
-    const uint32_t *rep;         // [tiles][M][rmax_bucket][64] replica descriptors
-    const int32_t *rmax;         // [tiles][M] most replicas of model m over the tile's lanes
-    const float *lat;            // [M][C][lat_stride] stage latencies (batch size 1)
-    int32_t M, C, lat_stride;
+    const uint64_t *rep8;        // [tiles][M][64] group indices of the first 8 replicas, one byte each
+    const uint8_t *repx;         // [tiles][M][rep_extra][64] group indices of replicas 8, 9, ...
+    const uint8_t *rmax;         // [tiles][M] most replicas of model m over the tile's lanes
+    const uint32_t *ginfo;       // [tiles][Gmax+1][64] group descriptors (row Gmax is kEmpty)
+    const float *lat;            // [M][lat_row] compact stage latencies (batch size 1)
+    int32_t M, lat_row, rep_extra;
     int32_t n_seeds, B, tiles, nslots, Gmax;
+    int32_t lat_in_lds;          // 1: the block keeps a copy of lat in LDS
+    int32_t uniform_stages;      // 1: all stages of a (model, config) have the same latency; lat is [M][C]
+    int32_t wave_lds_bytes;      // LDS bytes of one wavefront's private region
+    int32_t rmax_lds_bytes;      // M rounded up to 16
     int64_t Rmax;                // longest stream (row pitch of per-request outputs)
     double fixed_overhead;
     uint32_t flags;
@@ -61,11 +75,11 @@ struct MixedArgs {
     int64_t *fp_ops;             // [n_seeds][tiles*64]
 };
 
-// Picks the compiled (stage, replica) bucket and launches.  Returns a HIP error.
-hipError_t launch_sim_mixed(const MixedArgs &args, int smax, int rmax_bucket, size_t lds_bytes,
+// Launches the plain simulator with `waves_per_block` wavefronts per workgroup.
+hipError_t launch_sim_mixed(const MixedArgs &args, int smax_bucket, int waves_per_block, size_t lds_bytes,
                             hipStream_t stream, std::string *err);
-// Smallest compiled bucket >= value, or -1.
+// Smallest compiled stage bucket >= value, or -1.
 int smax_bucket_for(int smax);
-int rmax_bucket_for(int rmax);
+constexpr int kMaxWavesPerBlock = 4;
 
 }  // namespace mmsim

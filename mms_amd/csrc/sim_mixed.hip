@@ -5,167 +5,374 @@
 // placements at once.  One lane simulates one (placement, arrival seed) pair;
 // the 64 lanes of a wavefront hold 64 placements that walk the SAME request
 // stream in lockstep, so everything that depends only on the request
-// (arrival time, model id, SLO) is wave-uniform and is fetched with scalar
-// loads, while everything that depends on the placement is per lane:
+// (arrival time, model id, SLO) is wave-uniform, while everything that depends
+// on the placement is per lane.  Nothing in a request's dependency chain
+// touches global memory:
 //
-//   * per-lane stage clocks live in LDS as clk[slot][lane] (8 bytes each).
-//     The slots of a lane are its groups' pipeline stages laid end to end;
-//     the bank an access hits depends on the lane only, so any per-lane slot
-//     choice is conflict free.
-//   * the replicas of the request's model are 32-bit descriptors
-//     rep[tile][model][j][lane] (coalesced 256-byte rows), listed in the
-//     order the reference scans them; a descriptor carries the group's first
-//     slot, stage count, latency-table column and group index.
-//   * group choice (strictly smallest last-stage clock, first listed wins
-//     ties) and the SLO decision are selects / exec-masked stores, with
-//     wave-uniform early exits when no lane has another replica or stage.
+//   * requests are fetched 64 at a time with one coalesced 1 KiB load per
+//     wavefront (one block ahead, into registers), parked in LDS and read
+//     back with broadcast LDS reads;
+//   * the replicas of the request's model are group indices, one byte each,
+//     eight to a 64-bit word rep8[tile][model][lane] (one coalesced 512-byte
+//     load per request, listed in the order the reference scans them),
+//     fetched one chunk of requests ahead into registers; the load count per
+//     chunk is fixed so the wait counters let the prefetch overlap;
+//   * a per-lane table of group descriptors (last-stage clock slot, stage
+//     count, latency-row offset) lives in LDS as ginfo[group][lane];
+//   * per-lane stage clocks live in LDS as clk[slot][lane] (8 bytes each);
+//     the slots of a lane are its groups' pipeline stages laid end to end.
+//     The bank an access hits depends on the lane only, so any per-lane
+//     group or slot choice is conflict free;
+//   * stage latencies live in a compact table lat[model][config stage] that
+//     the workgroup keeps in LDS (shared by its wavefronts).  When every
+//     (model, config) has one latency for all its stages the table shrinks
+//     to lat[model][config] and the per-stage latency reads disappear.
+//
+// Group choice (strictly smallest last-stage clock, first listed wins ties)
+// is a select chain; the stage walk and the commit are nests of divergent
+// ifs, which the compiler turns into exec narrowing with a wave-uniform exit
+// as soon as no lane has another stage.
+//
+// A lane whose request cannot meet its SLO even if it only had to wait for
+// the chosen group's last stage skips the walk: with t >= arrival at every
+// stage and rounding monotone,
+//   fl(fl(fl(max(arrival, clk_last) + lat_last) + overhead) - arrival)
+// never exceeds the latency the full walk would produce, so "that bound > slo"
+// implies the reference's reject.  It only shortens the walk of the
+// wavefront; results are identical.
 //
 // Arithmetic is fp64 add / max / sub / compare in the reference's order;
-// fp32 operands (latencies, SLOs) are widened first.  Compiled with
-// -ffp-contract=off (there is no multiply to contract anyway).
+// fp32 operands (latencies, SLOs) are widened first.  Arrival times and
+// latencies are never NaN and latencies never negative (the host rejects
+// them), so the hardware max is an exact select.  Compiled with
+// -ffp-contract=off; there is no multiply anyway.
 //
-// Workgroup = one wavefront.  Lanes never exchange data, so there are no
-// barriers.  blockIdx.x = tile * n_seeds + seed, which puts the waves that
-// read the same stream on the same XCD when n_seeds is a multiple of 8.
+// Workgroup = up to 4 wavefronts that share only the read-only latency
+// table; after the single barrier that publishes it, wavefronts run
+// independently (lanes never exchange data).
+// blockIdx.x = tile_group * n_seeds + seed: with n_seeds a multiple of 8 all
+// wavefronts that read one stream sit on one XCD and share its L2.
 
 #include "mmsim_internal.h"
+#include "walk_asm.inc"
 
 namespace mmsim {
 
 namespace {
 
-template <int N>
-struct ChunkFor {
-    // requests whose descriptors are fetched ahead as one group; bounded so
-    // that the descriptor registers of a chunk stay within ~64 VGPRs
-    static constexpr int value = N <= 8 ? 8 : (N <= 16 ? 4 : (N <= 32 ? 2 : 1));
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// max of two doubles that are never NaN: one v_max_f64 without the input
+// quieting the generic fmax lowering adds.
+__device__ __forceinline__ double vmax(double x, double y) {
+    double r;
+    asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y));
+    return r;
+}
+
+// 32-bit LDS byte address of a pointer into shared memory (for ds_* in inline asm).
+__device__ __forceinline__ uint32_t lds_addr(const void *p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
+template <int I>
+struct Idx {
+    static constexpr int value = I;
 };
 
-template <int SMAX, int RMAX>
-__global__ __launch_bounds__(kWave) void sim_mixed_kernel(const MixedArgs a) {
-    extern __shared__ double lds_clk[];  // [nslots][64] then optional group counters
+// f(Idx<0>), f(Idx<1>), ... while f returns true, at most N times.  Compile-time
+// recursion: every array index inside f is a constant, arrays stay in registers.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_while(F &&f) {
+    if constexpr (I < N) {
+        if (f(Idx<I>{})) static_while<I + 1, N>(static_cast<F &&>(f));
+    }
+}
 
-    const int lane = threadIdx.x;
-    const int seed = blockIdx.x % a.n_seeds;
-    const int tile = blockIdx.x / a.n_seeds;
-    const int wave = seed * a.tiles + tile;
+// if (c(0)) { b(0); if (c(1)) { b(1); ... } } with per-lane conditions.
+template <int I, int N, typename C, typename B>
+__device__ __forceinline__ void static_nest(C &&c, B &&b) {
+    if constexpr (I < N) {
+        if (c(Idx<I>{})) {
+            b(Idx<I>{});
+            static_nest<I + 1, N>(static_cast<C &&>(c), static_cast<B &&>(b));
+        }
+    }
+}
+
+// Stage walk in blocks [0,1) [1,2) [2,4) [4,8) ...: one wave-uniform test per
+// block ("does any lane reach this depth?"), nested per-lane ifs inside.
+template <int LO, int HI, int N, typename C, typename B>
+__device__ __forceinline__ void walk_blocks(C &&c, B &&b) {
+    if constexpr (LO < N) {
+        if (__ballot(c(Idx<LO>{})) != 0ull) {
+            static_nest<LO, (HI < N ? HI : N)>(static_cast<C &&>(c), static_cast<B &&>(b));
+            walk_blocks<HI, 2 * HI, N>(static_cast<C &&>(c), static_cast<B &&>(b));
+        }
+    }
+}
+
+constexpr int kChunk = 8;  // requests whose replica words are fetched ahead together
+
+struct Chunk {
+    int m[kChunk];        // wave-uniform model id (or -1)
+    int nrep[kChunk];     // wave-uniform replica bound of the tile for that model
+    uint64_t g8[kChunk];  // per-lane group indices of the first 8 replicas
+};
+
+template <int SMAX, bool LATLDS, bool UNIFORM>
+__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(const MixedArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    constexpr int CH = kChunk;
+    constexpr int RREG = kPackedReplicas;
+
+    const int W = (int)(blockDim.x >> 6);
+    const int wv = uniform((int)(threadIdx.x >> 6));
+    const int lane = (int)(threadIdx.x & 63);
+    const int seed = (int)(blockIdx.x % (unsigned)a.n_seeds);
+    const int tile = (int)(blockIdx.x / (unsigned)a.n_seeds) * W + wv;
+    const bool live = tile < a.tiles;
     const bool want_model = (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const bool want_ops = (a.flags & MMSIM_WANT_OP_COUNT) != 0;
 
-    double *clk = lds_clk + lane;  // clk[slot * 64]
+    // ---- LDS: [latency table][per wavefront: request block | replica bounds | group descriptors | clocks | group counters]
+    float *lat_lds = reinterpret_cast<float *>(lds_raw);
+    const int lat_floats = LATLDS ? a.M * a.lat_row : 0;
+    const int lat_bytes = (lat_floats * 4 + 15) & ~15;
+    unsigned char *mine = lds_raw + lat_bytes + wv * a.wave_lds_bytes;
+    Req *stage = reinterpret_cast<Req *>(mine);
+    int4 *stage4 = reinterpret_cast<int4 *>(mine);
+    uint8_t *rmax_lds = mine + kStageBytes;
+    uint32_t *ginfo = reinterpret_cast<uint32_t *>(mine + kStageBytes + a.rmax_lds_bytes) + lane;
+    const int ginfo_bytes = (a.Gmax + 1) * kWave * 4;
+    double *clk = reinterpret_cast<double *>(mine + kStageBytes + a.rmax_lds_bytes + ginfo_bytes) + lane;
+    uint32_t *gcnt =
+        reinterpret_cast<uint32_t *>(mine + kStageBytes + a.rmax_lds_bytes + ginfo_bytes + a.nslots * (kWave * 8)) + lane;
+
+    for (int i = (int)threadIdx.x; i < lat_floats; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
+    if (live) {
+        for (int i = lane; i < a.M; i += kWave) rmax_lds[i] = a.rmax[(size_t)tile * a.M + i];
+        const uint32_t *gsrc = a.ginfo + (size_t)tile * (a.Gmax + 1) * kWave + lane;
+        for (int g = 0; g <= a.Gmax; ++g) ginfo[g * kWave] = gsrc[g * kWave];
+    }
+    __syncthreads();
+    if (!live) return;  // padding wavefront of the last workgroup
+
     for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
-    uint32_t *gcnt = reinterpret_cast<uint32_t *>(lds_clk + (size_t)a.nslots * kWave) + lane;
     if (want_group)
         for (int g = 0; g < 2 * a.Gmax; ++g) gcnt[g * kWave] = 0u;
 
+    const int wave = seed * a.tiles + tile;
     const int64_t off = a.stream_off[seed];
     const int64_t R = a.stream_off[seed + 1] - off;
-    const Req *__restrict__ reqs = a.streams + off;
-    const uint32_t *__restrict__ rep_tile = a.rep + (size_t)tile * a.M * RMAX * kWave + lane;
-    const int32_t *__restrict__ rmax_tile = a.rmax + (size_t)tile * a.M;
-    const float *__restrict__ lat = a.lat;
+    const int4 *__restrict__ reqs4 = reinterpret_cast<const int4 *>(a.streams + off);
+    const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * a.M * kWave + lane;
+    const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * a.M * a.rep_extra * kWave + lane;
     int32_t *model_good = a.model_good + (size_t)wave * a.M * kWave + lane;
     double *fin_out = a.finish + (size_t)wave * a.Rmax * kWave + lane;
     uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + lane;
+    const double overhead = a.fixed_overhead;
 
     int32_t n_good = 0;
     double lat_sum = 0.0;
     int64_t fp_ops = 0;
 
-    constexpr int CH = ChunkFor<RMAX>::value;
+    int4 ahead = make_int4(0, 0, -1, 0);  // this lane's request of the next block
+    if (R > 0) ahead = reqs4[lane < R ? lane : R - 1];
 
-    for (int64_t base = 0; base < R; base += CH) {
-        Req rq[CH];
-        int32_t nrep[CH];
-        uint32_t desc[CH][RMAX];
-#pragma unroll
-        for (int u = 0; u < CH; ++u) {
-            const int64_t i = base + u < R ? base + u : R - 1;
-            rq[u] = reqs[i];
+    for (int64_t blk = 0; blk < R; blk += kWave) {
+        stage4[lane] = ahead;
+        {
+            const int64_t nx = blk + kWave + lane;
+            ahead = reqs4[nx < R ? nx : R - 1];
         }
-#pragma unroll
-        for (int u = 0; u < CH; ++u) {
-            const bool live = base + u < R && rq[u].m >= 0;
-            nrep[u] = live ? rmax_tile[rq[u].m] : 0;
-        }
-#pragma unroll
-        for (int u = 0; u < CH; ++u) {
-            const uint32_t *row = rep_tile + (size_t)(rq[u].m < 0 ? 0 : rq[u].m) * RMAX * kWave;
-#pragma unroll
-            for (int j = 0; j < RMAX; ++j) desc[u][j] = j < nrep[u] ? row[j * kWave] : kEmpty;
-        }
+        const int nblk = (int)(R - blk < kWave ? R - blk : kWave);  // requests in this block
 
-#pragma unroll
-        for (int u = 0; u < CH; ++u) {
-            if (base + u >= R) break;
-            const double tstamp = rq[u].t;
-            const int32_t m = rq[u].m;
-            const double slo = (double)rq[u].slo;
+        // Always CH loads per chunk, whatever the requests are.
+        auto load_chunk = [&](Chunk &c, int cb) {
+            static_while<0, CH>([&](auto U) {
+                constexpr int u = decltype(U)::value;
+                const int idx = cb + u;  // < 64
+                const int m = uniform(stage[idx].m);
+                const bool ok = idx < nblk && m >= 0;
+                c.m[u] = m;
+                c.nrep[u] = ok ? uniform((int)rmax_lds[ok ? m : 0]) : 0;
+                c.g8[u] = rep_tile[(size_t)(ok ? m : 0) * kWave];
+                return true;
+            });
+        };
 
-            // ---- choose the replica group: strictly smallest last-stage clock (:590-598)
-            double best = 1e100;
-            uint32_t sel = kEmpty;
-            int nvalid = 0;
-#pragma unroll
-            for (int j = 0; j < RMAX; ++j) {
-                if (j >= nrep[u]) break;  // wave-uniform
-                const uint32_t d = desc[u][j];
-                const bool valid = d != kEmpty;
-                nvalid += valid ? 1 : 0;
-                const uint32_t last = valid ? desc_slot0(d) + desc_stages(d) - 1u : 0u;
-                const double c = clk[last * kWave];
-                const bool better = valid && c < best;
-                best = better ? c : best;
-                sel = better ? d : sel;
-            }
-            const bool has = sel != kEmpty;
-            const int S = has ? (int)desc_stages(sel) : 0;
-            const uint32_t slot0 = has ? desc_slot0(sel) : 0u;
-            const float *lrow = lat + ((size_t)(m < 0 ? 0 : m) * a.C + (has ? desc_cfg(sel) : 0u)) * a.lat_stride;
-            double *gclk = clk + slot0 * kWave;
+        Chunk cur, nxt;
+        load_chunk(cur, 0);
+        for (int cb = 0; cb < nblk; cb += CH) {
+            const bool more = cb + CH < nblk;
+            load_chunk(nxt, more ? cb + CH : cb);
 
-            // ---- walk the pipeline stages (:605-608)
-            double t = tstamp;
-            double tmp[SMAX];
-            int kdone = 0;  // wave-uniform: stages walked by the deepest lane
-#pragma unroll
-            for (int k = 0; k < SMAX; ++k) {
-                const bool active = k < S;
-                if (__ballot(active) == 0ull) break;
-                kdone = k + 1;
-                if (active) {
-                    const double c = gclk[k * kWave];
-                    const double l = (double)lrow[k];
-                    t = (c > t ? c : t) + l;
-                    tmp[k] = t;
+            static_while<0, CH>([&](auto U) {
+                constexpr int u = decltype(U)::value;
+                if (cb + u >= nblk) return false;
+                const Req r = stage[cb + u];  // broadcast read
+                const double tstamp = r.t;
+                const double slo = (double)r.slo;
+                const int m = cur.m[u];
+                const int n = cur.nrep[u];
+                const uint32_t glo = (uint32_t)cur.g8[u], ghi = (uint32_t)(cur.g8[u] >> 32);
+
+                // ---- choose the replica group: strictly smallest last-stage clock (:590-598)
+                double best = 1e100;
+                uint32_t sel = kEmpty;
+                int nvalid = 0;
+                auto consider = [&](uint32_t d, double c) {
+                    const bool valid = (int32_t)d >= 0;
+                    const bool better = valid && c < best;
+                    best = better ? c : best;
+                    sel = better ? d : sel;
+                    if (want_ops) nvalid += valid ? 1 : 0;
+                };
+                // Scan 4 or 8 list entries without branching: entries past a lane's own
+                // replicas name the empty descriptor row, whose clock read is ignored.
+                auto scan = [&](auto NJ) {
+                    constexpr int nj = decltype(NJ)::value;
+                    uint32_t info[nj];
+                    double cl[nj];
+                    static_while<0, nj>([&](auto J) {
+                        constexpr int j = decltype(J)::value;
+                        const uint32_t g = ((j < 4 ? glo : ghi) >> (8 * (j & 3))) & 0xFFu;
+                        info[j] = ginfo[g * kWave];
+                        return true;
+                    });
+                    static_while<0, nj>([&](auto J) {
+                        constexpr int j = decltype(J)::value;
+                        cl[j] = clk[desc_last_slot(info[j]) * kWave];
+                        return true;
+                    });
+                    static_while<0, nj>([&](auto J) {
+                        constexpr int j = decltype(J)::value;
+                        consider(info[j], cl[j]);
+                        return true;
+                    });
+                };
+                if (n > 4)
+                    scan(Idx<8>{});
+                else if (n > 0)
+                    scan(Idx<4>{});
+                if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
+                    const uint8_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
+                    for (int j = RREG; j < n; ++j) {
+                        const uint32_t d = ginfo[(uint32_t)row[(size_t)(j - RREG) * kWave] * kWave];
+                        consider(d, clk[desc_last_slot(d) * kWave]);
+                    }
                 }
-            }
-            const double finish_time = t + a.fixed_overhead;  // :610
-            const double latency = finish_time - tstamp;
-            const bool acc = has && latency <= slo;  // :613
 
-            if (acc) {  // :614-619
-                n_good += 1;
-                lat_sum += latency;
-            }
-#pragma unroll
-            for (int k = 0; k < SMAX; ++k) {
-                if (k >= kdone) break;
-                if (acc && k < S) gclk[k * kWave] = tmp[k];
-            }
-            if (want_group && has) {  // :611, :618
-                const uint32_t g = desc_group(sel);
-                gcnt[g * kWave] += 1u;
-                if (acc) gcnt[(a.Gmax + g) * kWave] += 1u;
-            }
-            if (want_ops && has) fp_ops += 2 * S + nvalid + 3;
-            if (want_model && m >= 0) model_good[(size_t)m * kWave] += acc ? 1 : 0;
-            if (want_req) {
-                fin_out[(base + u) * kWave] = acc ? finish_time : tstamp;
-                good_out[(base + u) * kWave] = acc ? 1 : 0;
-            }
+                const bool has = (int32_t)sel >= 0;
+                const int sm1 = has ? (int)desc_stages_m1(sel) : -1;  // stages - 1
+                const uint32_t slot0 = has ? desc_last_slot(sel) - (uint32_t)sm1 : 0u;
+                double *gclk = clk + slot0 * kWave;
+                const uint32_t lidx = (uint32_t)(m < 0 ? 0 : m) * (uint32_t)a.lat_row + (has ? desc_lat_off(sel) : 0u);
+                const float *lrow = (LATLDS ? lat_lds : a.lat) + lidx;
+
+                // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
+                int walk = -1;  // stages - 1 of lanes that walk
+                double l_const = 0.0;
+                if (has) {
+                    const double l_last = (double)lrow[UNIFORM ? 0 : sm1];
+                    l_const = l_last;
+                    const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
+                    walk = bound > slo ? -1 : sm1;
+                }
+
+                double finish_time;
+                bool acc;
+                if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
+                    // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
+                    uint64_t saved_exec;
+                    int accepted;
+                    double t, latency;
+                    const uint32_t cb = lds_addr(gclk);
+                    if constexpr (UNIFORM) {
+                        if constexpr (SMAX == 4)
+                            asm volatile(MMSIM_WALK_U4_TEXT
+                                         : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t), [fin] "=&v"(finish_time),
+                                           [lat] "=&v"(latency), [ng] "+v"(n_good), [ls] "+v"(lat_sum)
+                                         : [walk] "v"(walk), [cb] "v"(cb), [lc] "v"(l_const), [ts] "v"(tstamp), [slo] "v"(slo),
+                                           [oh] "s"(overhead)
+                                         : "vcc", "memory", MMSIM_WALK_U4_CLOBBERS);
+                        else
+                            asm volatile(MMSIM_WALK_U16_TEXT
+                                         : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t), [fin] "=&v"(finish_time),
+                                           [lat] "=&v"(latency), [ng] "+v"(n_good), [ls] "+v"(lat_sum)
+                                         : [walk] "v"(walk), [cb] "v"(cb), [lc] "v"(l_const), [ts] "v"(tstamp), [slo] "v"(slo),
+                                           [oh] "s"(overhead)
+                                         : "vcc", "memory", MMSIM_WALK_U16_CLOBBERS);
+                    } else {
+                        const uint32_t lb = lds_addr(lrow);
+                        if constexpr (SMAX == 4)
+                            asm volatile(MMSIM_WALK_N4_TEXT
+                                         : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t), [fin] "=&v"(finish_time),
+                                           [lat] "=&v"(latency), [ng] "+v"(n_good), [ls] "+v"(lat_sum)
+                                         : [walk] "v"(walk), [cb] "v"(cb), [lb] "v"(lb), [ts] "v"(tstamp), [slo] "v"(slo),
+                                           [oh] "s"(overhead)
+                                         : "vcc", "memory", MMSIM_WALK_N4_CLOBBERS);
+                        else
+                            asm volatile(MMSIM_WALK_N16_TEXT
+                                         : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t), [fin] "=&v"(finish_time),
+                                           [lat] "=&v"(latency), [ng] "+v"(n_good), [ls] "+v"(lat_sum)
+                                         : [walk] "v"(walk), [cb] "v"(cb), [lb] "v"(lb), [ts] "v"(tstamp), [slo] "v"(slo),
+                                           [oh] "s"(overhead)
+                                         : "vcc", "memory", MMSIM_WALK_N16_CLOBBERS);
+                    }
+                    acc = accepted != 0;
+                } else {
+                    // ---- the same in plain C++ (other stage buckets, latency table in global memory):
+                    //      fetch, then the dependent chain (:605-608)
+                    double cv[SMAX];
+                    float lv[SMAX];
+                    walk_blocks<0, 1, SMAX>(
+                        [&](auto K) { return decltype(K)::value <= walk; },
+                        [&](auto K) {
+                            constexpr int k = decltype(K)::value;
+                            cv[k] = gclk[k * kWave];
+                            if (!UNIFORM) lv[k] = lrow[k];
+                        });
+                    double t = tstamp;
+                    walk_blocks<0, 1, SMAX>(
+                        [&](auto K) { return decltype(K)::value <= walk; },
+                        [&](auto K) {
+                            constexpr int k = decltype(K)::value;
+                            t = vmax(t, cv[k]) + (UNIFORM ? l_const : (double)lv[k]);
+                            cv[k] = t;
+                        });
+                    finish_time = t + overhead;  // :610
+                    const double latency = finish_time - tstamp;
+                    acc = walk >= 0 && latency <= slo;  // :613
+                    if (acc) {  // :614-619
+                        n_good += 1;
+                        lat_sum += latency;
+                    }
+                    const int commit = acc ? walk : -1;
+                    walk_blocks<0, 1, SMAX>(
+                        [&](auto K) { return decltype(K)::value <= commit; },
+                        [&](auto K) {
+                            constexpr int k = decltype(K)::value;
+                            gclk[k * kWave] = cv[k];
+                        });
+                }
+                if (want_group && has) {  // :611, :618
+                    const uint32_t g = desc_group(sel);
+                    gcnt[g * kWave] += 1u;
+                    if (acc) gcnt[(a.Gmax + g) * kWave] += 1u;
+                }
+                if (want_ops && has) fp_ops += 2 * (sm1 + 1) + nvalid + 3;
+                if (want_model && m >= 0) model_good[(size_t)m * kWave] += acc ? 1 : 0;
+                if (want_req) {
+                    fin_out[(blk + cb + u) * kWave] = acc ? finish_time : tstamp;
+                    good_out[(blk + cb + u) * kWave] = acc ? 1 : 0;
+                }
+                return true;
+            });
+            cur = nxt;
         }
     }
 
@@ -183,56 +390,50 @@ __global__ __launch_bounds__(kWave) void sim_mixed_kernel(const MixedArgs a) {
     }
 }
 
-template <int SMAX, int RMAX>
-hipError_t launch_one(const MixedArgs &args, size_t lds_bytes, hipStream_t stream) {
-    auto kern = sim_mixed_kernel<SMAX, RMAX>;
+template <int SMAX, bool LATLDS, bool UNIFORM>
+hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
+    auto kern = sim_mixed_kernel<SMAX, LATLDS, UNIFORM>;
     if (lds_bytes > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return e;
     }
-    const dim3 grid((unsigned)(args.tiles * args.n_seeds));
-    hipLaunchKernelGGL(kern, grid, dim3(kWave), lds_bytes, stream, args);
+    const unsigned tile_groups = (unsigned)((args.tiles + wpb - 1) / wpb);
+    const dim3 grid(tile_groups * (unsigned)args.n_seeds);
+    hipLaunchKernelGGL(kern, grid, dim3(wpb * kWave), lds_bytes, stream, args);
     return hipGetLastError();
 }
 
 template <int SMAX>
-hipError_t launch_r(const MixedArgs &args, int rb, size_t lds_bytes, hipStream_t stream) {
-    switch (rb) {
-        case 1: return launch_one<SMAX, 1>(args, lds_bytes, stream);
-        case 2: return launch_one<SMAX, 2>(args, lds_bytes, stream);
-        case 4: return launch_one<SMAX, 4>(args, lds_bytes, stream);
-        case 8: return launch_one<SMAX, 8>(args, lds_bytes, stream);
-        case 16: return launch_one<SMAX, 16>(args, lds_bytes, stream);
-        case 64: return launch_one<SMAX, 64>(args, lds_bytes, stream);
-        default: return hipErrorInvalidValue;
-    }
+hipError_t launch_s(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
+    if (args.lat_in_lds)
+        return args.uniform_stages ? launch_one<SMAX, true, true>(args, wpb, lds_bytes, stream)
+                                   : launch_one<SMAX, true, false>(args, wpb, lds_bytes, stream);
+    return args.uniform_stages ? launch_one<SMAX, false, true>(args, wpb, lds_bytes, stream)
+                               : launch_one<SMAX, false, false>(args, wpb, lds_bytes, stream);
 }
 
 }  // namespace
 
 int smax_bucket_for(int smax) {
-    for (int b : {1, 4, 8, 16, 32})
+    for (int b : {1, 4, 16, 32})
         if (smax <= b) return b;
     return -1;
 }
 
-int rmax_bucket_for(int rmax) {
-    for (int b : {1, 2, 4, 8, 16, 64})
-        if (rmax <= b) return b;
-    return -1;
-}
-
-hipError_t launch_sim_mixed(const MixedArgs &args, int sb, int rb, size_t lds_bytes, hipStream_t stream,
+hipError_t launch_sim_mixed(const MixedArgs &args, int sb, int wpb, size_t lds_bytes, hipStream_t stream,
                             std::string *err) {
     hipError_t e;
-    switch (sb) {
-        case 1: e = launch_r<1>(args, rb, lds_bytes, stream); break;
-        case 4: e = launch_r<4>(args, rb, lds_bytes, stream); break;
-        case 8: e = launch_r<8>(args, rb, lds_bytes, stream); break;
-        case 16: e = launch_r<16>(args, rb, lds_bytes, stream); break;
-        case 32: e = launch_r<32>(args, rb, lds_bytes, stream); break;
-        default: e = hipErrorInvalidValue; break;
+    if (wpb < 1 || wpb > kMaxWavesPerBlock) {
+        e = hipErrorInvalidValue;
+    } else {
+        switch (sb) {
+            case 1: e = launch_s<1>(args, wpb, lds_bytes, stream); break;
+            case 4: e = launch_s<4>(args, wpb, lds_bytes, stream); break;
+            case 16: e = launch_s<16>(args, wpb, lds_bytes, stream); break;
+            case 32: e = launch_s<32>(args, wpb, lds_bytes, stream); break;
+            default: e = hipErrorInvalidValue; break;
+        }
     }
     if (e != hipSuccess && err) *err = std::string("sim_mixed launch: ") + hipGetErrorString(e);
     return e;
