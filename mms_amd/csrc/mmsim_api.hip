@@ -73,6 +73,11 @@ struct mmsim_workload {
     int32_t M = 0;
     DevBuf<Req> reqs;
     std::vector<int32_t> model_num_requests;  // requests per model id (placement independent)
+    // arrivals regrouped by model (batching simulator): offsets per model, then per arrival
+    // its time, its deadline time + (double)slo and its index in the stream
+    std::vector<int64_t> mq_off;
+    DevBuf<double> mq_t, mq_dl;
+    DevBuf<int32_t> mq_idx;
 };
 
 // Ordered replica lists per (placement, model): the rows of m_id2g_id.
@@ -82,6 +87,10 @@ struct RepLists {
     std::vector<int32_t> group_cfg;   // [B][Gmax]
     std::vector<int64_t> off;         // [B*M+1]
     std::vector<int32_t> grp;         // group index per replica
+    // models of each group in the order the batching simulator scans them (g_id2m_id);
+    // left empty, they are derived from the replica lists as the reference does (:424-430)
+    std::vector<int64_t> g2m_off;     // [B*Gmax+1]
+    std::vector<int32_t> g2m_m;
 };
 
 struct mmsim_batch {
@@ -107,6 +116,14 @@ struct mmsim_batch {
     DevBuf<double> finish;
     DevBuf<uint8_t> good;
     DevBuf<int64_t> fp_ops;
+    // batching simulator
+    DevBuf<int64_t> mq_off;
+    DevBuf<double> mq_t, mq_dl;
+    DevBuf<int32_t> mq_idx, status, batch_sizes;
+    DevBuf<uint16_t> g2m_off, g2m_idx;
+    DevBuf<float> lat_nb;
+    std::vector<uint8_t> hosted;  // [B][M] model has a replica (batching: decides model_num_requests)
+    BatchingArgs bargs{};
 
     MixedArgs args{};
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
@@ -175,7 +192,18 @@ int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLi
 // Builds every device table of a batch from replica lists and launches nothing.
 int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seeds, const mmsim_tables *t,
                 const RepLists &rl, uint32_t flags, mmsim_batch **out) {
-    if (flags & MMSIM_BATCHING) return fail(MMSIM_E_UNSUPPORTED, "batching simulator is not available in this build");
+    const bool batching = (flags & MMSIM_BATCHING) != 0;
+    if (batching && (flags & MMSIM_WANT_OP_COUNT)) return fail(MMSIM_E_UNSUPPORTED, "operation counts are only available for the plain simulator");
+    if (batching) {
+        if (!t->batch_sizes || t->batch_sizes[0] != 1) return fail(MMSIM_E_INVALID, "tables: batch_sizes[0] must be 1");
+        for (int b = 0; b < t->NB; ++b) {
+            if (t->batch_sizes[b] < 1) return fail(MMSIM_E_INVALID, "tables: batch size < 1");
+            int col = 0;
+            for (int v = t->batch_sizes[b]; v > 1; v >>= 1) ++col;
+            if (col >= t->NB) return fail(MMSIM_E_INVALID, "tables: floor(log2(batch size)) must index a latency column");
+        }
+        if (t->M > 65535) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: more than 65535 models");
+    }
     const int32_t M = t->M, C = t->C, B = rl.B, Gmax = rl.Gmax;
     if (n_seeds < 1 || !wls) return fail(MMSIM_E_INVALID, "need at least one workload");
     for (int s = 0; s < n_seeds; ++s) {
@@ -222,7 +250,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     //      latencies for configuration 0, then configuration 1, ... (the cfg_pp[c] real
     //      stages only).  When every (model, config) has one latency for all its stages the
     //      row is just one value per configuration.
-    bool uniform_stages = true;
+    bool uniform_stages = !batching;  // the batching kernel reads per-stage, per-batch-size latencies
     for (int32_t m = 0; m < M && uniform_stages; ++m)
         for (int c = 0; c < C && uniform_stages; ++c) {
             const float *row = t->cfg_lat + ((size_t)m * C + c) * t->Smax * t->NB;
@@ -243,23 +271,42 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 lat[(size_t)m * lat_row + lat_off[c] + k] = v;
             }
 
-    // ---- LDS budget: shared latency table + per-wavefront private region
+    // ---- LDS budget
     const int32_t rmax_lds_bytes = (M + 15) & ~15;
-    const size_t wave_bytes = ((size_t)kStageBytes + rmax_lds_bytes + (size_t)(Gmax + 1) * kWave * sizeof(uint32_t) +
-                               (size_t)nslots * kWave * sizeof(double) +
-                               ((flags & MMSIM_WANT_GROUP_COUNTS) ? (size_t)2 * Gmax * kWave * sizeof(uint32_t) : 0) + 15) & ~(size_t)15;
-    const size_t lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
+    size_t wave_bytes = 0;
     int lat_in_lds = 1;
     int wpb = 0;
-    if (lat_bytes + wave_bytes <= (size_t)ctx->max_lds) wpb = (int)std::min<size_t>(kMaxWavesPerBlock, ((size_t)ctx->max_lds - lat_bytes) / wave_bytes);
-    if (wpb == 0) {
-        lat_in_lds = 0;
+    int heap_cap = 0;
+    if (!batching) {
+        // shared latency table + per-wavefront private region
+        wave_bytes = ((size_t)kStageBytes + rmax_lds_bytes + (size_t)(Gmax + 1) * kWave * sizeof(uint32_t) +
+                      (size_t)nslots * kWave * sizeof(double) +
+                      ((flags & MMSIM_WANT_GROUP_COUNTS) ? (size_t)2 * Gmax * kWave * sizeof(uint32_t) : 0) + 15) & ~(size_t)15;
+        const size_t lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
+        if (lat_bytes + wave_bytes <= (size_t)ctx->max_lds)
+            wpb = (int)std::min<size_t>(kMaxWavesPerBlock, ((size_t)ctx->max_lds - lat_bytes) / wave_bytes);
+        if (wpb == 0) {
+            lat_in_lds = 0;
+            wpb = (int)std::min<size_t>(kMaxWavesPerBlock, (size_t)ctx->max_lds / wave_bytes);
+        }
+        if (wpb == 0) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
+        wpb = std::min(wpb, b->tiles);
+        b->lds_bytes = (lat_in_lds ? lat_bytes : 0) + (size_t)wpb * wave_bytes;
+    } else {
+        // per wavefront: descriptors | clocks | event times | queue heads | event groups | arrivals per model.
+        // Events: the reference's heap holds about one entry per group plus a few stale ones;
+        // provision 2*G+8 if that fits, never less than G+4.
+        const size_t fixed = (size_t)(Gmax + 1) * kWave * 4 + (size_t)nslots * kWave * 8 + (size_t)M * kWave * 4 + (size_t)M * 4 + 16;
+        for (heap_cap = 2 * Gmax + 8; heap_cap >= Gmax + 4; --heap_cap) {
+            wave_bytes = (fixed + (size_t)heap_cap * kWave * 12 + 15) & ~(size_t)15;
+            if (wave_bytes <= (size_t)ctx->max_lds) break;
+        }
+        if (heap_cap < Gmax + 4) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: per-wavefront state does not fit in LDS (too many models/stages/groups)");
         wpb = (int)std::min<size_t>(kMaxWavesPerBlock, (size_t)ctx->max_lds / wave_bytes);
+        wpb = std::min(wpb, b->tiles);
+        b->lds_bytes = (size_t)wpb * wave_bytes;
     }
-    if (wpb == 0) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
-    wpb = std::min(wpb, b->tiles);
     b->waves_per_block = wpb;
-    b->lds_bytes = (lat_in_lds ? lat_bytes : 0) + (size_t)wpb * wave_bytes;
 
     // ---- lane assignment.  A wavefront walks as many pipeline stages as its deepest
     //      lane needs, so placements are ordered by depth before they are cut into
@@ -332,6 +379,60 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
     }
 
+    // ---- batching simulator: models of each group, full latency table, which models a lane hosts
+    std::vector<uint16_t> g2m_off, g2m_idx;
+    std::vector<float> lat_nb;
+    int members_max = 1;
+    if (batching) {
+        b->hosted.assign((size_t)B * M, 0);
+        std::vector<std::vector<int32_t>> lists(Gmax);
+        std::vector<std::vector<int32_t>> all((size_t)B * Gmax);
+        for (int32_t p = 0; p < B; ++p) {
+            size_t total = 0;
+            for (int32_t g = 0; g < rl.num_groups[p]; ++g) {
+                std::vector<int32_t> &dst = all[(size_t)p * Gmax + g];
+                if (!rl.g2m_off.empty())
+                    dst.assign(rl.g2m_m.begin() + rl.g2m_off[(size_t)p * Gmax + g], rl.g2m_m.begin() + rl.g2m_off[(size_t)p * Gmax + g + 1]);
+                total += dst.size();
+            }
+            for (int32_t m = 0; m < M; ++m) {
+                const int64_t lo = rl.off[(size_t)p * M + m], hi = rl.off[(size_t)p * M + m + 1];
+                b->hosted[(size_t)p * M + m] = hi > lo;
+                if (rl.g2m_off.empty())  // ascending model id within a group, as :424-430 builds it
+                    for (int64_t x = lo; x < hi; ++x) {
+                        all[(size_t)p * Gmax + rl.grp[(size_t)x]].push_back(m);
+                        ++total;
+                    }
+            }
+            if (total > 65535) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: more than 65535 (group, model) pairs in a placement");
+            members_max = std::max<int>(members_max, (int)total);
+        }
+        g2m_off.assign((size_t)b->tiles * (Gmax + 1) * kWave, 0);
+        g2m_idx.assign((size_t)b->tiles * members_max * kWave, 0);
+        for (int32_t p = 0; p < B; ++p) {
+            const int tile = b->pos[p] / kWave, lane = b->pos[p] % kWave;
+            uint16_t at = 0;
+            for (int32_t g = 0; g <= Gmax; ++g) {
+                g2m_off[((size_t)tile * (Gmax + 1) + g) * kWave + lane] = at;
+                if (g < rl.num_groups[p])
+                    for (int32_t m : all[(size_t)p * Gmax + g]) {
+                        if (m < 0 || m >= M) return fail(MMSIM_E_INVALID, "group model list names a model outside 0..M-1");
+                        g2m_idx[((size_t)tile * members_max + at) * kWave + lane] = (uint16_t)m;
+                        ++at;
+                    }
+            }
+        }
+        lat_nb.resize((size_t)M * lat_row * t->NB);
+        for (int32_t m = 0; m < M; ++m)
+            for (int c = 0; c < C; ++c)
+                for (int k = 0; k < t->cfg_pp[c]; ++k)
+                    for (int q = 0; q < t->NB; ++q) {
+                        const float v = t->cfg_lat[(((size_t)m * C + c) * t->Smax + k) * t->NB + q];
+                        if (v != v || v < 0.0f) return fail(MMSIM_E_INVALID, "tables: a stage latency is NaN or negative");
+                        lat_nb[((size_t)m * lat_row + lat_off[c] + k) * t->NB + q] = v;
+                    }
+    }
+
     // ---- request streams back to back
     std::vector<int64_t> soff(n_seeds + 1, 0);
     for (int s = 0; s < n_seeds; ++s) {
@@ -360,7 +461,39 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     HIP_TRY(b->lat.alloc(lat.size()));
     HIP_TRY(hipMemcpyAsync(b->lat.p, lat.data(), sizeof(float) * lat.size(), hipMemcpyHostToDevice, st));
 
+    if (batching) {
+        std::vector<int64_t> mqo((size_t)n_seeds * (M + 1));
+        int64_t total = 0;
+        for (int s = 0; s < n_seeds; ++s) {
+            for (int32_t m = 0; m <= M; ++m) mqo[(size_t)s * (M + 1) + m] = total + wls[s]->mq_off[m];
+            total += wls[s]->mq_off[M];
+        }
+        HIP_TRY(b->mq_t.alloc((size_t)total));
+        HIP_TRY(b->mq_dl.alloc((size_t)total));
+        HIP_TRY(b->mq_idx.alloc((size_t)total));
+        int64_t at = 0;
+        for (int s = 0; s < n_seeds; ++s) {
+            const size_t n = (size_t)wls[s]->mq_off[M];
+            if (n > 0) {
+                HIP_TRY(hipMemcpyAsync(b->mq_t.p + at, wls[s]->mq_t.p, sizeof(double) * n, hipMemcpyDeviceToDevice, st));
+                HIP_TRY(hipMemcpyAsync(b->mq_dl.p + at, wls[s]->mq_dl.p, sizeof(double) * n, hipMemcpyDeviceToDevice, st));
+                HIP_TRY(hipMemcpyAsync(b->mq_idx.p + at, wls[s]->mq_idx.p, sizeof(int32_t) * n, hipMemcpyDeviceToDevice, st));
+            }
+            at += (int64_t)n;
+        }
+        HIP_TRY(b->mq_off.alloc(mqo.size()));
+        HIP_TRY(hipMemcpyAsync(b->mq_off.p, mqo.data(), sizeof(int64_t) * mqo.size(), hipMemcpyHostToDevice, st));
+        HIP_TRY(b->g2m_off.alloc(g2m_off.size()));
+        HIP_TRY(hipMemcpyAsync(b->g2m_off.p, g2m_off.data(), sizeof(uint16_t) * g2m_off.size(), hipMemcpyHostToDevice, st));
+        HIP_TRY(b->g2m_idx.alloc(g2m_idx.size()));
+        HIP_TRY(hipMemcpyAsync(b->g2m_idx.p, g2m_idx.data(), sizeof(uint16_t) * g2m_idx.size(), hipMemcpyHostToDevice, st));
+        HIP_TRY(b->lat_nb.alloc(lat_nb.size()));
+        HIP_TRY(hipMemcpyAsync(b->lat_nb.p, lat_nb.data(), sizeof(float) * lat_nb.size(), hipMemcpyHostToDevice, st));
+        HIP_TRY(b->batch_sizes.alloc((size_t)t->NB));
+        HIP_TRY(hipMemcpyAsync(b->batch_sizes.p, t->batch_sizes, sizeof(int32_t) * (size_t)t->NB, hipMemcpyHostToDevice, st));
+    }
     const size_t lanes_padded = (size_t)b->waves * kWave;
+    HIP_TRY(b->status.alloc(lanes_padded));
     HIP_TRY(b->n_good.alloc(lanes_padded));
     HIP_TRY(b->lat_sum.alloc(lanes_padded));
     if (flags & MMSIM_WANT_MODEL_COUNTS) HIP_TRY(b->model_good.alloc(lanes_padded * M));
@@ -408,6 +541,45 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.finish = b->finish.p;
     a.good = b->good.p;
     a.fp_ops = b->fp_ops.p;
+    if (batching) {
+        BatchingArgs &q = b->bargs;
+        q.streams = b->streams.p;
+        q.stream_off = b->stream_off.p;
+        q.mq_off = b->mq_off.p;
+        q.mq_t = b->mq_t.p;
+        q.mq_dl = b->mq_dl.p;
+        q.mq_idx = b->mq_idx.p;
+        q.rep8 = b->rep8.p;
+        q.repx = b->repx.p;
+        q.ginfo = b->ginfo.p;
+        q.g2m_off = b->g2m_off.p;
+        q.g2m_idx = b->g2m_idx.p;
+        q.lat = b->lat_nb.p;
+        q.batch_sizes = b->batch_sizes.p;
+        q.M = M;
+        q.lat_row = lat_row;
+        q.NB = t->NB;
+        q.rep_extra = RX;
+        q.members_max = members_max;
+        q.heap_cap = heap_cap;
+        q.n_seeds = n_seeds;
+        q.B = B;
+        q.tiles = b->tiles;
+        q.nslots = nslots;
+        q.Gmax = Gmax;
+        q.wave_lds_bytes = (int32_t)wave_bytes;
+        q.Rmax = b->Rmax;
+        q.fixed_overhead = t->fixed_overhead;
+        q.flags = flags;
+        q.n_good = b->n_good.p;
+        q.lat_sum = b->lat_sum.p;
+        q.status = b->status.p;
+        q.model_good = b->model_good.p;
+        q.group_req = b->group_req.p;
+        q.group_good = b->group_good.p;
+        q.finish = b->finish.p;
+        q.good = b->good.p;
+    }
     *out = b.release();
     return MMSIM_OK;
 }
@@ -487,10 +659,34 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
         host[i].slo = slos[i];
         if (model_ids[i] >= 0) w->model_num_requests[model_ids[i]] += 1;
     }
+    w->mq_off.assign((size_t)M + 1, 0);
+    for (int32_t m = 0; m < M; ++m) w->mq_off[m + 1] = w->mq_off[m] + w->model_num_requests[m];
+    const size_t known = (size_t)w->mq_off[M];
+    std::vector<double> mq_t(known), mq_dl(known);
+    std::vector<int32_t> mq_idx(known);
+    {
+        std::vector<int64_t> fill(w->mq_off.begin(), w->mq_off.end() - 1);
+        for (int64_t i = 0; i < R; ++i)
+            if (model_ids[i] >= 0) {
+                const size_t q = (size_t)fill[model_ids[i]]++;
+                mq_t[q] = tstamps[i];
+                mq_dl[q] = tstamps[i] + (double)slos[i];  // controller.py:679
+                mq_idx[q] = (int32_t)i;
+            }
+    }
+    if (R > 0x7FFFFFFF) return fail(MMSIM_E_UNSUPPORTED, "workload_create: more than 2^31-1 requests");
     HIP_TRY(hipSetDevice(ctx->device));
     HIP_TRY(w->reqs.alloc((size_t)R));
+    HIP_TRY(w->mq_t.alloc(known));
+    HIP_TRY(w->mq_dl.alloc(known));
+    HIP_TRY(w->mq_idx.alloc(known));
     if (R > 0) {
         HIP_TRY(hipMemcpyAsync(w->reqs.p, host.data(), sizeof(Req) * (size_t)R, hipMemcpyHostToDevice, ctx->stream));
+        if (known > 0) {
+            HIP_TRY(hipMemcpyAsync(w->mq_t.p, mq_t.data(), sizeof(double) * known, hipMemcpyHostToDevice, ctx->stream));
+            HIP_TRY(hipMemcpyAsync(w->mq_dl.p, mq_dl.data(), sizeof(double) * known, hipMemcpyHostToDevice, ctx->stream));
+            HIP_TRY(hipMemcpyAsync(w->mq_idx.p, mq_idx.data(), sizeof(int32_t) * known, hipMemcpyHostToDevice, ctx->stream));
+        }
         HIP_TRY(hipStreamSynchronize(ctx->stream));
     }
     *out = w.release();
@@ -522,9 +718,15 @@ int mmsim_batch_run(mmsim_batch *b) {
     HIP_TRY(hipSetDevice(ctx->device));
     if (b->flags & MMSIM_WANT_MODEL_COUNTS)
         HIP_TRY(hipMemsetAsync(b->model_good.p, 0, b->model_good.bytes(), ctx->stream));
+    if ((b->flags & MMSIM_BATCHING) && (b->flags & MMSIM_WANT_GROUP_COUNTS)) {
+        HIP_TRY(hipMemsetAsync(b->group_req.p, 0, b->group_req.bytes(), ctx->stream));
+        HIP_TRY(hipMemsetAsync(b->group_good.p, 0, b->group_good.bytes(), ctx->stream));
+    }
     HIP_TRY(hipEventRecord(b->ev_start, ctx->stream));
     std::string err;
-    hipError_t e = launch_sim_mixed(b->args, b->smax_bucket, b->waves_per_block, b->lds_bytes, ctx->stream, &err);
+    hipError_t e = (b->flags & MMSIM_BATCHING)
+                       ? launch_sim_batching(b->bargs, b->waves_per_block, b->lds_bytes, ctx->stream, &err)
+                       : launch_sim_mixed(b->args, b->smax_bucket, b->waves_per_block, b->lds_bytes, ctx->stream, &err);
     if (e != hipSuccess) return fail(MMSIM_E_HIP, err);
     HIP_TRY(hipEventRecord(b->ev_stop, ctx->stream));
     b->ran = true;
@@ -558,6 +760,12 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
     std::vector<double> ls(lanes_padded);
     HIP_TRY(hipMemcpy(ng.data(), b->n_good.p, sizeof(int32_t) * lanes_padded, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(ls.data(), b->lat_sum.p, sizeof(double) * lanes_padded, hipMemcpyDeviceToHost));
+    std::vector<int32_t> st_host;
+    int any_bad = 0;
+    if (b->flags & MMSIM_BATCHING) {
+        st_host.resize(lanes_padded);
+        HIP_TRY(hipMemcpy(st_host.data(), b->status.p, sizeof(int32_t) * lanes_padded, hipMemcpyDeviceToHost));
+    }
     std::vector<int64_t> ops;
     if (b->flags & MMSIM_WANT_OP_COUNT) {
         if (!out->fp_ops) return fail(MMSIM_E_INVALID, "batch_fetch: fp_ops array missing");
@@ -569,7 +777,8 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
             const size_t src = (size_t)s * tiles * kWave + b->pos[p];
             out->n_good[(size_t)s * B + p] = ng[src];
             out->latency_sum[(size_t)s * B + p] = ls[src];
-            if (out->status) out->status[(size_t)s * B + p] = 0;
+            if (out->status) out->status[(size_t)s * B + p] = st_host.empty() ? 0 : st_host[src];
+            if (!st_host.empty() && st_host[src] != 0) any_bad = st_host[src];
             if (!ops.empty()) out->fp_ops[(size_t)s * B + p] = ops[src];
         }
     // device rows are [wave][x][64] with wave = seed*tiles + tile; lane l of a seed is placement l
@@ -589,8 +798,9 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
         if (rc) return rc;
         for (int s = 0; s < b->n_seeds; ++s)
             for (int32_t p = 0; p < B; ++p)
-                std::memcpy(out->model_num_requests + ((size_t)s * B + p) * M, b->wl[s]->model_num_requests.data(),
-                            sizeof(int32_t) * (size_t)M);
+                for (int32_t m = 0; m < M; ++m)  // the batching loop only counts requests of hosted models (:754-757, :773)
+                    out->model_num_requests[((size_t)s * B + p) * M + m] =
+                        (b->hosted.empty() || b->hosted[(size_t)p * M + m]) ? b->wl[s]->model_num_requests[m] : 0;
     }
     if (wg) {
         int rc = unpack_i32(b->group_req, Gmax, out->group_num_requests);
@@ -621,6 +831,10 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
                 }
             }
     }
+    if (any_bad && !out->status)
+        return fail(any_bad, any_bad == MMSIM_E_OVERFLOW
+                                 ? "a simulation ran out of idle-event slots; its results are invalid (pass status[] to see which)"
+                                 : "a simulation hit an input the batching simulator does not support (all replica clocks infinite)");
     return MMSIM_OK;
 }
 
@@ -732,11 +946,86 @@ int mmsim_simulate_requests_mixed(mmsim_ctx *ctx, double *finish, uint8_t *good,
     return rc;
 }
 
-int mmsim_simulate_requests_mixed_batching(mmsim_ctx *, double *, uint8_t *, const double *, const int32_t *,
-                                           const float *, const int32_t *, const int32_t *, const int32_t *,
-                                           const float *, const int32_t *, int64_t, int32_t, int32_t, int32_t, int32_t,
-                                           double, int32_t *, int32_t *, int32_t *, int32_t *) {
-    return fail(MMSIM_E_UNSUPPORTED, "batching simulator is not available in this build");
+int mmsim_simulate_requests_mixed_batching(mmsim_ctx *ctx, double *finish, uint8_t *good, const double *tstamps,
+                                           const int32_t *model_ids, const float *slos, const int32_t *m_id2g_id,
+                                           const int32_t *g_id2m_id, const int32_t *num_stages,
+                                           const float *stage_latency, const int32_t *batch_sizes, int64_t num_requests,
+                                           int32_t M, int32_t G, int32_t Smax, int32_t NB, double fixed_overhead,
+                                           int32_t *model_num_requests, int32_t *model_num_good_requests,
+                                           int32_t *group_num_requests, int32_t *group_num_good_requests) {
+    if (!ctx) return fail(MMSIM_E_INVALID, "simulate_requests_mixed_batching: null context");
+    if (M < 1 || G < 1 || Smax < 1 || NB < 1 || num_requests < 0)
+        return fail(MMSIM_E_INVALID, "simulate_requests_mixed_batching: bad size");
+    if (!m_id2g_id || !g_id2m_id || !num_stages || !stage_latency || !batch_sizes || !model_num_requests ||
+        !model_num_good_requests || !group_num_requests || !group_num_good_requests ||
+        (num_requests > 0 && (!finish || !good)))
+        return fail(MMSIM_E_INVALID, "simulate_requests_mixed_batching: null pointer");
+    if (G > MMSIM_MAX_GROUPS) return fail(MMSIM_E_UNSUPPORTED, "simulate_requests_mixed_batching: more than 254 groups");
+    mmsim_tables t{};
+    t.M = M;
+    t.C = G;  // every group is its own latency-table column
+    t.Smax = Smax;
+    t.NB = NB;
+    t.cfg_lat = stage_latency;
+    t.cfg_pp = num_stages;
+    t.batch_sizes = batch_sizes;
+    t.fixed_overhead = fixed_overhead;
+    int rc = check_tables(&t);
+    if (rc) return rc;
+    RepLists rl;
+    rl.B = 1;
+    rl.M = M;
+    rl.Gmax = G;
+    rl.num_groups.assign(1, G);
+    rl.group_cfg.resize(G);
+    for (int g = 0; g < G; ++g) rl.group_cfg[g] = g;
+    rl.off.assign((size_t)M + 1, 0);
+    for (int32_t m = 0; m < M; ++m)
+        for (int32_t j = 0; j < G; ++j) {
+            const int32_t g = m_id2g_id[(size_t)m * G + j];
+            if (g < 0) break;
+            if (g >= G) return fail(MMSIM_E_INVALID, "simulate_requests_mixed_batching: m_id2g_id names a group >= G");
+            rl.grp.push_back(g);
+            rl.off[m + 1] += 1;
+        }
+    for (int32_t m = 0; m < M; ++m) rl.off[m + 1] += rl.off[m];
+    rl.g2m_off.assign((size_t)G + 1, 0);
+    for (int32_t g = 0; g < G; ++g) {
+        for (int32_t j = 0; j < M; ++j) {
+            const int32_t m = g_id2m_id[(size_t)g * M + j];
+            if (m < 0) break;
+            if (m >= M) return fail(MMSIM_E_INVALID, "simulate_requests_mixed_batching: g_id2m_id names a model >= M");
+            rl.g2m_m.push_back(m);
+        }
+        rl.g2m_off[g + 1] = (int64_t)rl.g2m_m.size();
+    }
+
+    mmsim_workload *wl = nullptr;
+    rc = mmsim_workload_create(ctx, num_requests, M, tstamps, model_ids, slos, &wl);
+    if (rc) return rc;
+    mmsim_batch *b = nullptr;
+    const mmsim_workload *wls[1] = {wl};
+    const uint32_t flags = MMSIM_BATCHING | MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS | MMSIM_WANT_PER_REQUEST;
+    rc = build_batch(ctx, wls, 1, &t, rl, flags, &b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
+    if (rc == MMSIM_OK) {
+        int64_t ng = 0;
+        double ls = 0.0;
+        mmsim_result r{};
+        r.n_good = &ng;
+        r.latency_sum = &ls;
+        r.model_num_requests = model_num_requests;
+        r.model_num_good = model_num_good_requests;
+        r.group_num_requests = group_num_requests;
+        r.group_num_good = group_num_good_requests;
+        r.finish = finish;
+        r.good = good;
+        rc = mmsim_batch_fetch(b, &r);
+    }
+    mmsim_batch_destroy(b);
+    mmsim_workload_destroy(wl);
+    return rc;
 }
 
 }  // extern "C"

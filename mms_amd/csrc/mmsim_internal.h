@@ -75,6 +75,43 @@ struct MixedArgs {
     int64_t *fp_ops;             // [n_seeds][tiles*64]
 };
 
+// Arguments of the batching simulation kernel.  Replica lists and group
+// descriptors are shared with the plain kernel; on top come, per seed, the
+// arrivals regrouped by model (a model's FIFO is always a window of that list)
+// and, per lane, the models of each group.
+struct BatchingArgs {
+    const Req *streams;          // all seeds' requests, back to back
+    const int64_t *stream_off;   // [n_seeds+1]
+    const int64_t *mq_off;       // [n_seeds][M+1] offsets into mq_* of the arrivals of each model
+    const double *mq_t;          // arrival time of each model-ordered arrival
+    const double *mq_dl;         // its deadline: arrival + (double)slo
+    const int32_t *mq_idx;       // its index in the seed's stream
+    const uint64_t *rep8;        // as in MixedArgs
+    const uint8_t *repx;
+    const uint32_t *ginfo;       // [tiles][Gmax+1][64]
+    const uint16_t *g2m_off;     // [tiles][Gmax+1][64] start of each group's model list
+    const uint16_t *g2m_idx;     // [tiles][members_max][64] model ids, ascending per group
+    const float *lat;            // [M][lat_row][NB]
+    const int32_t *batch_sizes;  // [NB]
+    int32_t M, lat_row, NB, rep_extra, members_max, heap_cap;
+    int32_t n_seeds, B, tiles, nslots, Gmax;
+    int32_t wave_lds_bytes;
+    int64_t Rmax;
+    double fixed_overhead;
+    uint32_t flags;
+    // outputs
+    int32_t *n_good;             // [n_seeds][tiles*64]
+    double *lat_sum;             // [n_seeds][tiles*64]
+    int32_t *status;             // [n_seeds][tiles*64] 0 or MMSIM_E_OVERFLOW
+    int32_t *model_good;         // [waves][M][64]
+    int32_t *group_req;          // [waves][Gmax][64]
+    int32_t *group_good;         // [waves][Gmax][64]
+    double *finish;              // [waves][Rmax][64]
+    uint8_t *good;               // [waves][Rmax][64]
+};
+hipError_t launch_sim_batching(const BatchingArgs &args, int waves_per_block, size_t lds_bytes, hipStream_t stream,
+                               std::string *err);
+
 // Launches the plain simulator with `waves_per_block` wavefronts per workgroup.
 hipError_t launch_sim_mixed(const MixedArgs &args, int smax_bucket, int waves_per_block, size_t lds_bytes,
                             hipStream_t stream, std::string *err);

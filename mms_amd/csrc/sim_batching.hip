@@ -1,0 +1,337 @@
+// Batching request-loop simulation for gfx950.
+//
+// Restates the reference's simulate_requests_mixed_batching
+// (alpa_serve/simulator/controller.py:631-798) with one lane per
+// (placement, arrival seed) and the 64 lanes of a wavefront walking the same
+// request stream.  The outer loop over arrivals is in lockstep; what happens
+// between two arrivals (idle groups picking up queued requests, dropping
+// requests that can no longer meet their deadline, growing a batch) differs
+// per lane and runs as divergent per-lane loops.
+//
+// State of a lane:
+//   * stage clocks clk[slot][lane] in LDS, as in the plain simulator; a
+//     group's "idle since" time is its first-stage clock (the reference keeps
+//     a separate array that always holds the same value, :727 and :725);
+//   * one FIFO per model.  A model's queue only ever holds a contiguous run
+//     of that model's arrivals, so it is a (head, tail) window into the
+//     seed's arrivals regrouped by model; tail is the number of arrivals so
+//     far (the same for every lane that hosts the model) and head[m][lane]
+//     lives in LDS;
+//   * the pending idle events, a multiset of (time, group) that the
+//     reference keeps in a heap (:728, :739-740): a small unsorted array per
+//     lane in LDS, popped by lexicographic minimum.  If a lane would need
+//     more entries than were provisioned it is flagged MMSIM_E_OVERFLOW and
+//     stops; its results are then reported as invalid.
+//
+// Arithmetic follows the reference: deadlines are arrival + (double)slo,
+// check_slo adds the fixed overhead last (:666-672) while a committed batch
+// adds it first (:715), batch growth tests the FIRST request's deadline only
+// (:693-702).
+
+#include "mmsim_internal.h"
+
+namespace mmsim {
+
+namespace {
+
+__device__ __forceinline__ int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ double dmax(double a, double b) { return b > a ? b : a; }
+__device__ __forceinline__ int ilog2i(int v) { return 31 - __clz(v); }
+
+__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_batching_kernel(const BatchingArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+
+    const int W = (int)(blockDim.x >> 6);
+    const int wv = uniform_i((int)(threadIdx.x >> 6));
+    const int lane = (int)(threadIdx.x & 63);
+    const int seed = (int)(blockIdx.x % (unsigned)a.n_seeds);
+    const int tile = (int)(blockIdx.x / (unsigned)a.n_seeds) * W + wv;
+    if (tile >= a.tiles) return;  // no barriers in this kernel
+    const bool want_model = (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
+    const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
+    const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
+    const int M = a.M, Gmax = a.Gmax, NB = a.NB;
+
+    // ---- LDS of this wavefront: group descriptors | clocks | queue heads | event times | event groups | arrivals per model
+    unsigned char *mine = lds_raw + wv * a.wave_lds_bytes;
+    uint32_t *ginfo = reinterpret_cast<uint32_t *>(mine) + lane;
+    size_t o = (size_t)(Gmax + 1) * kWave * 4;
+    double *clk = reinterpret_cast<double *>(mine + o) + lane;
+    o += (size_t)a.nslots * kWave * 8;
+    double *ev_t = reinterpret_cast<double *>(mine + o) + lane;
+    o += (size_t)a.heap_cap * kWave * 8;
+    uint32_t *head = reinterpret_cast<uint32_t *>(mine + o) + lane;
+    o += (size_t)M * kWave * 4;
+    uint32_t *ev_g = reinterpret_cast<uint32_t *>(mine + o) + lane;
+    o += (size_t)a.heap_cap * kWave * 4;
+    volatile uint32_t *arrived = reinterpret_cast<volatile uint32_t *>(mine + o);  // [M], same for all lanes
+
+    {
+        const uint32_t *gsrc = a.ginfo + (size_t)tile * (Gmax + 1) * kWave + lane;
+        for (int g = 0; g <= Gmax; ++g) ginfo[g * kWave] = gsrc[g * kWave];
+        for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
+        for (int m = 0; m < M; ++m) head[m * kWave] = 0u;
+        for (int m = lane; m < M; m += kWave) arrived[m] = 0u;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    const int wave = seed * a.tiles + tile;
+    const int64_t off = a.stream_off[seed];
+    const int64_t R = a.stream_off[seed + 1] - off;
+    const Req *__restrict__ reqs = a.streams + off;
+    const int64_t *__restrict__ mq_off = a.mq_off + (size_t)seed * (M + 1);
+    const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * M * kWave + lane;
+    const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * M * a.rep_extra * kWave + lane;
+    const uint16_t *__restrict__ g2m_off = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
+    const uint16_t *__restrict__ g2m_idx = a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
+    int32_t *model_good = a.model_good + (size_t)wave * M * kWave + lane;
+    int32_t *group_req = a.group_req + (size_t)wave * Gmax * kWave + lane;
+    int32_t *group_good = a.group_good + (size_t)wave * Gmax * kWave + lane;
+    double *fin_out = a.finish + (size_t)wave * a.Rmax * kWave + lane;
+    uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + lane;
+    const double overhead = a.fixed_overhead;
+
+    int32_t n_good = 0;
+    double lat_sum = 0.0;
+    int hn = 0;          // pending idle events of this lane
+    int dead = 0;        // nonzero status: this lane stopped (out of event slots / unsupported input)
+
+    const uint32_t none = (uint32_t)Gmax;
+
+    // queue length of a model this lane hosts
+    auto qlen = [&](int m) -> int { return (int)(arrived[m] - head[m * kWave]); };
+
+    // :654-664 -- among the models of group g with a waiting request, the one whose head arrived first
+    auto select_model = [&](uint32_t g) -> int {
+        const int lo = g2m_off[g * kWave], hi = g2m_off[(g + 1) * kWave];
+        double min_arrival = 1e100;
+        int pick = -1;
+        for (int x = lo; x < hi; ++x) {
+            const int m = g2m_idx[(size_t)x * kWave];
+            if (qlen(m) > 0) {
+                const double t = a.mq_t[mq_off[m] + head[m * kWave]];
+                if (t < min_arrival) {
+                    min_arrival = t;
+                    pick = m;
+                }
+            }
+        }
+        return pick;
+    };
+
+    // :666-672
+    auto check_slo = [&](double t0, const double *gclk, int stages, const float *lat_mg, int col, double deadline) -> bool {
+        double t = t0;
+        for (int k = 0; k < stages; ++k) t = dmax(gclk[k * kWave], t) + (double)lat_mg[(size_t)k * NB + col];
+        return (t + overhead) <= deadline;
+    };
+
+    // :706-732 with :674-704 inlined; the reference's recursion on "nothing servable" is the outer loop
+    auto handle = [&](double t0, int m, uint32_t g) {
+        const uint32_t d = ginfo[g * kWave];
+        const int stages = (int)desc_stages_m1(d) + 1;
+        double *gclk = clk + (desc_last_slot(d) - desc_stages_m1(d)) * kWave;
+        for (;;) {
+            const float *lat_mg = a.lat + ((size_t)m * a.lat_row + desc_lat_off(d)) * NB;
+            const int64_t base = mq_off[m];
+            // drop heads that cannot meet their deadline even alone (:677-686)
+            bool found = false;
+            int64_t first = 0;
+            while (qlen(m) > 0) {
+                const int64_t q = base + head[m * kWave];
+                head[m * kWave] += 1u;
+                if (check_slo(t0, gclk, stages, lat_mg, 0, a.mq_dl[q])) {
+                    found = true;
+                    first = q;
+                    break;
+                }
+                if (want_group) group_req[g * kWave] += 1;
+                if (want_req) {
+                    const int32_t r = a.mq_idx[q];
+                    fin_out[(size_t)r * kWave] = a.mq_t[q];
+                    good_out[(size_t)r * kWave] = 0;
+                }
+            }
+            if (!found) {  // :709-713
+                m = select_model(g);
+                if (m < 0) return;
+                continue;
+            }
+            // grow the batch while the first request still meets its deadline (:693-702)
+            int bs = 1;
+            const double deadline = a.mq_dl[first];
+            for (int b = 1; b < NB; ++b) {
+                const int cand = a.batch_sizes[b];
+                if (cand - 1 > qlen(m)) break;
+                if (!check_slo(t0, gclk, stages, lat_mg, ilog2i(cand), deadline)) break;
+                bs = cand;
+            }
+            // run it (:715-732)
+            const int col = ilog2i(bs);
+            double t = t0 + overhead;
+            for (int k = 0; k < stages; ++k) {
+                t = dmax(t, gclk[k * kWave]) + (double)lat_mg[(size_t)k * NB + col];
+                gclk[k * kWave] = t;
+            }
+            const double idle_at = gclk[0];
+            for (int u = 0; u < bs; ++u) {
+                int64_t q = first;
+                if (u > 0) {
+                    q = base + head[m * kWave];
+                    head[m * kWave] += 1u;
+                }
+                lat_sum += t - a.mq_t[q];
+                if (want_req) {
+                    const int32_t r = a.mq_idx[q];
+                    fin_out[(size_t)r * kWave] = t;
+                    good_out[(size_t)r * kWave] = 1;
+                }
+            }
+            n_good += bs;
+            if (want_group) {
+                group_req[g * kWave] += bs;
+                group_good[g * kWave] += bs;
+            }
+            if (want_model) model_good[(size_t)m * kWave] += bs;
+            if (hn >= a.heap_cap) {
+                dead = MMSIM_E_OVERFLOW;
+                return;
+            }
+            ev_t[hn * kWave] = idle_at;
+            ev_g[hn * kWave] = g;
+            hn += 1;
+            return;
+        }
+    };
+
+    // index of the lexicographically smallest (time, group) event, hn > 0
+    auto min_event = [&]() -> int {
+        int best = 0;
+        double bt = ev_t[0];
+        uint32_t bg = ev_g[0];
+        for (int e = 1; e < hn; ++e) {
+            const double t = ev_t[e * kWave];
+            const uint32_t g = ev_g[e * kWave];
+            if (t < bt || (t == bt && g < bg)) {
+                best = e;
+                bt = t;
+                bg = g;
+            }
+        }
+        return best;
+    };
+    auto pop_event = [&](int e, double &t, uint32_t &g) {
+        t = ev_t[e * kWave];
+        g = ev_g[e * kWave];
+        hn -= 1;
+        ev_t[e * kWave] = ev_t[hn * kWave];
+        ev_g[e * kWave] = ev_g[hn * kWave];
+    };
+
+    for (int64_t i = 0; i < R; ++i) {
+        const Req r = reqs[i];
+        const double tstamp = r.t;
+        const int m = uniform_i(r.m);
+
+        // ---- idle events that are due (:739-744)
+        while (!dead && hn > 0) {
+            const int e = min_event();
+            if (!(ev_t[e * kWave] <= tstamp)) break;
+            double ti;
+            uint32_t g;
+            pop_event(e, ti, g);
+            const int m2 = select_model(g);
+            if (m2 < 0) break;  // the popped event is dropped, later due events stay (:742-743)
+            handle(ti, m2, g);
+        }
+
+        // ---- the arrival (:746-778)
+        bool queued = false;
+        uint32_t gsel = none;
+        if (m >= 0) {
+            const uint64_t g8 = rep_tile[(size_t)m * kWave];
+            const bool hosted = (uint32_t)(g8 & 0xFFu) != none;
+            if (hosted && !dead) {
+                // group with the strictly smallest last-stage clock (:760-770)
+                double best = 1e100;
+                int j = 0;
+                for (;;) {
+                    uint32_t g;
+                    if (j < kPackedReplicas)
+                        g = (uint32_t)(g8 >> (8 * j)) & 0xFFu;
+                    else if (j - kPackedReplicas < a.rep_extra)
+                        g = repx_tile[((size_t)m * a.rep_extra + (j - kPackedReplicas)) * kWave];
+                    else
+                        break;
+                    if (g == none) break;
+                    const double c = clk[desc_last_slot(ginfo[g * kWave]) * kWave];
+                    if (c < best) {
+                        best = c;
+                        gsel = g;
+                    }
+                    ++j;
+                }
+                queued = true;
+            }
+        }
+        if (m >= 0) {
+            // every lane sees the same arrival count; lanes that do not host m never read it
+            __builtin_amdgcn_wave_barrier();
+            if (lane == 0) arrived[m] += 1u;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (!queued) {
+            if (want_req && !dead) {
+                fin_out[(size_t)i * kWave] = tstamp;
+                good_out[(size_t)i * kWave] = 0;
+            }
+        } else if (gsel == none) {
+            dead = MMSIM_E_UNSUPPORTED;  // every replica's clock is infinite; the reference indexes out of range here
+        } else {
+            const uint32_t d = ginfo[gsel * kWave];
+            const double idle_since = clk[(desc_last_slot(d) - desc_stages_m1(d)) * kWave];
+            if (tstamp >= idle_since) handle(tstamp, m, gsel);  // :776-778
+        }
+    }
+    // ---- drain (:781-787)
+    while (!dead && hn > 0) {
+        const int e = min_event();
+        double ti;
+        uint32_t g;
+        pop_event(e, ti, g);
+        const int m2 = select_model(g);
+        if (m2 < 0) continue;
+        handle(ti, m2, g);
+    }
+
+    const size_t out = (size_t)seed * a.tiles * kWave + (size_t)tile * kWave + lane;
+    a.n_good[out] = n_good;
+    a.lat_sum[out] = lat_sum;
+    a.status[out] = dead;
+}
+
+}  // namespace
+
+hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_bytes, hipStream_t stream,
+                               std::string *err) {
+    hipError_t e = hipSuccess;
+    if (wpb < 1 || wpb > kMaxWavesPerBlock) {
+        e = hipErrorInvalidValue;
+    } else {
+        auto kern = sim_batching_kernel;
+        if (lds_bytes > 64 * 1024)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds_bytes);
+        if (e == hipSuccess) {
+            const unsigned tile_groups = (unsigned)((args.tiles + wpb - 1) / wpb);
+            hipLaunchKernelGGL(kern, dim3(tile_groups * (unsigned)args.n_seeds), dim3(wpb * kWave), lds_bytes, stream, args);
+            e = hipGetLastError();
+        }
+    }
+    if (e != hipSuccess && err) *err = std::string("sim_batching launch: ") + hipGetErrorString(e);
+    return e;
+}
+
+}  // namespace mmsim

@@ -1,0 +1,125 @@
+"""GPU parity of the batching simulator.
+
+Bars: served/dropped flags, finish times and all counts bit-exact against
+(a) the golden vectors written by the reference's own function and (b) the CPU
+oracle on the seeded benchmark configuration.  The per-lane latency sum is
+accumulated in service order on the GPU and in arrival order by the oracle, so
+it is compared to 1e-12 relative.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from mms_amd import _lib, engine as E
+from mms_amd.synthetic import make_config
+from oracle import oracle_c
+from randcase import random_case
+from helpers import oracle_batch
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "batching_vectors.npz")
+BSS = [1, 2, 4, 8, 16]
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return E.Engine.default()
+
+
+def _single(eng, c, bss):
+    R = len(c["tstamps"])
+    fin, good = np.empty(R), np.empty(R, bool)
+    cnt = E.simulate_requests_mixed_batching(eng, fin, good, c["tstamps"], c["model_ids"], c["slos"], c["m2g"],
+                                             c["g2m"], c["num_stages"], c["lat"], bss)
+    return fin, good, cnt
+
+
+def test_reference_golden_vectors(eng):
+    z = np.load(GOLDEN)
+    n = int(z["num_cases"])
+    for i in range(n):
+        g = lambda k: z[f"c{i}_{k}"]
+        c = {k: g(k) for k in ("tstamps", "model_ids", "slos", "m2g", "g2m", "num_stages", "lat")}
+        fin, good, cnt = _single(eng, c, BSS[:int(g("nb"))])
+        assert np.array_equal(good, g("good")), i
+        assert np.array_equal(fin.view(np.uint64), g("finish").view(np.uint64)), i
+        for a, k in zip(cnt, ("mreq", "mgood", "greq", "ggood")):
+            assert np.array_equal(a, g(k)), (i, k)
+
+
+def test_random_cases_match_oracle(eng):
+    for seed in range(200):
+        nb = 1 + seed % 5
+        c = random_case(3_000_000 + seed, max_m=6, max_g=4, max_s=4, max_r=200, nb=nb, load=1.0 + seed % 9,
+                        inf_slo=False)
+        bss = BSS[:nb]
+        f0, g0, c0, _ = oracle_c.simulate_requests_mixed_batching(
+            c["tstamps"], c["model_ids"], c["slos"], c["m2g"], c["g2m"], c["num_stages"], c["lat"], bss)
+        fin, good, cnt = _single(eng, c, bss)
+        assert np.array_equal(good, g0), seed
+        assert np.array_equal(fin.view(np.uint64), f0.view(np.uint64)), seed
+        for a, b in zip(cnt, c0):
+            assert np.array_equal(a, b), seed
+
+
+def _run(eng, cfg, sols, seeds, flags):
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(sols, table)
+    streams = [cfg.stream(s) for s in seeds]
+    dws = [E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models) for st in streams]
+    batch = E.Batch(eng, dws, table, packed, flags | _lib.BATCHING)
+    batch.run()
+    ms = batch.sync()
+    out = batch.fetch()
+    info = batch.info()
+    batch.close()
+    return out, table, packed, streams, info, ms
+
+
+def _check(out, ref, s, per_request=False):
+    assert np.all(out["status"][s] == 0)
+    assert np.array_equal(out["n_good"][s], ref["n_good"])
+    assert np.array_equal(out["model_num_requests"][s], ref["model_num_requests"])
+    assert np.array_equal(out["model_num_good"][s], ref["model_num_good"])
+    assert np.array_equal(out["group_num_requests"][s], ref["group_num_requests"])
+    assert np.array_equal(out["group_num_good"][s], ref["group_num_good"])
+    np.testing.assert_allclose(out["latency_sum"][s], ref["latency_sum"], rtol=1e-12, atol=0)
+    if per_request:
+        R = ref["finish"].shape[1]
+        assert np.array_equal(out["good"][s][:, :R], ref["good"])
+        assert np.array_equal(out["finish"][s][:, :R].view(np.uint64), ref["finish"].view(np.uint64))
+
+
+def test_config5_subsample_counts(eng):
+    cfg = make_config(5, 96)
+    flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
+    out, table, packed, streams, info, ms = _run(eng, cfg, cfg.placements, [0, 1], flags)
+    print(info, f"kernel {ms:.1f} ms", flush=True)
+    for s, st in enumerate(streams):
+        ref = oracle_batch(st, table, packed, batching=True)
+        _check(out, ref, s)
+
+
+def test_config5_full_traces_for_a_few_placements(eng):
+    cfg = make_config(5, 3)
+    flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS | _lib.WANT_PER_REQUEST
+    out, table, packed, streams, _, _ = _run(eng, cfg, cfg.placements, [2], flags)
+    ref = oracle_batch(streams[0], table, packed, batching=True, want_per_request=True)
+    _check(out, ref, 0, per_request=True)
+
+
+def test_batching_on_the_small_configs_too(eng):
+    # configuration 2's placements with a batch-size axis added to the profiles
+    from mms_amd.profiling import synthetic_profile
+    cfg = make_config(2, 70)
+    pcs = sorted({c for s in cfg.placements for c in s.group_configs})
+    cfg.batch_sizes = [1, 2, 4]
+    cfg.profiles = [synthetic_profile(f"m{m}", float(cfg.latencies[m]), pcs, batch_sizes=cfg.batch_sizes,
+                                      batch_slope=0.2) for m in range(cfg.num_models)]
+    flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS | _lib.WANT_PER_REQUEST
+    out, table, packed, streams, _, _ = _run(eng, cfg, cfg.placements, [0, 3], flags)
+    for s, st in enumerate(streams):
+        ref = oracle_batch(st, table, packed, batching=True, want_per_request=True)
+        _check(out, ref, s, per_request=True)
