@@ -309,3 +309,336 @@ def gen_train_workload(model_datas: List[ModelData], seed: int = 0,
                                                           seed=seed + i)
              for i, d in enumerate(model_datas)]
     return Workload.merge(*parts)
+
+
+# ----------------------------------------------------------------------------------------
+# Search primitives.  They only differ from the reference in what sits behind
+# evaluator.get_scores / get_stats; the order of candidates, the tie-breaking
+# (np.argsort / np.argmax on the returned lists) and the use of numpy's global
+# random generator follow base_policy.py:284-796 so that a search explores the
+# same candidates in the same order.
+# ----------------------------------------------------------------------------------------
+
+def _group_memory(sol, weight_mem):
+    return [sum(weight_mem[c][m] for m in ms) for c, ms in zip(sol.group_configs, sol.group_models)]
+
+
+def replica_placement_round_robin(init_sol: ModelPlacement, model_datas: List[ModelData],
+                                  cluster_env: ClusterEnv, workload: Workload, verbose: int):
+    """Deal models to groups in turn while memory allows (:284-326)."""
+    assert len(init_sol.group_configs) == len(init_sol.group_models)
+    num_groups = len(init_sol.group_configs)
+    weight_mem = weight_mem_table(init_sol.group_configs, model_datas)
+    sol = init_sol
+    group_mem = _group_memory(sol, weight_mem)
+    g = 0
+    progress = True
+    while progress:
+        progress = False
+        for m in range(len(model_datas)):
+            need = weight_mem[sol.group_configs[g]][m]
+            if m not in sol.group_models[g] and need + group_mem[g] <= cluster_env.mem_budget:
+                progress = True
+                group_mem[g] += need
+                sol = sol.add_model(g, m)
+                sol.verify(model_datas, cluster_env)
+                g = (g + 1) % num_groups
+    return sol
+
+
+def replica_placement_fast_greedy(init_sol: ModelPlacement, model_datas: List[ModelData],
+                                  cluster_env: ClusterEnv, workload: Workload,
+                                  evaluator: PlacementEvaluator, verbose: int):
+    """Repeatedly give the model with most unserved requests a replica on the
+    least loaded group that still has memory for it (:329-400)."""
+    tic = time.time()
+    if evaluator is None:
+        evaluator = PlacementEvaluator(model_datas, cluster_env, workload, "fast_simulator", False)
+    weight_mem = weight_mem_table(init_sol.group_configs, model_datas)
+    sol = init_sol
+    it = 0
+    while True:
+        overall_goodput, goodputs, group_num_requests, fullstats = evaluator.get_stats([sol])[0]
+        unserved = [s.num_requests * (1 - gp) for s, gp in zip(fullstats.per_model_stats, goodputs)]
+        model_order = np.argsort(unserved)[::-1]
+        group_order = np.argsort(group_num_requests)
+        group_mem = _group_memory(sol, weight_mem)
+
+        choice = None
+        for g_id in group_order:
+            cfg = sol.group_configs[g_id]
+            for m_id in model_order:
+                if m_id not in sol.group_models[g_id] and \
+                        weight_mem[cfg][m_id] + group_mem[g_id] <= cluster_env.mem_budget:
+                    choice = (g_id, m_id)
+                    break
+            if choice:
+                break
+        if not choice:
+            break
+        sol = sol.add_model(*choice).normalize()
+        if verbose >= 2:
+            print(f"iter: {it}, score: {overall_goodput:.4f}, elapsed: {time.time() - tic:.2f}, "
+                  f"best placement: {sol}, ")
+        it += 1
+    return sol
+
+
+def _beam_loop(init_sol, evaluator, beam_size, verbose, expand, tic):
+    """Common driver of the two beam searches: expand every beam member, score
+    the new candidates in one batch, keep the top ``beam_size`` (:439-479)."""
+    beam = [init_sol]
+    best_score, best_sol = -1, init_sol
+    visited = set()
+    it = 0
+    while True:
+        next_sols = []
+        for sol in beam:
+            expand(sol, visited, next_sols)
+        if not next_sols:
+            break
+        scores = evaluator.get_scores(next_sols)
+        top = np.argsort(scores)[::-1][:beam_size]
+        beam = []
+        for idx in top:
+            beam.append(next_sols[idx])
+            if scores[idx] > best_score:
+                best_score, best_sol = scores[idx], next_sols[idx]
+        if verbose >= 1:
+            print(f"iter: {it}, best score: {best_score:.4f}, iter score: {scores[top[0]]:.4f}, "
+                  f"iter #sol: {len(next_sols)}, elapsed: {time.time() - tic:.2f}, "
+                  f"best placement: {best_sol}, ")
+        it += 1
+    return best_sol
+
+
+def replica_placement_beam_search(init_sol: ModelPlacement, model_datas: List[ModelData],
+                                  cluster_env: ClusterEnv, workload: Workload,
+                                  evaluator: PlacementEvaluator, beam_size: int, verbose: int):
+    """Beam search over "add one replica" moves (:403-479).  Note the strict
+    ``<`` against the memory budget here, unlike the greedy search."""
+    tic = time.time()
+    if evaluator is None:
+        evaluator = PlacementEvaluator(model_datas, cluster_env, workload, "fast_simulator", False)
+    num_models, num_groups = len(model_datas), len(init_sol.group_configs)
+    weight_mem = weight_mem_table(init_sol.group_configs, model_datas)
+
+    def expand(sol, visited, out):
+        group_mem = _group_memory(sol, weight_mem)
+        for g_id in range(num_groups):
+            cfg = sol.group_configs[g_id]
+            for m_id in range(num_models):
+                if weight_mem[cfg][m_id] + group_mem[g_id] < cluster_env.mem_budget and \
+                        m_id not in sol.group_models[g_id]:
+                    cand = sol.add_model(g_id, m_id).normalize()
+                    if cand.group_models not in visited:
+                        visited.add(cand.group_models)
+                        out.append(cand)
+
+    return _beam_loop(init_sol, evaluator, beam_size, verbose, expand, tic)
+
+
+def replica_placement_on_last_group(init_sol: ModelPlacement, model_datas: List[ModelData],
+                                    cluster_env: ClusterEnv, workload: Workload,
+                                    evaluator: PlacementEvaluator, beam_size: int, verbose: int):
+    """Beam search that only fills the last group, also trying to swap the
+    new model with one of an earlier group (:482-580)."""
+    tic = time.time()
+    if evaluator is None:
+        evaluator = PlacementEvaluator(model_datas, cluster_env, workload, "fast_simulator", False)
+    num_models, num_groups = len(model_datas), len(init_sol.group_configs)
+    weight_mem = weight_mem_table(init_sol.group_configs, model_datas)
+    last = num_groups - 1
+
+    def expand(sol, visited, out):
+        group_mem = _group_memory(sol, weight_mem)
+        cfg = sol.group_configs[last]
+        for m_id in range(num_models):
+            if not (weight_mem[cfg][m_id] + group_mem[last] < cluster_env.mem_budget and
+                    m_id not in sol.group_models[last]):
+                continue
+            cand = sol.add_model(last, m_id)
+            key = cand.normalize().group_models
+            if key in visited:
+                continue
+            visited.add(key)
+            out.append(cand)
+            at = list(cand.group_models[last]).index(m_id)
+            for g2 in range(num_groups - 1):
+                for at2 in range(len(cand.group_models[g2])):
+                    if cand.group_models[last][at] in cand.group_models[g2] or \
+                            cand.group_models[g2][at2] in cand.group_models[last]:
+                        continue
+                    rows = [list(x) for x in cand.group_models]
+                    rows[last][at], rows[g2][at2] = rows[g2][at2], rows[last][at]
+                    swapped = ModelPlacement(cand.group_configs, rows)
+                    skey = swapped.normalize().group_models
+                    if skey not in visited:
+                        visited.add(skey)
+                        out.append(swapped)
+
+    return _beam_loop(init_sol, evaluator, beam_size, verbose, expand, tic)
+
+
+def swap_two_models(sol: ModelPlacement):
+    """Swap two random replicas of two random groups if that creates no duplicate (:583-595)."""
+    rows = sol.group_models
+    g1 = np.random.choice(len(rows))
+    g2 = np.random.choice(len(rows))
+    i1 = np.random.choice(len(rows[g1]))
+    i2 = np.random.choice(len(rows[g2]))
+    if rows[g1][i1] in rows[g2] or rows[g2][i2] in rows[g1]:
+        return sol
+    new_rows = [list(x) for x in rows]
+    new_rows[g1][i1], new_rows[g2][i2] = new_rows[g2][i2], new_rows[g1][i1]
+    return ModelPlacement(sol.group_configs, new_rows)
+
+
+def swap_two_models_from_two_groups(sol: ModelPlacement, g_id_1, g_id_2):
+    """As :598-608, including its two return shapes."""
+    rows = sol.group_models
+    i1 = np.random.choice(len(rows[g_id_1]))
+    i2 = np.random.choice(len(rows[g_id_2]))
+    if rows[g_id_1][i1] in rows[g_id_2] or rows[g_id_2][i2] in rows[g_id_1]:
+        return False, sol
+    new_rows = [list(x) for x in rows]
+    new_rows[g_id_1][i1], new_rows[g_id_2][i2] = new_rows[g_id_2][i2], new_rows[g_id_1][i1]
+    return ModelPlacement(sol.group_configs, new_rows)
+
+
+def mutate_one_model(sol: ModelPlacement, num_models: int):
+    """Replace one random replica by a random model (:611-620)."""
+    rows = sol.group_models
+    g = np.random.choice(len(rows))
+    new_m = np.random.choice(num_models)
+    if new_m in rows[g]:
+        return sol
+    i = np.random.choice(len(rows[g]))
+    new_rows = [list(x) for x in rows]
+    new_rows[g][i] = new_m
+    return ModelPlacement(sol.group_configs, new_rows)
+
+
+def fit_mem_budget(group_config, group_models, model_num_unserved, weight_mem, mem_budget):
+    """In place: drop the least needed models until the group fits, then add
+    the most needed ones while it still fits (:775-796)."""
+    group_models.sort(key=lambda m: model_num_unserved[m])
+    used = sum(weight_mem[group_config][m] for m in group_models)
+    while used > mem_budget:
+        used -= weight_mem[group_config][group_models[0]]
+        del group_models[0]
+    for m in reversed(np.argsort(model_num_unserved)):
+        if m in group_models:
+            continue
+        if used + weight_mem[group_config][m] <= mem_budget:
+            group_models.append(m)
+            used += weight_mem[group_config][m]
+            continue
+        break
+
+
+def merge_two_groups(group_configs, group_models, model_num_unserved, weight_mem, mem_budget):
+    """In place: fuse two random groups of equal config into one of twice the
+    pipeline depth (:720-743)."""
+    for _ in range(10):
+        g1 = np.random.choice(len(group_models))
+        g2 = np.random.choice(len(group_models))
+        if g1 != g2 and group_configs[g1] == group_configs[g2]:
+            break
+    else:
+        return
+    old = group_configs[g1]
+    new_cfg = ParallelConfig(old.dp, old.op, old.pp * 2)
+    merged = list(set(group_models[g1] + group_models[g2]))
+    fit_mem_budget(new_cfg, merged, model_num_unserved, weight_mem, mem_budget)
+    group_configs[g1] = new_cfg
+    group_models[g1] = merged
+    del group_configs[g2]
+    del group_models[g2]
+
+
+def split_one_group(group_configs, group_models, model_num_unserved, weight_mem, mem_budget):
+    """In place: halve the pipeline depth of a random group with even depth
+    and deal its models to the two halves (:746-772)."""
+    for _ in range(10):
+        g = np.random.choice(len(group_models))
+        if group_configs[g].pp % 2 == 0:
+            break
+    else:
+        return
+    old = group_configs[g]
+    new_cfg = ParallelConfig(old.dp, old.op, old.pp // 2)
+    group_models[g].sort(key=lambda m: model_num_unserved[m])
+    half_a, half_b = group_models[g][::2], group_models[g][1::2]
+    fit_mem_budget(new_cfg, half_a, model_num_unserved, weight_mem, mem_budget)
+    fit_mem_budget(new_cfg, half_b, model_num_unserved, weight_mem, mem_budget)
+    group_configs[g] = new_cfg
+    group_models[g] = half_a
+    group_configs.append(new_cfg)
+    group_models.append(half_b)
+
+
+def evolutionary_search(init_sols: List[ModelPlacement], model_datas: List[ModelData],
+                        cluster_env: ClusterEnv, evaluator: PlacementEvaluator, num_iter: int,
+                        verbose: int):
+    """Population search: sample parents by score, merge/split groups and
+    mutate models toward the unserved ones, score the whole population in one
+    batch per iteration (:623-717)."""
+    tic = time.time()
+    pop_size = 1024
+    mutate_one_model_prob = 0.05
+    merge_group_prob = 0.08
+    split_group_prob = 0.08
+    num_models = len(model_datas)
+    mem_budget = cluster_env.mem_budget
+
+    weight_mem = {}
+    for m_id, x in enumerate(model_datas):
+        for c, entry in x.profiling_result.para_dict.items():
+            weight_mem.setdefault(c, [inf] * num_models)[m_id] = max(entry.weight_mem)
+
+    best_score, best_sol = -1, None
+    visited = set()
+    cur_sols = init_sols
+    for it in range(num_iter):
+        stats = evaluator.get_stats(cur_sols)
+        scores = np.array([x[0] for x in stats])
+        weights = scores / np.sum(scores)
+        unserved_cache = [None] * len(stats)
+
+        top = np.argmax(scores)
+        if scores[top] > best_score:
+            best_score, best_sol = scores[top], cur_sols[top]
+
+        next_sols = []
+        while len(next_sols) < pop_size:
+            idx = np.random.choice(len(scores), p=weights)
+            sol = cur_sols[idx]
+            if unserved_cache[idx] is None:
+                goodputs, fullstats = stats[idx][1], stats[idx][3]
+                raw = [s.num_requests * (1 - gp) for s, gp in zip(fullstats.per_model_stats, goodputs)]
+                unserved_cache[idx] = raw / np.sum(raw)
+            unserved = unserved_cache[idx]
+
+            group_configs = list(sol.group_configs)
+            group_models = [list(x) for x in sol.group_models]
+            if np.random.uniform() < merge_group_prob:
+                merge_two_groups(group_configs, group_models, unserved, weight_mem, mem_budget)
+            if np.random.uniform() < split_group_prob:
+                split_one_group(group_configs, group_models, unserved, weight_mem, mem_budget)
+            for g in range(len(group_models)):
+                for i in range(len(group_models[g])):
+                    if np.random.uniform() < mutate_one_model_prob:
+                        new_m = np.random.choice(num_models, p=unserved)
+                        if new_m not in group_models[g]:
+                            group_models[g][i] = new_m
+            child = ModelPlacement(group_configs, group_models).normalize()
+            next_sols.append(child)
+            visited.add(child.group_models)
+
+        if verbose >= 1:
+            print(f"iter: {it}, best score: {best_score:.4f}, iter avg-score: {np.mean(scores):.4f}, "
+                  f"iter #sol: {len(scores)}, visited #sol: {len(visited)}, "
+                  f"elapsed: {time.time() - tic:.2f}, best sol: {best_sol}, ")
+        cur_sols = next_sols + [best_sol]
+    return best_sol

@@ -1,0 +1,79 @@
+"""Test-only stand-in for the GPU library, built on the CPU oracle.
+
+``install(monkeypatch)`` swaps the entry points of ``mms_amd.engine`` that
+reach libmmsim for oracle-backed ones, so that the host-side logic (packing,
+PlacementEvaluator, approximate_one_case, the search policies) can be tested
+on a machine without a GPU.  Nothing outside tests/ may use this; the shipped
+package has no such path.
+"""
+import numpy as np
+
+from mms_amd import _lib, engine as E
+from oracle import oracle_c
+
+
+class _HostWorkload:
+    def __init__(self, engine, tstamps, model_ids, slos, num_models):
+        self.tstamps = np.ascontiguousarray(tstamps, np.float64)
+        self.model_ids = np.ascontiguousarray(model_ids, np.int32)
+        self.slos = np.ascontiguousarray(slos, np.float32)
+        self.R = len(self.tstamps)
+        self.M = int(num_models)
+
+    def close(self):
+        pass
+
+
+class _HostEngine:
+    device = -1
+
+    def device_info(self):
+        return {"name": "cpu-oracle", "arch": "none", "compute_units": 0, "clock_khz": 0,
+                "lds_bytes_per_block": 0, "hbm_bytes": 0}
+
+
+def _evaluate(engine, workloads, table, sols, flags=0, fixed_overhead=0.011):
+    packed = E.pack_placements(sols, table)
+    lat, pp = table.arrays()
+    num_groups, group_cfg, gm_off, gm_idx = packed
+    outs = []
+    for w in workloads:
+        outs.append(oracle_c.eval_placements(
+            w.tstamps, w.model_ids, w.slos, lat, pp, table.batch_sizes, num_groups, group_cfg, gm_off,
+            gm_idx, batching=bool(flags & _lib.BATCHING), fixed_overhead=fixed_overhead,
+            want_counts=True, want_per_request=bool(flags & _lib.WANT_PER_REQUEST)))
+    res = {"n_good": np.stack([o["n_good"] for o in outs]),
+           "latency_sum": np.stack([o["latency_sum"] for o in outs]),
+           "status": np.zeros((len(outs), len(sols)), np.int32), "kernel_ms": 0.0, "info": {}}
+    for k in ("model_num_requests", "model_num_good", "group_num_requests", "group_num_good"):
+        res[k] = np.stack([o[k] for o in outs])
+    if flags & _lib.WANT_PER_REQUEST:
+        res["finish"] = np.stack([o["finish"] for o in outs])
+        res["good"] = np.stack([o["good"] for o in outs])
+    return res
+
+
+def _simulate_requests_mixed(engine, finish, good, tstamps, model_ids, slos, m2g, num_stages, lat,
+                             num_requests=None, fixed_overhead=0.011):
+    f, g, cnt, _ = oracle_c.simulate_requests_mixed(tstamps, model_ids, slos, m2g, num_stages, lat, fixed_overhead)
+    finish[:] = f
+    good[:] = g
+    return cnt
+
+
+def _simulate_requests_mixed_batching(engine, finish, good, tstamps, model_ids, slos, m2g, g2m, num_stages,
+                                      lat, batch_sizes, num_requests=None, fixed_overhead=0.011):
+    f, g, cnt, _ = oracle_c.simulate_requests_mixed_batching(tstamps, model_ids, slos, m2g, g2m, num_stages,
+                                                             lat, batch_sizes, fixed_overhead)
+    finish[:] = f
+    good[:] = g
+    return cnt
+
+
+def install(monkeypatch):
+    host = _HostEngine()
+    monkeypatch.setattr(E.Engine, "default", classmethod(lambda cls: host))
+    monkeypatch.setattr(E, "DeviceWorkload", _HostWorkload)
+    monkeypatch.setattr(E, "evaluate", _evaluate)
+    monkeypatch.setattr(E, "simulate_requests_mixed", _simulate_requests_mixed)
+    monkeypatch.setattr(E, "simulate_requests_mixed_batching", _simulate_requests_mixed_batching)

@@ -1,0 +1,238 @@
+"""Host-side logic that needs no GPU: the C ABI surface, table packing,
+workload generation and statistics, helpers."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from mms_amd import _lib, engine as E
+from mms_amd.placement_policy import ClusterEnv, ModelData, ModelPlacement
+from mms_amd.profiling import (LatencyMemData, ParallelConfig, ProfilingResult, load_test_prof_result,
+                               synthetic_profile)
+from mms_amd.simulator.workload import (DeterministicProcess, GammaProcess, PoissonProcess, Request,
+                                        Workload)
+from mms_amd.synthetic import gamma_arrivals_fast, make_config, power_law_rates
+from mms_amd.util import (GB, decompose2tok, get2tok, get_factors, get_partitions, is_valid_size,
+                          to_str_round)
+from oracle import oracle_py
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- C ABI ------------------------------------------------------------------------------
+
+def test_library_loads_and_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "mmsim.h")).read()
+    declared = set(re.findall(r"\b(mmsim_[a-z_0-9]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in mmsim.h but not exported"
+    assert declared == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
+    assert lib.mmsim_abi_version() == int(re.search(r"#define MMSIM_ABI_VERSION (\d+)", header).group(1))
+
+
+def test_no_device_means_a_loud_error_not_a_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    with pytest.raises(_lib.MmsimError) as e:
+        E.Engine(0)
+    assert e.value.code == _lib.E_HIP and "HIP device" in str(e.value)
+
+
+def test_struct_layouts_match_the_header():
+    assert ctypes.sizeof(_lib.Tables) == 48
+    assert ctypes.sizeof(_lib.Placements) == 40
+    assert ctypes.sizeof(_lib.Result) == 10 * 8
+    assert ctypes.sizeof(_lib.BatchInfo) == 8 * 4 + 3 * 8
+
+
+# ---- table build (controller.py:412-476) --------------------------------------------------
+
+def test_latency_table_values_follow_the_reference_formula():
+    profs = [load_test_prof_result("alpa/bert-1.3b"), load_test_prof_result("test-2GB-100ms"),
+             load_test_prof_result("alpa/bert-2.6b")]
+    table = E.LatencyTable(profs)
+    cfgs = [ParallelConfig(1, 1, 4), ParallelConfig(1, 1, 1), ParallelConfig(1, 1, 8), ParallelConfig(1, 1, 2)]
+    ids = [table.config_id(c) for c in cfgs]
+    assert ids == [0, 1, 2, 3] and table.config_id(cfgs[2]) == 2
+    lat, pp = table.arrays()
+    assert lat.shape == (3, 4, 8, 1) and pp.tolist() == [4, 1, 8, 2]
+    # the independent restatement builds the per-placement table; compare column by column
+    m2g, g2m, ns, ref = oracle_py.build_tables(cfgs, [[0, 1, 2]] * 4, profs)
+    for c, cfg in enumerate(cfgs):
+        assert np.array_equal(lat[:, c, :cfg.pp, 0], ref[:, c, :cfg.pp, 0])
+    assert np.float32(0.028 * (1 + 0.009 * 4)) == lat[0, 0, 0, 0]
+    assert np.isinf(lat[2, 0]).all() and np.isinf(lat[1, 2]).all()      # configs without a profile
+    # batch sizes: the penalty still comes from the batch-1 stage list
+    prof = synthetic_profile("x", 0.2, [ParallelConfig(1, 1, 2)], batch_sizes=(1, 2, 4), batch_slope=0.15)
+    t2 = E.LatencyTable([prof], [1, 2, 4])
+    t2.config_id(ParallelConfig(1, 1, 2))
+    lat2, _ = t2.arrays()
+    want = [np.float32(prof.para_dict[ParallelConfig(1, 1, 2)].latency[b][0] * (1 + 0.009 * 2)) for b in (1, 2, 4)]
+    assert lat2[0, 0, 0].tolist() == want and lat2[0, 0, 1].tolist() == want
+
+
+def test_pack_placements_layout():
+    table = E.LatencyTable([load_test_prof_result("test-2GB-100ms")] * 5)
+    sols = [ModelPlacement([ParallelConfig(1, 1, 2)] * 2, [[0, 1, 2, 3], (0, 1)]),
+            ModelPlacement([ParallelConfig(1, 1, 4)], [np.array([3, 2])]),
+            ModelPlacement([], []),
+            ModelPlacement([ParallelConfig(1, 1, 1), ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 1)], [[], [4], []])]
+    ng, gc, off, idx = E.pack_placements(sols, table)
+    assert ng.tolist() == [2, 1, 0, 3]
+    assert gc.tolist() == [[0, 0, 0], [1, 0, 0], [0, 0, 0], [2, 0, 2]]
+    assert off.tolist() == [[0, 4, 6, 6], [6, 8, 8, 8], [8, 8, 8, 8], [8, 8, 9, 9]]
+    assert idx.tolist() == [0, 1, 2, 3, 0, 1, 3, 2, 4]
+
+
+def test_placement_helpers():
+    p = ModelPlacement([ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 1), ParallelConfig(1, 1, 4)], [[3, 1], [0], [2, 0]])
+    q = p.add_model(1, 5)
+    assert p.group_models[1] == [0] and q.group_models[1] == [0, 5] and q.group_configs is p.group_configs
+    n = q.normalize()
+    assert n.group_models == ((0, 2), (0, 5), (1, 3))
+    assert n.group_configs == (ParallelConfig(1, 1, 4), ParallelConfig(1, 1, 1), ParallelConfig(1, 1, 2))
+    c = p.copy()
+    c.group_models[0].append(9)
+    assert p.group_models[0] == [3, 1]
+    md = [ModelData(f"m{i}", 1, 1, 1, load_test_prof_result("test-2GB-100ms")) for i in range(4)]
+    ModelPlacement([ParallelConfig(1, 1, 1)], [[0, 1]]).verify(md, ClusterEnv(1, 4.5 * GB))
+    with pytest.raises(AssertionError):
+        ModelPlacement([ParallelConfig(1, 1, 1)], [[0, 1, 2]]).verify(md, ClusterEnv(1, 4.5 * GB))
+    with pytest.raises(AssertionError):
+        ModelPlacement([ParallelConfig(1, 1, 2)], [[0, 0]]).verify(md, ClusterEnv(2, 4.5 * GB))
+    with pytest.raises(AssertionError):      # no profile for this config -> infinite memory
+        ModelPlacement([ParallelConfig(1, 2, 1)], [[0]]).verify(md, ClusterEnv(2, 4.5 * GB))
+
+
+# ---- workloads (workload.py) ------------------------------------------------------------------
+
+def test_gamma_arrivals_fast_equals_the_sequential_loop():
+    for rate, cv, dur, seed in [(2.5, 1, 60, 0), (1, 4, 300, 7), (0.05, 8, 1000, 3), (30, 8, 100, 5),
+                                (0.3, 6, 50, 11), (0.01, 2, 400, 2), (0.02, 1, 90, 4), (0.011, 3, 95, 8)]:
+        slow = np.array(GammaProcess(rate, cv).generate_arrivals(0, dur, seed))
+        fast = gamma_arrivals_fast(rate, cv, 0, dur, seed)
+        assert slow.shape == fast.shape and np.array_equal(slow, fast)
+    # tiny blocks force the "draw another block" branch many times
+    refills = 0
+    for seed in range(40):
+        slow = np.array(GammaProcess(0.011, 1).generate_arrivals(5.0, 95, seed))
+        fast = gamma_arrivals_fast(0.011, 1, 5.0, 95, seed)
+        assert np.array_equal(slow, fast)
+        refills += len(slow) > 1          # block size is 1 here, so more than one arrival means a refill
+    assert refills > 5
+
+
+def test_workload_generation_statistics_and_merge():
+    w = GammaProcess(10, 3).generate_workload("m", 0, 2000, slo=0.5, seed=1)
+    assert abs(w.rate - 10) / 10 < 0.1 and abs(w.cv - 3) / 3 < 0.15
+    assert np.all(np.diff(w.arrivals) >= 0) and [r.idx for r in w.requests] == list(range(len(w)))
+    p = PoissonProcess(5).generate_workload("p", 0, 1000, seed=2)
+    assert abs(p.cv - 1) < 0.1
+    d = DeterministicProcess(4).generate_workload("d", 1.0, 10)
+    assert len(d) == 40 and d.arrivals[0] == 1.0 and abs(d.arrivals[1] - 1.25) < 1e-12 and d.cv < 1e-9
+    merged = w + p
+    assert len(merged) == len(w) + len(p)
+    assert np.all(np.diff(merged.arrivals) >= 0)
+    assert [r.idx for r in merged.requests] == list(range(len(merged)))
+    assert {r.model_name for r in merged.requests} == {"m", "p"}
+    assert Workload.merge(w) is w
+    parts = merged.split_time_interval(500)
+    assert sum(len(x) for x in parts) == len(merged) and len(parts) in (4, 5)
+    rr = merged.split_round_robin(3)
+    assert [len(x) for x in rr] == [len(merged[i::3]) for i in range(3)]
+    assert len(Workload.empty()) == 0 and Workload.empty().split_time_interval(1) == []
+    with pytest.raises(NotImplementedError):
+        merged[3]
+    assert str(merged).startswith("Workload(len=")
+
+
+def test_compute_stats_conventions():
+    arrivals = np.arange(100, dtype=float)
+    reqs = [Request("a" if i % 4 else "b", None, 1.0, i, {}) for i in range(100)]
+    w = Workload(arrivals, reqs)
+    good = np.ones(100, bool)
+    good[::10] = False
+    finish = arrivals + np.where(good, 0.5 + 0.001 * np.arange(100), 0.0)
+    st = w.compute_stats(arrivals, finish, good, warmup=10)
+    # skip = int(10/99*100) = 10 -> requests 10..89 are counted
+    assert st.num_requests == 80
+    assert [s.name for s in st.per_model_stats] == ["b", "a"]          # ascending request count
+    a = st.per_model_stats[1]
+    idx = np.array([i for i in range(10, 90) if i % 4])
+    ok = good[idx]
+    lat = (finish - arrivals)[idx][ok]
+    assert a.num_requests == len(idx) and a.goodput == np.mean(ok)
+    assert a.latency_p90 == np.sort(lat)[int(0.9 * len(lat))] and a.latency_p99 == np.sort(lat)[int(0.99 * len(lat))]
+    assert st.goodput == np.mean(good[10:90]) and st.latency_mean == np.mean((finish - arrivals)[10:90])
+    none_good = w.compute_stats(arrivals, arrivals.copy(), np.zeros(100, bool), warmup=10)
+    assert all(s.goodput == 0 and s.throughput == 0 and s.latency_mean == 0 for s in none_good.per_model_stats)
+    Workload.print_stats(st)
+
+
+# ---- profiles ---------------------------------------------------------------------------------
+
+def test_profiles():
+    p = load_test_prof_result("alpa/bert-1.3b")
+    assert p.para_dict[ParallelConfig(1, 1, 8)].latency[1][-1] == 0.016
+    assert p.para_dict[ParallelConfig(1, 1, 2)].weight_mem == [1.3 * GB, 1.3 * GB]
+    with pytest.raises(ValueError):
+        load_test_prof_result("nope")
+    r = ProfilingResult("x", {}, 0, 0)
+    r.add_result(ParallelConfig(1, 1, 2), 1, [0.2, 0.3], [1, 1], [5, 5])
+    r.add_result(ParallelConfig(1, 1, 2), 1, [0.25, 0.25], [2, 2], [6, 6], "better")    # smaller bottleneck wins
+    r.add_result(ParallelConfig(1, 1, 2), 1, [0.1, 0.4], [3, 3], [7, 7])                # larger bottleneck ignored
+    r.add_result(ParallelConfig(1, 1, 2), 2, [0.3, 0.3], [4, 4], [8, 8])
+    e = r.para_dict[ParallelConfig(1, 1, 2)]
+    assert e.latency == {1: [0.25, 0.25], 2: [0.3, 0.3]} and e.weight_mem == [6, 6] and e.metadata == "better"
+    s = synthetic_profile("s", 0.2, [ParallelConfig(1, 2, 4), ParallelConfig(1, 1, 1)], (1, 2), 0.15, stage_comm=0.002)
+    assert s.para_dict[ParallelConfig(1, 2, 4)].latency[2] == [0.2 * 1.15 / 4 * 1.05 + 0.002] * 4
+    assert s.para_dict[ParallelConfig(1, 1, 1)].latency[1] == [0.2]
+
+
+# ---- helpers (util.py) ------------------------------------------------------------------------
+
+def test_partition_helpers():
+    assert get_factors(12) == [1, 2, 3, 4, 6, 12] and get_factors(1) == [1] and get_factors(49) == [1, 7, 49]
+    assert get2tok(34) == [1, 2, 4, 8, 16, 32] and get2tok(1) == [1]
+    assert decompose2tok(13) == [1, 4, 8] and decompose2tok(0) == [] and decompose2tok(64) == [64]
+    assert get_partitions(5, 1) == [[5]]
+    assert get_partitions(4, 2) == [[3, 1], [2, 2], [1, 3]]
+    for n, k in [(16, 3), (24, 3), (12, 4)]:
+        parts = get_partitions(n, k)
+        assert all(sum(p) == n and len(p) == k and min(p) >= 1 for p in parts)
+        assert len({tuple(p) for p in parts}) == len(parts)
+    # n = 12: a trailing part must be <= 12 % 8 or leave a multiple of 8
+    assert [p[-1] for p in get_partitions(12, 2)] == [1, 2, 3, 4]
+    assert is_valid_size(16, 5) and not is_valid_size(12, 5)
+    assert to_str_round([1, 2.5, "x", None, {"a": 0.1234567}], 2) == "[1, 2.50, x, None, {'a': '0.12'}]"
+
+
+def test_synthetic_configs_are_deterministic_and_as_specified():
+    c1 = make_config(1)
+    s = c1.stream(0)
+    assert 1000 < len(s.tstamps) < 1500 and s.slos.dtype == np.float32 and np.all(s.slos == np.float32(0.5))
+    assert c1.placements[0].group_configs == [ParallelConfig(1, 1, 4)] * 2
+    c2a, c2b = make_config(2), make_config(2, 10)
+    assert len(c2a.placements) == 64
+    assert [p.group_models for p in c2a.placements[:10]] == [p.group_models for p in c2b.placements]
+    for p in c2a.placements:
+        assert sum(c.pp for c in p.group_configs) == 16 and all(2 <= len(ms) <= 6 for ms in p.group_models)
+    assert np.array_equal(c2a.stream(3).tstamps, c2b.stream(3).tstamps)
+    c3 = make_config(3, 130)
+    assert c3.placements[0].group_models[0] == [0, 32, 1, 0] and len(c3.placements[129].group_configs) == 32
+    assert abs(power_law_rates(64, 200.0, 0.5).sum() - 200.0) < 1e-9
+    c4 = make_config(4, 8)
+    for p in c4.placements:
+        assert sum(c.op * c.pp for c in p.group_configs) == 64
+        assert all(c.op in (1, 2, 4) and 8 <= len(ms) <= 24 for c, ms in zip(p.group_configs, p.group_models))
+    c5 = make_config(5, 4)
+    assert c5.batching and c5.batch_sizes == [1, 2, 4, 8] and set(np.round(c5.latencies, 2)) == {0.06, 0.12, 0.25, 0.5}
+    w = c2a.workload(1)
+    st = c2a.stream(1)
+    assert np.array_equal(w.arrivals, st.tstamps)
+    assert [r.model_name for r in w.requests] == [f"m{m}" for m in st.model_ids]

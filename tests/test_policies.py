@@ -1,0 +1,234 @@
+"""Placement evaluator, approximate_one_case and the search policies.
+
+Every test runs twice: with the CPU oracle standing in for the library
+(host logic, runs anywhere) and, marked ``gpu``, through libmmsim itself.
+
+The known answers of ``test_*_reference_answer`` are the ones the reference
+asserts in its own tests/serve/test_placement_policy.py:24-77; they depend on
+the simulator's goodput counts, the tie-breaking of the searches and the
+seeded training workload all being right.
+"""
+import json
+import os
+from functools import partial
+
+import numpy as np
+import pytest
+
+import oracle_backend
+from mms_amd.placement_policy import (ClusterEnv, ModelData, ModelParallelismGreedy, ModelParallelismRR,
+                                      ModelParallelismSearch, ModelPlacement, ModelPlacementWithReplacement,
+                                      PlacementEvaluator, SelectiveReplicationGreedy,
+                                      SelectiveReplicationReplacement, SelectiveReplicationSearch,
+                                      SelectiveReplicationUniform, gen_train_workload)
+from mms_amd.placement_policy.base_policy import (evolutionary_search, replica_placement_beam_search,
+                                                  replica_placement_on_last_group)
+from mms_amd.profiling import ParallelConfig, load_test_prof_result
+from mms_amd.simulator.controller import DummyController, approximate_one_case
+from mms_amd.simulator.executable import Executable
+from mms_amd.simulator.workload import GammaProcess, Workload
+from mms_amd.util import GB, ServingCase
+
+
+@pytest.fixture(params=["oracle", pytest.param("gpu", marks=pytest.mark.gpu)])
+def backend(request, monkeypatch):
+    if request.param == "oracle":
+        oracle_backend.install(monkeypatch)
+    return request.param
+
+
+def four_models(slo=1, rate=5, cv=1, prof="test-2GB-100ms"):
+    return [ModelData(f"m{i}", slo, rate, cv, load_test_prof_result(prof)) for i in range(4)]
+
+
+def _golden_cases():
+    with open(os.path.join(os.path.dirname(__file__), "golden", "search_vectors.json")) as f:
+        return json.load(f)["cases"]
+
+
+@pytest.mark.parametrize("case", _golden_cases(), ids=lambda c: c["name"])
+def test_policies_return_what_the_reference_returns(backend, case):
+    """Final placement, its score, goodput and per-group request counts as
+    recorded from the reference's own policies (tests/golden/make_search_vectors.py)."""
+    import mms_amd.placement_policy as pp
+    n, slo, rate, cv = case["models"][:4]
+    prof = case["models"][4] if len(case["models"]) > 4 else "test-2GB-100ms"
+    model_datas = [ModelData(f"m{i}", slo, rate, cv, load_test_prof_result(prof)) for i in range(n)]
+    cluster_env = ClusterEnv(*case["cluster"])
+    placement, _ = getattr(pp, case["policy"])(**case["kwargs"]).solve_placement(model_datas, cluster_env)
+    assert [list(c) for c in placement.group_configs] == case["placement"]["group_configs"]
+    assert [[int(m) for m in ms] for ms in placement.group_models] == case["placement"]["group_models"]
+    wl = gen_train_workload(model_datas)
+    ev = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+    score = ev.get_scores([placement])[0]
+    assert abs(score - case["score"]) <= 1e-12 * abs(case["score"])
+    goodput, _, group_num_requests, _ = ev.get_stats([placement])[0]
+    assert goodput == case["goodput"]
+    assert [int(x) for x in group_num_requests] == case["group_num_requests"]
+
+
+def test_assertions_of_the_reference_test_file(backend):
+    """tests/serve/test_placement_policy.py:24-77.  Its expectation for
+    SelectiveReplicationGreedy (every model on exactly two groups) is not what
+    the reference's present code returns -- see ref_test_sr_greedy in
+    search_vectors.json -- so only the three that hold are asserted here."""
+    cluster_env = ClusterEnv(num_devices=4, mem_budget=4.5 * GB)
+    placement, _ = SelectiveReplicationSearch().solve_placement(four_models(), cluster_env)
+    assert all(g == ParallelConfig(1, 1, 1) for g in placement.group_configs)
+    for i in range(4):
+        assert sum(list(x).count(i) for x in placement.group_models) == 2
+
+    placement, _ = ModelParallelismGreedy(group_size=2).solve_placement(four_models(), cluster_env)
+    assert len(placement.group_configs) == 2
+    assert placement.group_configs[0].pp == 2 and placement.group_configs[1].pp == 2
+    assert list(placement.group_models[0]) == [0, 1, 2, 3]
+    assert list(placement.group_models[1]) == [0, 1, 2, 3]
+
+    cluster_env = ClusterEnv(num_devices=4, mem_budget=2.5 * GB)
+    placement, _ = ModelParallelismSearch().solve_placement(four_models(0.4, 4, 8), cluster_env)
+    assert len(placement.group_configs) == 1
+    assert placement.group_configs[0].pp == 4
+    assert list(placement.group_models[0]) == [0, 1, 2, 3]
+
+
+def test_place_models_api_with_a_controller(backend):
+    calls = []
+
+    class Recorder(DummyController):
+        def create_mesh_group_manager(self, *a, **k):
+            calls.append(("mesh", a))
+
+        def create_replica(self, *a, **k):
+            calls.append(("replica", a))
+
+    cluster_env = ClusterEnv(num_devices=4, mem_budget=4.5 * GB)
+    for policy in [SelectiveReplicationGreedy(), ModelParallelismGreedy()]:
+        calls.clear()
+        controller = Recorder()
+        placement = policy.place_models(controller, cluster_env, four_models())
+        n_mesh = sum(1 for c in calls if c[0] == "mesh")
+        n_rep = sum(1 for c in calls if c[0] == "replica")
+        assert n_mesh == len(placement.group_configs)
+        assert n_rep == sum(len(ms) for ms in placement.group_models)
+
+
+def _case(sol, model_datas, workload):
+    def register_models(controller):
+        for d in model_datas:
+            controller.register_model.remote(d.name, partial(Executable, d.profiling_result))
+    return ServingCase(register_models, lambda start=0: workload, lambda controller: sol)
+
+
+def test_evaluator_batch_equals_one_by_one(backend):
+    model_datas = four_models(0.5, 6, 4)
+    cluster_env = ClusterEnv(num_devices=4, mem_budget=4.5 * GB)
+    wl = gen_train_workload(model_datas, simulation_min_samples=4000)
+    sols = [ModelPlacement([ParallelConfig(1, 1, 2)] * 2, [[0, 1], [2, 3]]),
+            ModelPlacement([ParallelConfig(1, 1, 4)], [(0, 1, 2, 3)]),
+            ModelPlacement([ParallelConfig(1, 1, 1)] * 4, [[0, 1], [1, 2], np.array([2, 3]), [3, 0]]),
+            ModelPlacement([ParallelConfig(1, 1, 1)] * 4, [[0], [0], [1], []])]
+    ev = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+    scores = ev.get_scores(sols)
+    stats = ev.get_stats(sols)
+    for sol, score, st in zip(sols, scores, stats):
+        one_stats, _ = approximate_one_case(_case(sol, model_datas, wl), fast_stats=True)
+        n_rep = sum(len(x) for x in sol.group_models)
+        want = one_stats.goodput - one_stats.latency_mean / 10000 + n_rep / 1000000
+        assert abs(score - want) <= 1e-12 * abs(want)
+        goodput, model_goodput, group_num_requests, full = st
+        assert goodput == one_stats.goodput
+        assert tuple(group_num_requests) == tuple(one_stats.group_num_requests)
+        assert model_goodput == [x.goodput for x in one_stats.per_model_stats]
+        assert [x.num_requests for x in full.per_model_stats] == [x.num_requests for x in one_stats.per_model_stats]
+        assert abs(full.latency_mean - one_stats.latency_mean) <= 1e-12 * one_stats.latency_mean
+        assert full.num_requests == one_stats.num_requests == len(wl)
+    # static one-placement helpers of the reference API
+    s0 = PlacementEvaluator.get_goodput_simulation(sols[0], model_datas, cluster_env, wl, "fast_simulator")
+    assert abs(s0 - scores[0]) <= 1e-12 * abs(s0)
+    assert ev.get_scores([]) == [] and ev.get_stats([]) == []
+    with pytest.raises(NotImplementedError):
+        PlacementEvaluator(model_datas, cluster_env, wl, "simulator", False)
+
+
+def test_approximate_one_case_full_stats_and_unknown_model(backend):
+    model_datas = four_models(0.5, 6, 2)
+    wl = gen_train_workload(model_datas, simulation_min_samples=3000)
+    extra = GammaProcess(2, 1).generate_workload("not-registered", 0, 100, slo=1.0, seed=77)
+    wl = Workload.merge(wl, extra)
+    sol = ModelPlacement([ParallelConfig(1, 1, 2)] * 2, [[0, 1, 2], [1, 2, 3]])
+    stats, placement = approximate_one_case(_case(sol, model_datas, wl))          # compute_stats path
+    assert placement is sol
+    names = [s.name for s in stats.per_model_stats]
+    assert "not-registered" in names
+    assert stats.per_model_stats[names.index("not-registered")].goodput == 0
+    assert len(stats.group_num_requests) == 2
+    fast, _ = approximate_one_case(_case(sol, model_datas, wl), fast_stats=True)
+    assert 0 < fast.goodput < 1
+    assert fast.num_requests == len(wl)
+
+
+def test_placement_with_replacement_is_simulated_per_segment(backend):
+    model_datas = four_models(0.5, 6, 2)
+    wl = gen_train_workload(model_datas, simulation_min_samples=3000)
+    # (segments must have the same number of groups: the per-group counts are summed, controller.py:388)
+    a = ModelPlacement([ParallelConfig(1, 1, 1)] * 4, [[0, 1], [0, 1], [2, 3], [2, 3]])
+    b = ModelPlacement([ParallelConfig(1, 1, 1)] * 4, [[0], [1], [2], [3]])
+    cut = float(wl.arrivals[len(wl) // 2])
+    both = ModelPlacementWithReplacement([0.0, cut], [a, b])
+    stats, _ = approximate_one_case(_case(both, model_datas, wl), fast_stats=True)
+    # the same by hand: first half on a, second half on b, clocks reset in between
+    i = int(np.searchsorted(wl.arrivals, cut, side="right"))
+    sa, _ = approximate_one_case(_case(a, model_datas, wl[:i]), fast_stats=True)
+    sb, _ = approximate_one_case(_case(b, model_datas, wl[i:]), fast_stats=True)
+    good = sa.goodput * i + sb.goodput * (len(wl) - i)
+    assert abs(stats.goodput - good / len(wl)) < 1e-12
+    ev = PlacementEvaluator(model_datas, ClusterEnv(4, 4.5 * GB), wl, "fast_simulator", False)
+    assert abs(ev.get_stats([both])[0][0] - stats.goodput) < 1e-15
+
+
+def test_other_policies_and_searches_run(backend):
+    cluster_env = ClusterEnv(num_devices=4, mem_budget=4.5 * GB)
+    model_datas = four_models(0.6, 4, 3)
+    wl = gen_train_workload(model_datas, simulation_min_samples=2500)
+    rr, _ = ModelParallelismRR().solve_placement(model_datas, cluster_env, wl)
+    assert rr.group_configs == [ParallelConfig(1, 1, 4)]
+    uni, _ = SelectiveReplicationUniform().solve_placement(model_datas, cluster_env, wl)
+    assert [list(x) for x in uni.group_models] == [[0, 1], [1, 2], [2, 3], [3, 0]]
+    rep, _ = SelectiveReplicationReplacement(40).solve_placement(model_datas, cluster_env, wl)
+    assert isinstance(rep, ModelPlacementWithReplacement) and len(rep.placements) >= 2
+    rep.verify(model_datas, cluster_env)
+    ev = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+    init = ModelPlacement([ParallelConfig(1, 1, 2)] * 2, [[], []])
+    beam = replica_placement_beam_search(init, model_datas, cluster_env, wl, ev, 2, 0)
+    beam.verify(model_datas, cluster_env)
+    last = replica_placement_on_last_group(init, model_datas, cluster_env, wl, ev, 2, 0)
+    last.verify(model_datas, cluster_env)
+    np.random.seed(0)
+    evo = evolutionary_search([beam], model_datas, cluster_env, ev, 2, 0)
+    assert ev.get_scores([evo])[0] >= ev.get_scores([beam])[0] - 1e-12
+    sep = ModelParallelismSearch(use_separation=True)
+    mixed = [ModelData("a", 1, 3, 2, load_test_prof_result("test-2GB-100ms")),
+             ModelData("b", 2, 2, 2, load_test_prof_result("test-4GB-150ms"))]
+    placement, _ = sep.solve_placement(mixed, ClusterEnv(4, 4.5 * GB))
+    placement.verify(mixed, ClusterEnv(4, 4.5 * GB))
+
+
+def test_batching_evaluator(backend, monkeypatch):
+    import mms_amd.util as U
+    from mms_amd.profiling import synthetic_profile
+    monkeypatch.setattr(U, "batchsize_config", [1, 2, 4])
+    import mms_amd.simulator.controller as ctl
+    monkeypatch.setattr(ctl, "batchsize_config", [1, 2, 4])
+    pcs = [ParallelConfig(1, 1, 1), ParallelConfig(1, 1, 2)]
+    model_datas = [ModelData(f"m{i}", 0.8, 8, 3, synthetic_profile(f"m{i}", 0.1 + 0.02 * i, pcs, (1, 2, 4), 0.2))
+                   for i in range(3)]
+    wl = gen_train_workload(model_datas, simulation_min_samples=3000)
+    sols = [ModelPlacement([pcs[1]] * 2, [[0, 1], [1, 2]]), ModelPlacement([pcs[0]] * 4, [[0], [1], [2], [0, 1]])]
+    ev = PlacementEvaluator(model_datas, ClusterEnv(4, 8 * GB), wl, "fast_simulator", False, enable_batching=True)
+    plain = PlacementEvaluator(model_datas, ClusterEnv(4, 8 * GB), wl, "fast_simulator", False)
+    sb, sp = ev.get_scores(sols), plain.get_scores(sols)
+    assert all(b > p for b, p in zip(sb, sp))          # batching serves more under this load
+    for sol, st in zip(sols, ev.get_stats(sols)):
+        one, _ = approximate_one_case(_case(sol, model_datas, wl), fast_stats=True, enable_batching=True)
+        assert st[0] == one.goodput
+        assert tuple(st[2]) == tuple(one.group_num_requests)
