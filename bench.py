@@ -65,6 +65,9 @@ def main():
     ap.add_argument("--seeds", type=int, default=None, help="use only the first N arrival seeds")
     ap.add_argument("--cpu-sample", type=int, default=1024, help="placements timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
+                    help="also launch one plain device copy of BYTES (read BYTES, write BYTES) so that "
+                         "FETCH_SIZE / WRITE_SIZE counters of a profiled run can be scaled")
     ap.add_argument("--flags", type=str, default="scores", choices=["scores", "model", "stats"],
                     help="scores: goodput+latency only; model: + per-model counts; stats: + per-group counts")
     args = ap.parse_args()
@@ -85,6 +88,16 @@ def main():
     R_total = sum(len(s.tstamps) for s in streams)
     log(f"[bench] {cfg.name}: {B} placements x {len(seeds)} seeds, {R_total} requests over seeds, "
         f"inputs generated in {time.perf_counter() - t0:.1f}s")
+
+    if args.copy_calibration:
+        import torch
+        src = torch.ones(args.copy_calibration // 4, dtype=torch.int32, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)                      # the calibration launch (the fill above is a write-only kernel)
+        torch.cuda.synchronize()
+        log(f"[bench] copy calibration: one device copy of {args.copy_calibration} bytes")
+        del src, dst
 
     eng = E.Engine.default()
     dev = eng.device_info()

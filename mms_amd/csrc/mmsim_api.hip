@@ -105,6 +105,7 @@ struct mmsim_batch {
 
     DevBuf<Req> streams;
     DevBuf<int64_t> stream_off;
+    DevBuf<uint32_t> rep32, repx32;
     DevBuf<uint64_t> rep8;
     DevBuf<uint8_t> repx;
     DevBuf<uint8_t> rmax;
@@ -279,8 +280,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     int heap_cap = 0;
     if (!batching) {
         // shared latency table + per-wavefront private region
-        wave_bytes = ((size_t)kStageBytes + rmax_lds_bytes + (size_t)(Gmax + 1) * kWave * sizeof(uint32_t) +
-                      (size_t)nslots * kWave * sizeof(double) +
+        wave_bytes = ((size_t)kStageBytes + rmax_lds_bytes + (size_t)nslots * kWave * sizeof(double) +
                       ((flags & MMSIM_WANT_GROUP_COUNTS) ? (size_t)2 * Gmax * kWave * sizeof(uint32_t) : 0) + 15) & ~(size_t)15;
         const size_t lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
         if (lat_bytes + wave_bytes <= (size_t)ctx->max_lds)
@@ -352,12 +352,22 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 pack_desc(slot0[(size_t)p * Gmax + g], (uint32_t)t->cfg_pp[c], (uint32_t)lat_off[c], (uint32_t)g);
         }
     }
-    // ---- replica lists as group indices: first 8 packed [tiles][M][64] x u64, the rest
-    //      [tiles][M][RX][64] x u8; missing entries name the empty row Gmax
+    // ---- replica lists.  Plain simulator: descriptors, the first 8 as [tiles][M][2][64] x (4 x u32),
+    //      the rest [tiles][M][RX][64] x u32, missing entries empty.  Batching simulator: group
+    //      indices, first 8 packed [tiles][M][64] x u64, the rest [tiles][M][RX][64] x u8, missing
+    //      entries name the empty descriptor row Gmax.
     const int RX = std::max(rmax_all - kPackedReplicas, 0);
     const uint64_t none8 = 0x0101010101010101ull * (uint64_t)Gmax;
-    std::vector<uint64_t> rep8((size_t)b->tiles * M * kWave, none8);
-    std::vector<uint8_t> repx((size_t)b->tiles * M * RX * kWave, (uint8_t)Gmax);
+    std::vector<uint32_t> rep32, repx32;
+    std::vector<uint64_t> rep8;
+    std::vector<uint8_t> repx;
+    if (batching) {
+        rep8.assign((size_t)b->tiles * M * kWave, none8);
+        repx.assign((size_t)b->tiles * M * RX * kWave, (uint8_t)Gmax);
+    } else {
+        rep32.assign((size_t)b->tiles * M * 2 * kWave * 4, kEmpty);
+        repx32.assign((size_t)b->tiles * M * RX * kWave, kEmpty);
+    }
     std::vector<uint8_t> rmax((size_t)b->tiles * M, 0);
     for (int32_t p = 0; p < B; ++p) {
         const int tile = b->pos[p] / kWave, lane = b->pos[p] % kWave;
@@ -368,14 +378,21 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             uint64_t word = none8;
             for (int64_t x = lo; x < hi; ++x) {
                 const int32_t g = rl.grp[(size_t)x];
-                if (g < 0 || g >= rl.num_groups[p]) return fail(MMSIM_E_INVALID, "replica list names a group that does not exist");
                 const int j = (int)(x - lo);
-                if (j < kPackedReplicas)
-                    word = (word & ~(0xFFull << (8 * j))) | ((uint64_t)g << (8 * j));
-                else
-                    repx[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = (uint8_t)g;
+                if (batching) {
+                    if (j < kPackedReplicas)
+                        word = (word & ~(0xFFull << (8 * j))) | ((uint64_t)g << (8 * j));
+                    else
+                        repx[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = (uint8_t)g;
+                } else {
+                    const uint32_t d = ginfo[((size_t)tile * (Gmax + 1) + g) * kWave + lane];
+                    if (j < kPackedReplicas)  // word j/4 of the lane, component j%4
+                        rep32[((((size_t)tile * M + m) * 2 + (size_t)(j / 4)) * kWave + lane) * 4 + (size_t)(j % 4)] = d;
+                    else
+                        repx32[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = d;
+                }
             }
-            rep8[((size_t)tile * M + m) * kWave + lane] = word;
+            if (batching) rep8[((size_t)tile * M + m) * kWave + lane] = word;
         }
     }
 
@@ -450,12 +467,20 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                                    hipMemcpyDeviceToDevice, st));
     HIP_TRY(b->stream_off.alloc(soff.size()));
     HIP_TRY(hipMemcpyAsync(b->stream_off.p, soff.data(), sizeof(int64_t) * soff.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(b->rep8.alloc(rep8.size()));
-    HIP_TRY(hipMemcpyAsync(b->rep8.p, rep8.data(), sizeof(uint64_t) * rep8.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(b->repx.alloc(repx.size()));
-    if (!repx.empty()) HIP_TRY(hipMemcpyAsync(b->repx.p, repx.data(), repx.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(b->ginfo.alloc(ginfo.size()));
-    HIP_TRY(hipMemcpyAsync(b->ginfo.p, ginfo.data(), sizeof(uint32_t) * ginfo.size(), hipMemcpyHostToDevice, st));
+    if (batching) {
+        HIP_TRY(b->rep8.alloc(rep8.size()));
+        HIP_TRY(hipMemcpyAsync(b->rep8.p, rep8.data(), sizeof(uint64_t) * rep8.size(), hipMemcpyHostToDevice, st));
+        HIP_TRY(b->repx.alloc(repx.size()));
+        if (!repx.empty()) HIP_TRY(hipMemcpyAsync(b->repx.p, repx.data(), repx.size(), hipMemcpyHostToDevice, st));
+        HIP_TRY(b->ginfo.alloc(ginfo.size()));
+        HIP_TRY(hipMemcpyAsync(b->ginfo.p, ginfo.data(), sizeof(uint32_t) * ginfo.size(), hipMemcpyHostToDevice, st));
+    } else {
+        HIP_TRY(b->rep32.alloc(rep32.size()));
+        HIP_TRY(hipMemcpyAsync(b->rep32.p, rep32.data(), sizeof(uint32_t) * rep32.size(), hipMemcpyHostToDevice, st));
+        HIP_TRY(b->repx32.alloc(repx32.size()));
+        if (!repx32.empty())
+            HIP_TRY(hipMemcpyAsync(b->repx32.p, repx32.data(), sizeof(uint32_t) * repx32.size(), hipMemcpyHostToDevice, st));
+    }
     HIP_TRY(b->rmax.alloc(rmax.size()));
     HIP_TRY(hipMemcpyAsync(b->rmax.p, rmax.data(), rmax.size(), hipMemcpyHostToDevice, st));
     HIP_TRY(b->lat.alloc(lat.size()));
@@ -513,10 +538,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     MixedArgs &a = b->args;
     a.streams = b->streams.p;
     a.stream_off = b->stream_off.p;
-    a.rep8 = b->rep8.p;
-    a.repx = b->repx.p;
+    a.rep32 = reinterpret_cast<const uint4 *>(b->rep32.p);
+    a.repx32 = b->repx32.p;
     a.rmax = b->rmax.p;
-    a.ginfo = b->ginfo.p;
     a.lat = b->lat.p;
     a.M = M;
     a.lat_row = lat_row;
@@ -858,7 +882,8 @@ int mmsim_batch_get_info(const mmsim_batch *b, mmsim_batch_info *out) {
     out->slots = b->nslots;
     out->lds_bytes = (int32_t)b->lds_bytes;
     out->requests_total = b->Rtotal;
-    out->table_bytes = (int64_t)(b->rep8.bytes() + b->repx.bytes() + b->ginfo.bytes() + b->rmax.bytes() + b->lat.bytes());
+    out->table_bytes = (int64_t)(b->rep32.bytes() + b->repx32.bytes() + b->rep8.bytes() + b->repx.bytes() + b->ginfo.bytes() +
+                                 b->rmax.bytes() + b->lat.bytes() + b->lat_nb.bytes());
     out->stream_bytes = (int64_t)b->streams.bytes();
     return MMSIM_OK;
 }

@@ -20,7 +20,9 @@ struct __attribute__((aligned(16))) Req {
 };
 static_assert(sizeof(Req) == 16, "Req must be 16 bytes");
 
-// Group descriptor: one 32-bit word per (placement, group), kept per lane in LDS.
+// Group descriptor: one 32-bit word per (placement, group).  The plain simulator
+// reads a model's replicas as descriptors; the batching simulator keeps a per
+// lane table of them in LDS and lists replicas as group indices.
 //   bits  0..7   clock slot of the group's LAST pipeline stage (slots are the
 //                placement's pipeline stages laid end to end)
 //   bits  8..12  stages of the group minus one
@@ -50,10 +52,9 @@ constexpr int kStageBytes = kWave * (int)sizeof(Req);  // one staged block of re
 struct MixedArgs {
     const Req *streams;          // all seeds' requests, back to back
     const int64_t *stream_off;   // [n_seeds+1] element offsets into streams
-    const uint64_t *rep8;        // [tiles][M][64] group indices of the first 8 replicas, one byte each
-    const uint8_t *repx;         // [tiles][M][rep_extra][64] group indices of replicas 8, 9, ...
+    const uint4 *rep32;          // [tiles][M][2][64] descriptors of the first 8 replicas, four to a 16-byte word
+    const uint32_t *repx32;      // [tiles][M][rep_extra][64] descriptors of replicas 8, 9, ...
     const uint8_t *rmax;         // [tiles][M] most replicas of model m over the tile's lanes
-    const uint32_t *ginfo;       // [tiles][Gmax+1][64] group descriptors (row Gmax is kEmpty)
     const float *lat;            // [M][lat_row] compact stage latencies (batch size 1)
     int32_t M, lat_row, rep_extra;
     int32_t n_seeds, B, tiles, nslots, Gmax;

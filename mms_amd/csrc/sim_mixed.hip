@@ -12,13 +12,14 @@
 //   * requests are fetched 64 at a time with one coalesced 1 KiB load per
 //     wavefront (one block ahead, into registers), parked in LDS and read
 //     back with broadcast LDS reads;
-//   * the replicas of the request's model are group indices, one byte each,
-//     eight to a 64-bit word rep8[tile][model][lane] (one coalesced 512-byte
-//     load per request, listed in the order the reference scans them),
-//     fetched one chunk of requests ahead into registers; the load count per
-//     chunk is fixed so the wait counters let the prefetch overlap;
-//   * a per-lane table of group descriptors (last-stage clock slot, stage
-//     count, latency-row offset) lives in LDS as ginfo[group][lane];
+//   * the replicas of the request's model are 32-bit descriptors (last-stage
+//     clock slot, stage count, latency-row offset, group index), eight per
+//     (tile, model, lane) in two 16-byte words rep32[tile][model][2][lane]
+//     (two coalesced 1 KiB loads per request, listed in the order the
+//     reference scans them).  They are fetched one chunk of requests ahead
+//     into registers together with the request's arrival time and SLO; the
+//     load count per chunk is fixed so the wait counters let the prefetch
+//     overlap the current chunk;
 //   * per-lane stage clocks live in LDS as clk[slot][lane] (8 bytes each);
 //     the slots of a lane are its groups' pipeline stages laid end to end.
 //     The bank an access hits depends on the lane only, so any per-lane
@@ -28,10 +29,13 @@
 //     (model, config) has one latency for all its stages the table shrinks
 //     to lat[model][config] and the per-stage latency reads disappear.
 //
+// A request therefore costs two dependent LDS round trips: (1) last-stage
+// clock and last-stage latency of every listed replica, (2) the stage clocks
+// of the chosen group; single-stage placements need only the first.
 // Group choice (strictly smallest last-stage clock, first listed wins ties)
-// is a select chain; the stage walk and the commit are nests of divergent
-// ifs, which the compiler turns into exec narrowing with a wave-uniform exit
-// as soon as no lane has another stage.
+// is a select chain; stage walk, SLO decision and commit are one
+// hand-scheduled inline-asm block (walk_asm.inc), with a C++ version for the
+// shapes the block is not generated for.
 //
 // A lane whose request cannot meet its SLO even if it only had to wait for
 // the chosen group's last stage skips the walk: with t >= arrival at every
@@ -112,18 +116,40 @@ __device__ __forceinline__ void walk_blocks(C &&c, B &&b) {
     }
 }
 
-constexpr int kChunk = 8;  // requests whose replica words are fetched ahead together
-
-struct Chunk {
-    int m[kChunk];        // wave-uniform model id (or -1)
-    int nrep[kChunk];     // wave-uniform replica bound of the tile for that model
-    uint64_t g8[kChunk];  // per-lane group indices of the first 8 replicas
+// Requests whose descriptors and fields are fetched ahead together.  The fetch
+// of a chunk has the time the previous chunk takes to arrive; four requests
+// cover the latency of the descriptor loads (eight measured no faster).
+template <int SMAX>
+struct ChunkFor {
+    static constexpr int value = 4;
 };
+
+template <int CH>
+struct Chunk {
+    int m[CH];        // wave-uniform model id (or -1)
+    int nrep[CH];     // wave-uniform replica bound of the tile for that model
+    double t[CH];     // arrival time (same in every lane)
+    float slo[CH];    // SLO (same in every lane)
+    uint4 da[CH];     // per-lane descriptors of replicas 0..3
+    uint4 db[CH];     // per-lane descriptors of replicas 4..7
+};
+
+template <int J>
+__device__ __forceinline__ uint32_t pick_desc(const uint4 &a, const uint4 &b) {
+    if constexpr (J == 0) return a.x;
+    if constexpr (J == 1) return a.y;
+    if constexpr (J == 2) return a.z;
+    if constexpr (J == 3) return a.w;
+    if constexpr (J == 4) return b.x;
+    if constexpr (J == 5) return b.y;
+    if constexpr (J == 6) return b.z;
+    return b.w;
+}
 
 template <int SMAX, bool LATLDS, bool UNIFORM>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(const MixedArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    constexpr int CH = kChunk;
+    constexpr int CH = ChunkFor<SMAX>::value;
     constexpr int RREG = kPackedReplicas;
 
     const int W = (int)(blockDim.x >> 6);
@@ -137,7 +163,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const bool want_ops = (a.flags & MMSIM_WANT_OP_COUNT) != 0;
 
-    // ---- LDS: [latency table][per wavefront: request block | replica bounds | group descriptors | clocks | group counters]
+    // ---- LDS: [latency table][per wavefront: request block | replica bounds | clocks | group counters]
     float *lat_lds = reinterpret_cast<float *>(lds_raw);
     const int lat_floats = LATLDS ? a.M * a.lat_row : 0;
     const int lat_bytes = (lat_floats * 4 + 15) & ~15;
@@ -145,18 +171,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     Req *stage = reinterpret_cast<Req *>(mine);
     int4 *stage4 = reinterpret_cast<int4 *>(mine);
     uint8_t *rmax_lds = mine + kStageBytes;
-    uint32_t *ginfo = reinterpret_cast<uint32_t *>(mine + kStageBytes + a.rmax_lds_bytes) + lane;
-    const int ginfo_bytes = (a.Gmax + 1) * kWave * 4;
-    double *clk = reinterpret_cast<double *>(mine + kStageBytes + a.rmax_lds_bytes + ginfo_bytes) + lane;
-    uint32_t *gcnt =
-        reinterpret_cast<uint32_t *>(mine + kStageBytes + a.rmax_lds_bytes + ginfo_bytes + a.nslots * (kWave * 8)) + lane;
+    double *clk = reinterpret_cast<double *>(mine + kStageBytes + a.rmax_lds_bytes) + lane;
+    uint32_t *gcnt = reinterpret_cast<uint32_t *>(mine + kStageBytes + a.rmax_lds_bytes + a.nslots * (kWave * 8)) + lane;
 
     for (int i = (int)threadIdx.x; i < lat_floats; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
-    if (live) {
+    if (live)
         for (int i = lane; i < a.M; i += kWave) rmax_lds[i] = a.rmax[(size_t)tile * a.M + i];
-        const uint32_t *gsrc = a.ginfo + (size_t)tile * (a.Gmax + 1) * kWave + lane;
-        for (int g = 0; g <= a.Gmax; ++g) ginfo[g * kWave] = gsrc[g * kWave];
-    }
     __syncthreads();
     if (!live) return;  // padding wavefront of the last workgroup
 
@@ -168,8 +188,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const int64_t off = a.stream_off[seed];
     const int64_t R = a.stream_off[seed + 1] - off;
     const int4 *__restrict__ reqs4 = reinterpret_cast<const int4 *>(a.streams + off);
-    const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * a.M * kWave + lane;
-    const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * a.M * a.rep_extra * kWave + lane;
+    const uint4 *__restrict__ rep_tile = a.rep32 + (size_t)tile * a.M * 2 * kWave + lane;
+    const uint32_t *__restrict__ repx_tile = a.repx32 + (size_t)tile * a.M * a.rep_extra * kWave + lane;
+    const float *lat_base = LATLDS ? lat_lds : a.lat;
     int32_t *model_good = a.model_good + (size_t)wave * a.M * kWave + lane;
     double *fin_out = a.finish + (size_t)wave * a.Rmax * kWave + lane;
     uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + lane;
@@ -190,21 +211,26 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         }
         const int nblk = (int)(R - blk < kWave ? R - blk : kWave);  // requests in this block
 
-        // Always CH loads per chunk, whatever the requests are.
-        auto load_chunk = [&](Chunk &c, int cb) {
+        // Always 2*CH loads per chunk, whatever the requests are.
+        auto load_chunk = [&](Chunk<CH> &c, int cb) {
             static_while<0, CH>([&](auto U) {
                 constexpr int u = decltype(U)::value;
                 const int idx = cb + u;  // < 64
-                const int m = uniform(stage[idx].m);
+                const Req r = stage[idx];  // broadcast read
+                const int m = uniform(r.m);
                 const bool ok = idx < nblk && m >= 0;
                 c.m[u] = m;
                 c.nrep[u] = ok ? uniform((int)rmax_lds[ok ? m : 0]) : 0;
-                c.g8[u] = rep_tile[(size_t)(ok ? m : 0) * kWave];
+                c.t[u] = r.t;
+                c.slo[u] = r.slo;
+                const uint4 *row = rep_tile + (size_t)(ok ? m : 0) * (2 * kWave);
+                c.da[u] = row[0];
+                c.db[u] = row[kWave];
                 return true;
             });
         };
 
-        Chunk cur, nxt;
+        Chunk<CH> cur, nxt;
         load_chunk(cur, 0);
         for (int cb = 0; cb < nblk; cb += CH) {
             const bool more = cb + CH < nblk;
@@ -213,44 +239,44 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             static_while<0, CH>([&](auto U) {
                 constexpr int u = decltype(U)::value;
                 if (cb + u >= nblk) return false;
-                const Req r = stage[cb + u];  // broadcast read
-                const double tstamp = r.t;
-                const double slo = (double)r.slo;
+                const double tstamp = cur.t[u];
+                const double slo = (double)cur.slo[u];
                 const int m = cur.m[u];
                 const int n = cur.nrep[u];
-                const uint32_t glo = (uint32_t)cur.g8[u], ghi = (uint32_t)(cur.g8[u] >> 32);
+                const float *lrow_m = lat_base + (size_t)(m < 0 ? 0 : m) * a.lat_row;
 
-                // ---- choose the replica group: strictly smallest last-stage clock (:590-598)
+                // ---- choose the replica group: strictly smallest last-stage clock (:590-598).
+                //      One LDS round trip fetches, for every listed replica, the clock of its last
+                //      stage and the latency of its last stage (needed by the early-reject bound).
                 double best = 1e100;
                 uint32_t sel = kEmpty;
+                float lsel = 0.0f;
                 int nvalid = 0;
-                auto consider = [&](uint32_t d, double c) {
+                auto lat_index = [&](uint32_t d) { return desc_lat_off(d) + (UNIFORM ? 0u : desc_stages_m1(d)); };
+                auto consider = [&](uint32_t d, double c, float l) {
                     const bool valid = (int32_t)d >= 0;
                     const bool better = valid && c < best;
                     best = better ? c : best;
                     sel = better ? d : sel;
+                    lsel = better ? l : lsel;
                     if (want_ops) nvalid += valid ? 1 : 0;
                 };
                 // Scan 4 or 8 list entries without branching: entries past a lane's own
-                // replicas name the empty descriptor row, whose clock read is ignored.
+                // replicas are empty descriptors, whose reads are harmless and ignored.
                 auto scan = [&](auto NJ) {
                     constexpr int nj = decltype(NJ)::value;
-                    uint32_t info[nj];
                     double cl[nj];
+                    float ll[nj];
                     static_while<0, nj>([&](auto J) {
                         constexpr int j = decltype(J)::value;
-                        const uint32_t g = ((j < 4 ? glo : ghi) >> (8 * (j & 3))) & 0xFFu;
-                        info[j] = ginfo[g * kWave];
+                        const uint32_t d = pick_desc<j>(cur.da[u], cur.db[u]);
+                        cl[j] = clk[desc_last_slot(d) * kWave];
+                        ll[j] = lrow_m[lat_index(d)];
                         return true;
                     });
                     static_while<0, nj>([&](auto J) {
                         constexpr int j = decltype(J)::value;
-                        cl[j] = clk[desc_last_slot(info[j]) * kWave];
-                        return true;
-                    });
-                    static_while<0, nj>([&](auto J) {
-                        constexpr int j = decltype(J)::value;
-                        consider(info[j], cl[j]);
+                        consider(pick_desc<j>(cur.da[u], cur.db[u]), cl[j], ll[j]);
                         return true;
                     });
                 };
@@ -259,10 +285,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 else if (n > 0)
                     scan(Idx<4>{});
                 if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
-                    const uint8_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
+                    const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
                     for (int j = RREG; j < n; ++j) {
-                        const uint32_t d = ginfo[(uint32_t)row[(size_t)(j - RREG) * kWave] * kWave];
-                        consider(d, clk[desc_last_slot(d) * kWave]);
+                        const uint32_t d = row[(size_t)(j - RREG) * kWave];
+                        consider(d, clk[desc_last_slot(d) * kWave], lrow_m[lat_index(d)]);
                     }
                 }
 
@@ -270,94 +296,107 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 const int sm1 = has ? (int)desc_stages_m1(sel) : -1;  // stages - 1
                 const uint32_t slot0 = has ? desc_last_slot(sel) - (uint32_t)sm1 : 0u;
                 double *gclk = clk + slot0 * kWave;
-                const uint32_t lidx = (uint32_t)(m < 0 ? 0 : m) * (uint32_t)a.lat_row + (has ? desc_lat_off(sel) : 0u);
-                const float *lrow = (LATLDS ? lat_lds : a.lat) + lidx;
-
-                // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
-                int walk = -1;  // stages - 1 of lanes that walk
-                double l_const = 0.0;
-                if (has) {
-                    const double l_last = (double)lrow[UNIFORM ? 0 : sm1];
-                    l_const = l_last;
-                    const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
-                    walk = bound > slo ? -1 : sm1;
-                }
+                const float *lrow = lrow_m + (has ? desc_lat_off(sel) : 0u);
+                const double l_last = (double)lsel;
 
                 double finish_time;
                 bool acc;
-                if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
-                    // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
-                    uint64_t saved_exec;
-                    int accepted;
-                    double t, latency;
-                    const uint32_t cb = lds_addr(gclk);
-                    if constexpr (UNIFORM) {
-                        if constexpr (SMAX == 4)
-                            asm volatile(MMSIM_WALK_U4_TEXT
-                                         : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t), [fin] "=&v"(finish_time),
-                                           [lat] "=&v"(latency), [ng] "+v"(n_good), [ls] "+v"(lat_sum)
-                                         : [walk] "v"(walk), [cb] "v"(cb), [lc] "v"(l_const), [ts] "v"(tstamp), [slo] "v"(slo),
-                                           [oh] "s"(overhead)
-                                         : "vcc", "memory", MMSIM_WALK_U4_CLOBBERS);
-                        else
-                            asm volatile(MMSIM_WALK_U16_TEXT
-                                         : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t), [fin] "=&v"(finish_time),
-                                           [lat] "=&v"(latency), [ng] "+v"(n_good), [ls] "+v"(lat_sum)
-                                         : [walk] "v"(walk), [cb] "v"(cb), [lc] "v"(l_const), [ts] "v"(tstamp), [slo] "v"(slo),
-                                           [oh] "s"(overhead)
-                                         : "vcc", "memory", MMSIM_WALK_U16_CLOBBERS);
-                    } else {
-                        const uint32_t lb = lds_addr(lrow);
-                        if constexpr (SMAX == 4)
-                            asm volatile(MMSIM_WALK_N4_TEXT
-                                         : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t), [fin] "=&v"(finish_time),
-                                           [lat] "=&v"(latency), [ng] "+v"(n_good), [ls] "+v"(lat_sum)
-                                         : [walk] "v"(walk), [cb] "v"(cb), [lb] "v"(lb), [ts] "v"(tstamp), [slo] "v"(slo),
-                                           [oh] "s"(overhead)
-                                         : "vcc", "memory", MMSIM_WALK_N4_CLOBBERS);
-                        else
-                            asm volatile(MMSIM_WALK_N16_TEXT
-                                         : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t), [fin] "=&v"(finish_time),
-                                           [lat] "=&v"(latency), [ng] "+v"(n_good), [ls] "+v"(lat_sum)
-                                         : [walk] "v"(walk), [cb] "v"(cb), [lb] "v"(lb), [ts] "v"(tstamp), [slo] "v"(slo),
-                                           [oh] "s"(overhead)
-                                         : "vcc", "memory", MMSIM_WALK_N16_CLOBBERS);
-                    }
-                    acc = accepted != 0;
-                } else {
-                    // ---- the same in plain C++ (other stage buckets, latency table in global memory):
-                    //      fetch, then the dependent chain (:605-608)
-                    double cv[SMAX];
-                    float lv[SMAX];
-                    walk_blocks<0, 1, SMAX>(
-                        [&](auto K) { return decltype(K)::value <= walk; },
-                        [&](auto K) {
-                            constexpr int k = decltype(K)::value;
-                            cv[k] = gclk[k * kWave];
-                            if (!UNIFORM) lv[k] = lrow[k];
-                        });
-                    double t = tstamp;
-                    walk_blocks<0, 1, SMAX>(
-                        [&](auto K) { return decltype(K)::value <= walk; },
-                        [&](auto K) {
-                            constexpr int k = decltype(K)::value;
-                            t = vmax(t, cv[k]) + (UNIFORM ? l_const : (double)lv[k]);
-                            cv[k] = t;
-                        });
-                    finish_time = t + overhead;  // :610
+                if constexpr (SMAX == 1) {
+                    // ---- single-stage groups: the clock read for the choice is the whole pipeline (:605-619)
+                    const double t = vmax(tstamp, best) + l_last;
+                    finish_time = t + overhead;
                     const double latency = finish_time - tstamp;
-                    acc = walk >= 0 && latency <= slo;  // :613
-                    if (acc) {  // :614-619
+                    acc = has && latency <= slo;
+                    if (acc) {
+                        gclk[0] = t;
                         n_good += 1;
                         lat_sum += latency;
                     }
-                    const int commit = acc ? walk : -1;
-                    walk_blocks<0, 1, SMAX>(
-                        [&](auto K) { return decltype(K)::value <= commit; },
-                        [&](auto K) {
-                            constexpr int k = decltype(K)::value;
-                            gclk[k * kWave] = cv[k];
-                        });
+                } else {
+                    // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
+                    int walk = -1;  // stages - 1 of lanes that walk
+                    if (has) {
+                        const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
+                        walk = bound > slo ? -1 : sm1;
+                    }
+                    if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
+                        // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
+                        uint64_t saved_exec;
+                        int accepted;
+                        double t, latency;
+                        const uint32_t cb_addr = lds_addr(gclk);
+                        if constexpr (UNIFORM) {
+                            if constexpr (SMAX == 4)
+                                asm volatile(MMSIM_WALK_U4_TEXT
+                                             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t),
+                                               [fin] "=&v"(finish_time), [lat] "=&v"(latency), [ng] "+v"(n_good),
+                                               [ls] "+v"(lat_sum)
+                                             : [walk] "v"(walk), [cb] "v"(cb_addr), [lc] "v"(l_last), [ts] "v"(tstamp),
+                                               [slo] "v"(slo), [oh] "s"(overhead)
+                                             : "vcc", "memory", MMSIM_WALK_U4_CLOBBERS);
+                            else
+                                asm volatile(MMSIM_WALK_U16_TEXT
+                                             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t),
+                                               [fin] "=&v"(finish_time), [lat] "=&v"(latency), [ng] "+v"(n_good),
+                                               [ls] "+v"(lat_sum)
+                                             : [walk] "v"(walk), [cb] "v"(cb_addr), [lc] "v"(l_last), [ts] "v"(tstamp),
+                                               [slo] "v"(slo), [oh] "s"(overhead)
+                                             : "vcc", "memory", MMSIM_WALK_U16_CLOBBERS);
+                        } else {
+                            const uint32_t lb = lds_addr(lrow);
+                            if constexpr (SMAX == 4)
+                                asm volatile(MMSIM_WALK_N4_TEXT
+                                             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t),
+                                               [fin] "=&v"(finish_time), [lat] "=&v"(latency), [ng] "+v"(n_good),
+                                               [ls] "+v"(lat_sum)
+                                             : [walk] "v"(walk), [cb] "v"(cb_addr), [lb] "v"(lb), [ts] "v"(tstamp),
+                                               [slo] "v"(slo), [oh] "s"(overhead)
+                                             : "vcc", "memory", MMSIM_WALK_N4_CLOBBERS);
+                            else
+                                asm volatile(MMSIM_WALK_N16_TEXT
+                                             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t),
+                                               [fin] "=&v"(finish_time), [lat] "=&v"(latency), [ng] "+v"(n_good),
+                                               [ls] "+v"(lat_sum)
+                                             : [walk] "v"(walk), [cb] "v"(cb_addr), [lb] "v"(lb), [ts] "v"(tstamp),
+                                               [slo] "v"(slo), [oh] "s"(overhead)
+                                             : "vcc", "memory", MMSIM_WALK_N16_CLOBBERS);
+                        }
+                        acc = accepted != 0;
+                    } else {
+                        // ---- the same in plain C++ (other stage buckets, latency table in global memory):
+                        //      fetch, then the dependent chain (:605-608)
+                        double cv[SMAX];
+                        float lv[SMAX];
+                        walk_blocks<0, 1, SMAX>(
+                            [&](auto K) { return decltype(K)::value <= walk; },
+                            [&](auto K) {
+                                constexpr int k = decltype(K)::value;
+                                cv[k] = gclk[k * kWave];
+                                if (!UNIFORM) lv[k] = lrow[k];
+                            });
+                        double t = tstamp;
+                        walk_blocks<0, 1, SMAX>(
+                            [&](auto K) { return decltype(K)::value <= walk; },
+                            [&](auto K) {
+                                constexpr int k = decltype(K)::value;
+                                t = vmax(t, cv[k]) + (UNIFORM ? l_last : (double)lv[k]);
+                                cv[k] = t;
+                            });
+                        finish_time = t + overhead;  // :610
+                        const double latency = finish_time - tstamp;
+                        acc = walk >= 0 && latency <= slo;  // :613
+                        if (acc) {  // :614-619
+                            n_good += 1;
+                            lat_sum += latency;
+                        }
+                        const int commit = acc ? walk : -1;
+                        walk_blocks<0, 1, SMAX>(
+                            [&](auto K) { return decltype(K)::value <= commit; },
+                            [&](auto K) {
+                                constexpr int k = decltype(K)::value;
+                                gclk[k * kWave] = cv[k];
+                            });
+                    }
                 }
                 if (want_group && has) {  // :611, :618
                     const uint32_t g = desc_group(sel);
