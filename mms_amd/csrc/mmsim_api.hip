@@ -226,6 +226,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
 
     // ---- per placement: slot layout; per (placement, model): replica count
     int smax = 1, rmax_all = 1, nslots = 1;
+    bool pow2_depths = true;  // every group has 1, 2, 4, 8 or 16 stages
     std::vector<uint8_t> slot0((size_t)B * Gmax, 0);
     for (int32_t p = 0; p < B; ++p) {
         int s = 0;
@@ -236,6 +237,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             slot0[(size_t)p * Gmax + g] = (uint8_t)s;
             s += pp;
             smax = std::max(smax, pp);
+            if ((pp & (pp - 1)) != 0 || pp > 16) pow2_depths = false;
         }
         nslots = std::max(nslots, s);
         for (int32_t m = 0; m < M; ++m)
@@ -547,6 +549,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.rep_extra = RX;
     a.lat_in_lds = lat_in_lds;
     a.uniform_stages = uniform_stages ? 1 : 0;
+    a.pow2_depths = pow2_depths ? 1 : 0;
     a.wave_lds_bytes = (int32_t)wave_bytes;
     a.rmax_lds_bytes = rmax_lds_bytes;
     a.n_seeds = n_seeds;

@@ -60,6 +60,7 @@ struct MixedArgs {
     int32_t n_seeds, B, tiles, nslots, Gmax;
     int32_t lat_in_lds;          // 1: the block keeps a copy of lat in LDS
     int32_t uniform_stages;      // 1: all stages of a (model, config) have the same latency; lat is [M][C]
+    int32_t pow2_depths;         // 1: every group of the batch has 1, 2, 4, 8 or 16 stages
     int32_t wave_lds_bytes;      // LDS bytes of one wavefront's private region
     int32_t rmax_lds_bytes;      // M rounded up to 16
     int64_t Rmax;                // longest stream (row pitch of per-request outputs)

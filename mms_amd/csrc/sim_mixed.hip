@@ -162,6 +162,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const bool want_ops = (a.flags & MMSIM_WANT_OP_COUNT) != 0;
+    const bool pow2 = a.pow2_depths != 0;  // every pipeline depth of the batch is 1, 2, 4, 8 or 16
 
     // ---- LDS: [latency table][per wavefront: request block | replica bounds | clocks | group counters]
     float *lat_lds = reinterpret_cast<float *>(lds_raw);
@@ -323,44 +324,42 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                         // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
                         uint64_t saved_exec;
                         int accepted;
-                        double t, latency;
+                        double latency;
                         const uint32_t cb_addr = lds_addr(gclk);
+#define MMSIM_WALK(NAME, LATNAME, LATVAL)                                                                           \
+    asm volatile(NAME##_TEXT                                                                                        \
+                 : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [fin] "=&v"(finish_time), [lat] "=&v"(latency),   \
+                   [ng] "+v"(n_good), [ls] "+v"(lat_sum)                                                            \
+                 : [walk] "v"(walk), [cb] "v"(cb_addr), [LATNAME] "v"(LATVAL), [ts] "v"(tstamp), [slo] "v"(slo),    \
+                   [oh] "s"(overhead)                                                                               \
+                 : "vcc", "memory", NAME##_CLOBBERS)
                         if constexpr (UNIFORM) {
-                            if constexpr (SMAX == 4)
-                                asm volatile(MMSIM_WALK_U4_TEXT
-                                             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t),
-                                               [fin] "=&v"(finish_time), [lat] "=&v"(latency), [ng] "+v"(n_good),
-                                               [ls] "+v"(lat_sum)
-                                             : [walk] "v"(walk), [cb] "v"(cb_addr), [lc] "v"(l_last), [ts] "v"(tstamp),
-                                               [slo] "v"(slo), [oh] "s"(overhead)
-                                             : "vcc", "memory", MMSIM_WALK_U4_CLOBBERS);
-                            else
-                                asm volatile(MMSIM_WALK_U16_TEXT
-                                             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t),
-                                               [fin] "=&v"(finish_time), [lat] "=&v"(latency), [ng] "+v"(n_good),
-                                               [ls] "+v"(lat_sum)
-                                             : [walk] "v"(walk), [cb] "v"(cb_addr), [lc] "v"(l_last), [ts] "v"(tstamp),
-                                               [slo] "v"(slo), [oh] "s"(overhead)
-                                             : "vcc", "memory", MMSIM_WALK_U16_CLOBBERS);
+                            if (pow2) {
+                                if constexpr (SMAX == 4)
+                                    MMSIM_WALK(MMSIM_WALK_PU4, lc, l_last);
+                                else
+                                    MMSIM_WALK(MMSIM_WALK_PU16, lc, l_last);
+                            } else {
+                                if constexpr (SMAX == 4)
+                                    MMSIM_WALK(MMSIM_WALK_U4, lc, l_last);
+                                else
+                                    MMSIM_WALK(MMSIM_WALK_U16, lc, l_last);
+                            }
                         } else {
                             const uint32_t lb = lds_addr(lrow);
-                            if constexpr (SMAX == 4)
-                                asm volatile(MMSIM_WALK_N4_TEXT
-                                             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t),
-                                               [fin] "=&v"(finish_time), [lat] "=&v"(latency), [ng] "+v"(n_good),
-                                               [ls] "+v"(lat_sum)
-                                             : [walk] "v"(walk), [cb] "v"(cb_addr), [lb] "v"(lb), [ts] "v"(tstamp),
-                                               [slo] "v"(slo), [oh] "s"(overhead)
-                                             : "vcc", "memory", MMSIM_WALK_N4_CLOBBERS);
-                            else
-                                asm volatile(MMSIM_WALK_N16_TEXT
-                                             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [t] "=&v"(t),
-                                               [fin] "=&v"(finish_time), [lat] "=&v"(latency), [ng] "+v"(n_good),
-                                               [ls] "+v"(lat_sum)
-                                             : [walk] "v"(walk), [cb] "v"(cb_addr), [lb] "v"(lb), [ts] "v"(tstamp),
-                                               [slo] "v"(slo), [oh] "s"(overhead)
-                                             : "vcc", "memory", MMSIM_WALK_N16_CLOBBERS);
+                            if (pow2) {
+                                if constexpr (SMAX == 4)
+                                    MMSIM_WALK(MMSIM_WALK_PN4, lb, lb);
+                                else
+                                    MMSIM_WALK(MMSIM_WALK_PN16, lb, lb);
+                            } else {
+                                if constexpr (SMAX == 4)
+                                    MMSIM_WALK(MMSIM_WALK_N4, lb, lb);
+                                else
+                                    MMSIM_WALK(MMSIM_WALK_N16, lb, lb);
+                            }
                         }
+#undef MMSIM_WALK
                         acc = accepted != 0;
                     } else {
                         // ---- the same in plain C++ (other stage buckets, latency table in global memory):

@@ -125,6 +125,54 @@ def test_config4_subsample_counts_and_a_few_full_traces(eng):
     assert_batch_matches(out, ref, 0, packed[0], per_request=True, where="cfg4 traces")
 
 
+@pytest.mark.parametrize("depths", [(1, 2, 4), (1, 2, 4, 8, 16), (1, 2, 3, 4), (1, 3, 5, 8, 11, 16)])
+@pytest.mark.parametrize("uniform", [True, False])
+def test_stage_walk_variants(eng, depths, uniform):
+    """Every hand-scheduled stage walk: depths that are all powers of two or not,
+    one latency per configuration or one per stage, 4- and 16-stage buckets;
+    130 placements of mixed depth so that lanes leave the walk at different levels."""
+    from types import SimpleNamespace
+    from mms_amd.profiling import LatencyMemData, ParallelConfig, ProfilingResult
+    from mms_amd.placement_policy.base_policy import ModelPlacement
+    rng = np.random.default_rng(1000 * len(depths) + 2 * sum(depths) + int(uniform))
+    M, R = 12, 4000
+    pcs = [ParallelConfig(1, 1, d) for d in depths]
+    profiles = []
+    for m in range(M):
+        para = {}
+        for pc in pcs:
+            total = rng.uniform(0.05, 0.3)
+            stages = np.full(pc.pp, total / pc.pp) if uniform else rng.dirichlet(np.ones(pc.pp)) * total
+            para[pc] = LatencyMemData(latency={1: [float(x) for x in stages]}, act_mem={1: [0.0] * pc.pp},
+                                      weight_mem=[1.0] * pc.pp)
+        profiles.append(ProfilingResult(f"m{m}", para_dict=para, preprocess_cpu=0, postprocess_cpu=0))
+    sols = []
+    for _ in range(130):
+        left, cfgs, models = 40, [], []
+        while left > 0:
+            d = int(rng.choice([x for x in depths if x <= left]))
+            left -= d
+            cfgs.append(ParallelConfig(1, 1, d))
+            models.append([int(x) for x in rng.choice(M, size=int(rng.integers(1, 6)), replace=False)])
+        sols.append(ModelPlacement(cfgs, models))
+    gaps = rng.exponential(0.02, size=R)
+    gaps[rng.random(R) < 0.1] = 0.0
+    st = SimpleNamespace(tstamps=np.cumsum(gaps), model_ids=rng.integers(0, M, R).astype(np.int32),
+                         slos=rng.uniform(0.2, 1.0, R).astype(np.float32))
+    table = E.LatencyTable(profiles, [1])
+    packed = E.pack_placements(sols, table)
+    dw = E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, M)
+    batch = E.Batch(eng, [dw], table, packed, ALL)
+    batch.run()
+    batch.sync()
+    out = batch.fetch()
+    assert batch.info()["smax_bucket"] == (4 if max(depths) <= 4 else 16)
+    batch.close()
+    ref = oracle_batch(st, table, packed, want_per_request=True)
+    assert_batch_matches(out, ref, 0, packed[0], per_request=True, where=f"depths {depths} uniform {uniform}")
+    assert 0.05 * R * 130 < ref["n_good"].sum() < 0.98 * R * 130    # both accepts and rejects are exercised
+
+
 def test_scores_only_mode_equals_full_mode(eng):
     cfg = make_config(2)
     a, *_ = _run_config(eng, cfg, cfg.placements, [0, 1], 0)
