@@ -9,6 +9,7 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <new>
@@ -280,16 +281,26 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     int lat_in_lds = 1;
     int wpb = 0;
     int heap_cap = 0;
+    // Wavefronts per workgroup: no more than it takes to give every CU its share of the
+    // batch (a small batch is spread over the CUs, one wavefront per workgroup), and
+    // no more than fit in LDS.  MMSIM_MAX_WAVES_PER_BLOCK lowers the cap (tuning knob).
+    int wpb_cap = kMaxWavesPerBlock;
+    {
+        const int64_t waves_total = (int64_t)b->tiles * n_seeds;
+        const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
+        wpb_cap = (int)std::min<int64_t>(wpb_cap, std::max<int64_t>(1, (waves_total + cus - 1) / cus));
+    }
+    if (const char *env = std::getenv("MMSIM_MAX_WAVES_PER_BLOCK")) wpb_cap = std::max(1, std::min(wpb_cap, std::atoi(env)));
     if (!batching) {
         // shared latency table + per-wavefront private region
         wave_bytes = ((size_t)kStageBytes + rmax_lds_bytes + (size_t)nslots * kWave * sizeof(double) +
                       ((flags & MMSIM_WANT_GROUP_COUNTS) ? (size_t)2 * Gmax * kWave * sizeof(uint32_t) : 0) + 15) & ~(size_t)15;
         const size_t lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
         if (lat_bytes + wave_bytes <= (size_t)ctx->max_lds)
-            wpb = (int)std::min<size_t>(kMaxWavesPerBlock, ((size_t)ctx->max_lds - lat_bytes) / wave_bytes);
+            wpb = (int)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / wave_bytes);
         if (wpb == 0) {
             lat_in_lds = 0;
-            wpb = (int)std::min<size_t>(kMaxWavesPerBlock, (size_t)ctx->max_lds / wave_bytes);
+            wpb = (int)std::min<size_t>(wpb_cap, (size_t)ctx->max_lds / wave_bytes);
         }
         if (wpb == 0) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
         wpb = std::min(wpb, b->tiles);
@@ -304,7 +315,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             if (wave_bytes <= (size_t)ctx->max_lds) break;
         }
         if (heap_cap < Gmax + 4) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: per-wavefront state does not fit in LDS (too many models/stages/groups)");
-        wpb = (int)std::min<size_t>(kMaxWavesPerBlock, (size_t)ctx->max_lds / wave_bytes);
+        wpb = (int)std::min<size_t>(kMaxWavesPerBlockBatching, (size_t)ctx->max_lds / wave_bytes);
         wpb = std::min(wpb, b->tiles);
         b->lds_bytes = (size_t)wpb * wave_bytes;
     }

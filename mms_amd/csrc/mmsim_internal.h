@@ -119,6 +119,7 @@ hipError_t launch_sim_mixed(const MixedArgs &args, int smax_bucket, int waves_pe
                             hipStream_t stream, std::string *err);
 // Smallest compiled stage bucket >= value, or -1.
 int smax_bucket_for(int smax);
-constexpr int kMaxWavesPerBlock = 4;
+constexpr int kMaxWavesPerBlock = 8;          // plain simulator
+constexpr int kMaxWavesPerBlockBatching = 4;  // batching simulator
 
 }  // namespace mmsim

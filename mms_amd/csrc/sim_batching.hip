@@ -38,7 +38,7 @@ __device__ __forceinline__ int uniform_i(int v) { return __builtin_amdgcn_readfi
 __device__ __forceinline__ double dmax(double a, double b) { return b > a ? b : a; }
 __device__ __forceinline__ int ilog2i(int v) { return 31 - __clz(v); }
 
-__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_batching_kernel(const BatchingArgs a) {
+__global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching_kernel(const BatchingArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
     const int W = (int)(blockDim.x >> 6);
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_batching_kernel(
 hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_bytes, hipStream_t stream,
                                std::string *err) {
     hipError_t e = hipSuccess;
-    if (wpb < 1 || wpb > kMaxWavesPerBlock) {
+    if (wpb < 1 || wpb > kMaxWavesPerBlockBatching) {
         e = hipErrorInvalidValue;
     } else {
         auto kern = sim_batching_kernel;

@@ -236,3 +236,25 @@ def test_synthetic_configs_are_deterministic_and_as_specified():
     st = c2a.stream(1)
     assert np.array_equal(w.arrivals, st.tstamps)
     assert [r.model_name for r in w.requests] == [f"m{m}" for m in st.model_ids]
+
+
+def test_alpa_serve_import_names_resolve_to_this_package():
+    import importlib
+    import sys
+    import mms_amd.compat as compat
+    compat.install()
+    try:
+        pp = importlib.import_module("alpa_serve.placement_policy")
+        ctl = importlib.import_module("alpa_serve.simulator.controller")
+        wl = importlib.import_module("alpa_serve.simulator.workload")
+        for name in ("ModelData", "ClusterEnv", "ModelParallelismGreedy", "ModelParallelismSearch",
+                     "SelectiveReplicationGreedy", "SelectiveReplicationSearch", "ModelParallelismILP"):
+            assert hasattr(pp, name), name
+        assert ctl.approximate_one_case.__module__ == "mms_amd.simulator.controller"
+        assert wl.Workload.__module__ == "mms_amd.simulator.workload"
+        from alpa_serve.placement_policy.base_policy import ModelPlacement, PlacementEvaluator  # noqa: F401
+        from alpa_serve.profiling import ParallelConfig, ProfilingResult  # noqa: F401
+        from alpa_serve.util import ServingCase, GB  # noqa: F401
+    finally:
+        for k in [k for k in sys.modules if k == "alpa_serve" or k.startswith("alpa_serve.")]:
+            del sys.modules[k]
