@@ -109,7 +109,8 @@ struct mmsim_batch {
     DevBuf<uint32_t> rep32, repx32;
     DevBuf<uint64_t> rep8;
     DevBuf<uint8_t> repx;
-    DevBuf<uint8_t> rmax;
+    DevBuf<uint8_t> rmax, slot_group;
+    DevBuf<int32_t> kerr;
     DevBuf<uint32_t> ginfo;
     DevBuf<float> lat;
     DevBuf<int32_t> n_good;
@@ -142,6 +143,7 @@ namespace {
 int check_tables(const mmsim_tables *t) {
     if (!t || !t->cfg_lat || !t->cfg_pp) return fail(MMSIM_E_INVALID, "tables: null pointer");
     if (t->M < 1 || t->C < 1 || t->Smax < 1 || t->NB < 1) return fail(MMSIM_E_INVALID, "tables: M, C, Smax, NB must be >= 1");
+    if (t->M > 0xFFFFFF) return fail(MMSIM_E_UNSUPPORTED, "more than 16777215 models");
     if (t->C > 255) return fail(MMSIM_E_UNSUPPORTED, "tables: more than 255 parallel configurations");
     if (t->Smax > MMSIM_MAX_STAGES) return fail(MMSIM_E_UNSUPPORTED, "tables: more than 32 pipeline stages");
     for (int c = 0; c < t->C; ++c)
@@ -277,7 +279,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
 
     // ---- LDS budget
     const int32_t rmax_lds_bytes = (M + 15) & ~15;
-    size_t wave_bytes = 0;
+    size_t wave_bytes = 0, lat_bytes = 0;
     int lat_in_lds = 1;
     int wpb = 0;
     int heap_cap = 0;
@@ -293,9 +295,12 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     if (const char *env = std::getenv("MMSIM_MAX_WAVES_PER_BLOCK")) wpb_cap = std::max(1, std::min(wpb_cap, std::atoi(env)));
     if (!batching) {
         // shared latency table + per-wavefront private region
-        wave_bytes = ((size_t)kStageBytes + rmax_lds_bytes + (size_t)nslots * kWave * sizeof(double) +
-                      ((flags & MMSIM_WANT_GROUP_COUNTS) ? (size_t)2 * Gmax * kWave * sizeof(uint32_t) : 0) + 15) & ~(size_t)15;
-        const size_t lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
+        // request block | replica bounds | clocks (one extra row that stays +inf) | slot owners | group counters
+        wave_bytes = ((size_t)mixed_clock_offset(rmax_lds_bytes) + (size_t)(nslots + 1) * kSlotBytes +
+                      ((flags & MMSIM_WANT_GROUP_COUNTS)
+                           ? (((size_t)nslots * kWave + 15) & ~(size_t)15) + (size_t)2 * Gmax * kWave * sizeof(uint32_t)
+                           : 0) + 15) & ~(size_t)15;
+        lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
         if (lat_bytes + wave_bytes <= (size_t)ctx->max_lds)
             wpb = (int)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / wave_bytes);
         if (wpb == 0) {
@@ -304,7 +309,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
         if (wpb == 0) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
         wpb = std::min(wpb, b->tiles);
-        b->lds_bytes = (lat_in_lds ? lat_bytes : 0) + (size_t)wpb * wave_bytes;
+        if (!lat_in_lds) lat_bytes = 0;
+        b->lds_bytes = lat_bytes + (size_t)wpb * wave_bytes;
+        if (b->lds_bytes > (size_t)kRepAddrMask) return fail(MMSIM_E_UNSUPPORTED, "LDS layout exceeds the descriptor's address field");
     } else {
         // per wavefront: descriptors | clocks | event times | queue heads | event groups | arrivals per model.
         // Events: the reference's heap holds about one entry per group plus a few stale ones;
@@ -378,8 +385,39 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         rep8.assign((size_t)b->tiles * M * kWave, none8);
         repx.assign((size_t)b->tiles * M * RX * kWave, (uint8_t)Gmax);
     } else {
-        rep32.assign((size_t)b->tiles * M * 2 * kWave * 4, kEmpty);
-        repx32.assign((size_t)b->tiles * M * RX * kWave, kEmpty);
+        rep32.resize((size_t)b->tiles * M * 2 * kWave * 4);
+        repx32.resize((size_t)b->tiles * M * RX * kWave);
+    }
+    // LDS byte address of clock slot `slot` of the lane that simulates position `ps` (plain simulator);
+    // slot == nslots is the lane's +inf clock.
+    auto clock_addr = [&](int ps, int slot) {
+        const int wv = (ps / kWave) % wpb, lane = ps % kWave;
+        return (uint32_t)(lat_bytes + (size_t)wv * wave_bytes + mixed_clock_offset(rmax_lds_bytes) + (size_t)slot * kSlotBytes +
+                          (size_t)lane * sizeof(double));
+    };
+    if (!batching) {  // missing replicas: the +inf clock, flagged empty
+        for (size_t i = 0; i < rep32.size(); ++i) {
+            const int lane = (int)((i / 4) % kWave);
+            const int tile = (int)(i / ((size_t)M * 2 * kWave * 4));
+            rep32[i] = kEmpty | clock_addr(tile * kWave + lane, nslots);
+        }
+        for (size_t i = 0; i < repx32.size(); ++i) {
+            const int lane = (int)(i % kWave);
+            const int tile = (int)(i / ((size_t)M * RX * kWave));
+            repx32[i] = kEmpty | clock_addr(tile * kWave + lane, nslots);
+        }
+    }
+    std::vector<uint8_t> slot_group;
+    if (!batching && (flags & MMSIM_WANT_GROUP_COUNTS)) {
+        slot_group.assign((size_t)b->tiles * nslots * kWave, 0);
+        for (int32_t p = 0; p < B; ++p) {
+            const int tile = b->pos[p] / kWave, lane = b->pos[p] % kWave;
+            for (int32_t g = 0; g < rl.num_groups[p]; ++g) {
+                const int pp = t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]];
+                for (int k = 0; k < pp; ++k)
+                    slot_group[((size_t)tile * nslots + slot0[(size_t)p * Gmax + g] + k) * kWave + lane] = (uint8_t)g;
+            }
+        }
     }
     std::vector<uint8_t> rmax((size_t)b->tiles * M, 0);
     for (int32_t p = 0; p < B; ++p) {
@@ -398,7 +436,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                     else
                         repx[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = (uint8_t)g;
                 } else {
-                    const uint32_t d = ginfo[((size_t)tile * (Gmax + 1) + g) * kWave + lane];
+                    const int32_t c = rl.group_cfg[(size_t)p * Gmax + g];
+                    const int pp = t->cfg_pp[c];
+                    const uint32_t d = pack_rep(clock_addr(b->pos[p], slot0[(size_t)p * Gmax + g] + pp - 1), (uint32_t)pp,
+                                                (uint32_t)(lat_off[c] + (uniform_stages ? 0 : pp - 1)));
                     if (j < kPackedReplicas)  // word j/4 of the lane, component j%4
                         rep32[((((size_t)tile * M + m) * 2 + (size_t)(j / 4)) * kWave + lane) * 4 + (size_t)(j % 4)] = d;
                     else
@@ -494,6 +535,12 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (!repx32.empty())
             HIP_TRY(hipMemcpyAsync(b->repx32.p, repx32.data(), sizeof(uint32_t) * repx32.size(), hipMemcpyHostToDevice, st));
     }
+    if (!slot_group.empty()) {
+        HIP_TRY(b->slot_group.alloc(slot_group.size()));
+        HIP_TRY(hipMemcpyAsync(b->slot_group.p, slot_group.data(), slot_group.size(), hipMemcpyHostToDevice, st));
+    }
+    HIP_TRY(b->kerr.alloc(1));
+    HIP_TRY(hipMemsetAsync(b->kerr.p, 0, sizeof(int32_t), st));
     HIP_TRY(b->rmax.alloc(rmax.size()));
     HIP_TRY(hipMemcpyAsync(b->rmax.p, rmax.data(), rmax.size(), hipMemcpyHostToDevice, st));
     HIP_TRY(b->lat.alloc(lat.size()));
@@ -554,6 +601,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.rep32 = reinterpret_cast<const uint4 *>(b->rep32.p);
     a.repx32 = b->repx32.p;
     a.rmax = b->rmax.p;
+    a.slot_group = b->slot_group.p;
+    a.lat_lds_bytes = (int32_t)lat_bytes;
+    a.error = b->kerr.p;
     a.lat = b->lat.p;
     a.M = M;
     a.lat_row = lat_row;
@@ -792,6 +842,11 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
     HIP_TRY(hipSetDevice(b->ctx->device));
     HIP_TRY(hipStreamSynchronize(b->ctx->stream));
 
+    if (!(b->flags & MMSIM_BATCHING)) {
+        int32_t kerr = 0;
+        HIP_TRY(hipMemcpy(&kerr, b->kerr.p, sizeof(int32_t), hipMemcpyDeviceToHost));
+        if (kerr != 0) return fail(MMSIM_E_HIP, "simulation kernel: dynamic LDS does not start at address 0; results are invalid");
+    }
     const int32_t B = b->B, M = b->M, Gmax = b->Gmax, tiles = b->tiles;
     const size_t lanes_padded = (size_t)b->waves * kWave;
     std::vector<int32_t> ng(lanes_padded);

@@ -20,9 +20,8 @@ struct __attribute__((aligned(16))) Req {
 };
 static_assert(sizeof(Req) == 16, "Req must be 16 bytes");
 
-// Group descriptor: one 32-bit word per (placement, group).  The plain simulator
-// reads a model's replicas as descriptors; the batching simulator keeps a per
-// lane table of them in LDS and lists replicas as group indices.
+// Group descriptor of the batching simulator: one 32-bit word per (placement,
+// group), kept per lane in LDS; replicas are listed as group indices.
 //   bits  0..7   clock slot of the group's LAST pipeline stage (slots are the
 //                placement's pipeline stages laid end to end)
 //   bits  8..12  stages of the group minus one
@@ -42,6 +41,29 @@ __host__ __device__ inline uint32_t desc_last_slot(uint32_t d) { return d & 0xFF
 __host__ __device__ inline uint32_t desc_stages_m1(uint32_t d) { return (d >> 8) & 0x1Fu; }
 __host__ __device__ inline uint32_t desc_lat_off(uint32_t d) { return (d >> 13) & 0x3FFu; }
 __host__ __device__ inline uint32_t desc_group(uint32_t d) { return (d >> 23) & 0xFFu; }
+
+// Replica descriptor of the plain simulator: one 32-bit word per (tile, model,
+// replica, lane), made for the lane that reads it, so that the hot loop gets
+// its LDS addresses with one AND:
+//   bits  3..17  LDS byte address (relative to the workgroup's dynamic LDS,
+//                8-byte aligned, so bits 0..2 are free) of the clock of the
+//                group's LAST stage, for this lane
+//   bits  0..2   stages - 1, low three bits
+//   bits 28..29  stages - 1, high two bits
+//   bits 18..27  index of the group's LAST-stage latency in the model's row of
+//                the compact latency table
+//   bit  31      "no such replica"; the address then names the lane's clock
+//                that is +inf forever, so it never wins the choice
+constexpr uint32_t kRepAddrMask = 0x3FFF8u;
+__host__ __device__ inline uint32_t pack_rep(uint32_t last_clock_addr, uint32_t stages, uint32_t lat_last) {
+    const uint32_t sm1 = stages - 1u;
+    return last_clock_addr | (sm1 & 7u) | ((sm1 >> 3) << 28) | (lat_last << 18);
+}
+__host__ __device__ inline uint32_t rep_addr(uint32_t d) { return d & kRepAddrMask; }
+__host__ __device__ inline uint32_t rep_stages_m1(uint32_t d) { return (d & 7u) | ((d >> 25) & 0x18u); }
+__host__ __device__ inline uint32_t rep_lat_last(uint32_t d) { return (d >> 18) & 0x3FFu; }
+constexpr int kSlotBytes = 64 * 8;  // one clock slot: 64 lanes x f64
+
 constexpr int kMaxLatRow = 1023;  // floats per model in the compact latency table
 constexpr int kPackedReplicas = 8;
 
@@ -55,12 +77,14 @@ struct MixedArgs {
     const uint4 *rep32;          // [tiles][M][2][64] descriptors of the first 8 replicas, four to a 16-byte word
     const uint32_t *repx32;      // [tiles][M][rep_extra][64] descriptors of replicas 8, 9, ...
     const uint8_t *rmax;         // [tiles][M] most replicas of model m over the tile's lanes
+    const uint8_t *slot_group;   // [tiles][nslots][64] group that owns each clock slot (only with group counters)
     const float *lat;            // [M][lat_row] compact stage latencies (batch size 1)
     int32_t M, lat_row, rep_extra;
     int32_t n_seeds, B, tiles, nslots, Gmax;
     int32_t lat_in_lds;          // 1: the block keeps a copy of lat in LDS
     int32_t uniform_stages;      // 1: all stages of a (model, config) have the same latency; lat is [M][C]
     int32_t pow2_depths;         // 1: every group of the batch has 1, 2, 4, 8 or 16 stages
+    int32_t lat_lds_bytes;       // LDS bytes of the shared latency table (0 if it stays in global memory)
     int32_t wave_lds_bytes;      // LDS bytes of one wavefront's private region
     int32_t rmax_lds_bytes;      // M rounded up to 16
     int64_t Rmax;                // longest stream (row pitch of per-request outputs)
@@ -75,7 +99,17 @@ struct MixedArgs {
     double *finish;              // [waves][Rmax][64]
     uint8_t *good;               // [waves][Rmax][64]
     int64_t *fp_ops;             // [n_seeds][tiles*64]
+    int32_t *error;              // set to 1 if the kernel finds its LDS layout assumption broken
 };
+
+// LDS layout of the plain simulator, shared by the kernel and by the host code
+// that bakes LDS addresses into the replica descriptors:
+//   [latency table][wavefront 0][wavefront 1]...
+//   wavefront: [64 staged requests][replica bounds][clocks: nslots+1 rows of 64 f64][slot owners][group counters]
+// Row nslots of the clocks is the +inf row that empty descriptors point at.
+__host__ __device__ inline uint32_t mixed_clock_offset(int32_t rmax_lds_bytes) {
+    return (uint32_t)(kStageBytes + rmax_lds_bytes);
+}
 
 // Arguments of the batching simulation kernel.  Replica lists and group
 // descriptors are shared with the plain kernel; on top come, per seed, the

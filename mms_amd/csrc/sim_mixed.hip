@@ -12,14 +12,16 @@
 //   * requests are fetched 64 at a time with one coalesced 1 KiB load per
 //     wavefront (one block ahead, into registers), parked in LDS and read
 //     back with broadcast LDS reads;
-//   * the replicas of the request's model are 32-bit descriptors (last-stage
-//     clock slot, stage count, latency-row offset, group index), eight per
-//     (tile, model, lane) in two 16-byte words rep32[tile][model][2][lane]
-//     (two coalesced 1 KiB loads per request, listed in the order the
-//     reference scans them).  They are fetched one chunk of requests ahead
-//     into registers together with the request's arrival time and SLO; the
-//     load count per chunk is fixed so the wait counters let the prefetch
-//     overlap the current chunk;
+//   * the replicas of the request's model are 32-bit descriptors made for the
+//     lane that reads them (LDS address of the group's last-stage clock,
+//     stage count, index of its last-stage latency), eight per (tile, model,
+//     lane) in two 16-byte words rep32[tile][model][2][lane] (two coalesced
+//     1 KiB loads per request, listed in the order the reference scans them).
+//     Missing replicas point at a clock that is +inf forever, so the scan
+//     needs no validity test.  Descriptors are fetched one chunk of requests
+//     ahead into registers together with the request's arrival time and SLO;
+//     the load count per chunk is fixed so the wait counters let the
+//     prefetch overlap the current chunk;
 //   * per-lane stage clocks live in LDS as clk[slot][lane] (8 bytes each);
 //     the slots of a lane are its groups' pipeline stages laid end to end.
 //     The bank an access hits depends on the lane only, so any per-lane
@@ -71,6 +73,12 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 __device__ __forceinline__ double vmax(double x, double y) {
     double r;
     asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y));
+    return r;
+}
+
+__device__ __forceinline__ double vmin(double x, double y) {
+    double r;
+    asm("v_min_f64 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y));
     return r;
 }
 
@@ -164,16 +172,22 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const bool want_ops = (a.flags & MMSIM_WANT_OP_COUNT) != 0;
     const bool pow2 = a.pow2_depths != 0;  // every pipeline depth of the batch is 1, 2, 4, 8 or 16
 
-    // ---- LDS: [latency table][per wavefront: request block | replica bounds | clocks | group counters]
+    // ---- LDS: [latency table][per wavefront: request block | replica bounds | clocks (+inf row last) |
+    //            slot owners | group counters].  The replica descriptors hold byte offsets into lds_raw.
+    if (lds_addr(lds_raw) != 0u) {  // the descriptors assume the dynamic LDS starts at address 0
+        if (threadIdx.x == 0) *a.error = 1;
+        return;
+    }
     float *lat_lds = reinterpret_cast<float *>(lds_raw);
     const int lat_floats = LATLDS ? a.M * a.lat_row : 0;
-    const int lat_bytes = (lat_floats * 4 + 15) & ~15;
-    unsigned char *mine = lds_raw + lat_bytes + wv * a.wave_lds_bytes;
-    Req *stage = reinterpret_cast<Req *>(mine);
+    unsigned char *mine = lds_raw + a.lat_lds_bytes + wv * a.wave_lds_bytes;
     int4 *stage4 = reinterpret_cast<int4 *>(mine);
     uint8_t *rmax_lds = mine + kStageBytes;
-    double *clk = reinterpret_cast<double *>(mine + kStageBytes + a.rmax_lds_bytes) + lane;
-    uint32_t *gcnt = reinterpret_cast<uint32_t *>(mine + kStageBytes + a.rmax_lds_bytes + a.nslots * (kWave * 8)) + lane;
+    const uint32_t clk_off = (uint32_t)(a.lat_lds_bytes + wv * a.wave_lds_bytes) + mixed_clock_offset(a.rmax_lds_bytes);
+    double *clk = reinterpret_cast<double *>(lds_raw + clk_off) + lane;
+    const int own_bytes = want_group ? ((a.nslots * kWave + 15) & ~15) : 0;
+    uint8_t *owner = lds_raw + clk_off + (a.nslots + 1) * kSlotBytes;  // owner[slot * 64 + lane]
+    uint32_t *gcnt = reinterpret_cast<uint32_t *>(owner + own_bytes) + lane;
 
     for (int i = (int)threadIdx.x; i < lat_floats; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
     if (live)
@@ -182,8 +196,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     if (!live) return;  // padding wavefront of the last workgroup
 
     for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
-    if (want_group)
+    clk[a.nslots * kWave] = __builtin_inf();
+    if (want_group) {
+        for (int s = 0; s < a.nslots; ++s) owner[s * kWave + lane] = a.slot_group[((size_t)tile * a.nslots + s) * kWave + lane];
         for (int g = 0; g < 2 * a.Gmax; ++g) gcnt[g * kWave] = 0u;
+    }
 
     const int wave = seed * a.tiles + tile;
     const int64_t off = a.stream_off[seed];
@@ -205,7 +222,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     if (R > 0) ahead = reqs4[lane < R ? lane : R - 1];
 
     for (int64_t blk = 0; blk < R; blk += kWave) {
-        stage4[lane] = ahead;
+        {   // park this block's requests; the model word also carries the tile's replica bound
+            int4 r = ahead;
+            const bool ok = blk + lane < R && r.z >= 0;
+            const int bound = (int)rmax_lds[ok ? r.z : 0];
+            r.z = ok ? (r.z | (bound << 24)) : -1;
+            stage4[lane] = r;
+        }
         {
             const int64_t nx = blk + kWave + lane;
             ahead = reqs4[nx < R ? nx : R - 1];
@@ -214,16 +237,21 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
 
         // Always 2*CH loads per chunk, whatever the requests are.
         auto load_chunk = [&](Chunk<CH> &c, int cb) {
+            int4 r[CH];
             static_while<0, CH>([&](auto U) {
                 constexpr int u = decltype(U)::value;
-                const int idx = cb + u;  // < 64
-                const Req r = stage[idx];  // broadcast read
-                const int m = uniform(r.m);
-                const bool ok = idx < nblk && m >= 0;
+                r[u] = stage4[cb + u];  // broadcast read; cb + u < 64
+                return true;
+            });
+            static_while<0, CH>([&](auto U) {
+                constexpr int u = decltype(U)::value;
+                const int w = uniform(r[u].z);
+                const bool ok = w >= 0;
+                const int m = ok ? (w & 0xFFFFFF) : -1;
                 c.m[u] = m;
-                c.nrep[u] = ok ? uniform((int)rmax_lds[ok ? m : 0]) : 0;
-                c.t[u] = r.t;
-                c.slo[u] = r.slo;
+                c.nrep[u] = ok ? (w >> 24) : 0;
+                c.t[u] = __hiloint2double(r[u].y, r[u].x);
+                c.slo[u] = __int_as_float(r[u].w);
                 const uint4 *row = rep_tile + (size_t)(ok ? m : 0) * (2 * kWave);
                 c.da[u] = row[0];
                 c.db[u] = row[kWave];
@@ -252,18 +280,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 double best = 1e100;
                 uint32_t sel = kEmpty;
                 float lsel = 0.0f;
-                int nvalid = 0;
-                auto lat_index = [&](uint32_t d) { return desc_lat_off(d) + (UNIFORM ? 0u : desc_stages_m1(d)); };
                 auto consider = [&](uint32_t d, double c, float l) {
-                    const bool valid = (int32_t)d >= 0;
-                    const bool better = valid && c < best;
-                    best = better ? c : best;
+                    const bool better = c < best;  // empty entries read a clock that is +inf
+                    best = vmin(best, c);
                     sel = better ? d : sel;
                     lsel = better ? l : lsel;
-                    if (want_ops) nvalid += valid ? 1 : 0;
                 };
                 // Scan 4 or 8 list entries without branching: entries past a lane's own
-                // replicas are empty descriptors, whose reads are harmless and ignored.
+                // replicas are empty descriptors, whose reads are harmless and never win.
                 auto scan = [&](auto NJ) {
                     constexpr int nj = decltype(NJ)::value;
                     double cl[nj];
@@ -271,8 +295,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     static_while<0, nj>([&](auto J) {
                         constexpr int j = decltype(J)::value;
                         const uint32_t d = pick_desc<j>(cur.da[u], cur.db[u]);
-                        cl[j] = clk[desc_last_slot(d) * kWave];
-                        ll[j] = lrow_m[lat_index(d)];
+                        cl[j] = *reinterpret_cast<const double *>(lds_raw + rep_addr(d));
+                        ll[j] = lrow_m[rep_lat_last(d)];
                         return true;
                     });
                     static_while<0, nj>([&](auto J) {
@@ -289,15 +313,15 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
                     for (int j = RREG; j < n; ++j) {
                         const uint32_t d = row[(size_t)(j - RREG) * kWave];
-                        consider(d, clk[desc_last_slot(d) * kWave], lrow_m[lat_index(d)]);
+                        consider(d, *reinterpret_cast<const double *>(lds_raw + rep_addr(d)), lrow_m[rep_lat_last(d)]);
                     }
                 }
 
                 const bool has = (int32_t)sel >= 0;
-                const int sm1 = has ? (int)desc_stages_m1(sel) : -1;  // stages - 1
-                const uint32_t slot0 = has ? desc_last_slot(sel) - (uint32_t)sm1 : 0u;
-                double *gclk = clk + slot0 * kWave;
-                const float *lrow = lrow_m + (has ? desc_lat_off(sel) : 0u);
+                const int sm1 = has ? (int)rep_stages_m1(sel) : -1;  // stages - 1
+                const uint32_t last_addr = rep_addr(sel);            // the lane's +inf clock when there is no replica
+                const uint32_t first_addr = last_addr - (uint32_t)(has ? sm1 : 0) * kSlotBytes;
+                const float *lrow = lrow_m + (has ? (int)rep_lat_last(sel) - sm1 : 0);
                 const double l_last = (double)lsel;
 
                 double finish_time;
@@ -309,7 +333,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     const double latency = finish_time - tstamp;
                     acc = has && latency <= slo;
                     if (acc) {
-                        gclk[0] = t;
+                        *reinterpret_cast<double *>(lds_raw + last_addr) = t;
                         n_good += 1;
                         lat_sum += latency;
                     }
@@ -325,7 +349,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                         uint64_t saved_exec;
                         int accepted;
                         double latency;
-                        const uint32_t cb_addr = lds_addr(gclk);
+                        const uint32_t cb_addr = first_addr;
 #define MMSIM_WALK(NAME, LATNAME, LATVAL)                                                                           \
     asm volatile(NAME##_TEXT                                                                                        \
                  : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [fin] "=&v"(finish_time), [lat] "=&v"(latency),   \
@@ -364,6 +388,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     } else {
                         // ---- the same in plain C++ (other stage buckets, latency table in global memory):
                         //      fetch, then the dependent chain (:605-608)
+                        double *gclk = reinterpret_cast<double *>(lds_raw + first_addr);
                         double cv[SMAX];
                         float lv[SMAX];
                         walk_blocks<0, 1, SMAX>(
@@ -398,11 +423,24 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     }
                 }
                 if (want_group && has) {  // :611, :618
-                    const uint32_t g = desc_group(sel);
+                    const uint32_t g = owner[(last_addr - clk_off) >> 3];  // (slot * 512 + lane * 8) / 8
                     gcnt[g * kWave] += 1u;
                     if (acc) gcnt[(a.Gmax + g) * kWave] += 1u;
                 }
-                if (want_ops && has) fp_ops += 2 * (sm1 + 1) + nvalid + 3;
+                if (want_ops) {
+                    asm volatile("" ::: "memory");  // keep this a wave-uniform branch, off the common path
+                    int nvalid = 0;
+                    static_while<0, RREG>([&](auto J) {
+                        constexpr int j = decltype(J)::value;
+                        nvalid += (j < n && (int32_t)pick_desc<j>(cur.da[u], cur.db[u]) >= 0) ? 1 : 0;
+                        return true;
+                    });
+                    if (n > RREG) {
+                        const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
+                        for (int j = RREG; j < n; ++j) nvalid += (int32_t)row[(size_t)(j - RREG) * kWave] >= 0 ? 1 : 0;
+                    }
+                    if (has) fp_ops += 2 * (sm1 + 1) + nvalid + 3;
+                }
                 if (want_model && m >= 0) model_good[(size_t)m * kWave] += acc ? 1 : 0;
                 if (want_req) {
                     fin_out[(blk + cb + u) * kWave] = acc ? finish_time : tstamp;
