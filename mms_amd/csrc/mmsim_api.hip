@@ -11,6 +11,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <limits>
 #include <memory>
 #include <new>
 
@@ -61,11 +62,15 @@ struct DevBuf {
 
 }  // namespace
 
+constexpr int kSideStreams = 4;
+
 struct mmsim_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     hipDeviceProp_t prop{};
     int max_lds = 0;
+    hipStream_t side[kSideStreams] = {};  // tile classes of one batch run side by side on these
+    hipEvent_t ev_fork = nullptr, ev_join[kSideStreams] = {};
 };
 
 struct mmsim_workload {
@@ -103,6 +108,16 @@ struct mmsim_batch {
     int64_t Rmax = 0, Rtotal = 0;
     std::vector<const mmsim_workload *> wl;
     std::vector<int32_t> pos;  // pos[placement] = tile * 64 + lane it is simulated on
+    // Plain simulator: tiles are grouped into classes by how many clock slots they need; a class is
+    // launched with its own LDS size and as many wavefronts per workgroup as then fit a CU.
+    struct TileClass {
+        int32_t tile0 = 0, tile1 = 0, nslots = 0, wpb = 1;
+        size_t wave_bytes = 0, lds_bytes = 0;
+    };
+    std::vector<TileClass> classes;
+    int32_t nseg = 1;          // streams are simulated in nseg launches per class, state kept in `state`
+    DevBuf<double> state;
+    int32_t launches = 0;      // kernel launches of one run
 
     DevBuf<Req> streams;
     DevBuf<int64_t> stream_off;
@@ -223,14 +238,13 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     b->B = B;
     b->M = M;
     b->Gmax = Gmax;
-    b->tiles = (B + kWave - 1) / kWave;
-    b->waves = b->tiles * n_seeds;
     b->wl.assign(wls, wls + n_seeds);
 
     // ---- per placement: slot layout; per (placement, model): replica count
     int smax = 1, rmax_all = 1, nslots = 1;
     bool pow2_depths = true;  // every group has 1, 2, 4, 8 or 16 stages
     std::vector<uint8_t> slot0((size_t)B * Gmax, 0);
+    std::vector<int32_t> slots_of(B, 0);  // clock slots placement p needs
     for (int32_t p = 0; p < B; ++p) {
         int s = 0;
         for (int32_t g = 0; g < rl.num_groups[p]; ++g) {
@@ -243,6 +257,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             if ((pp & (pp - 1)) != 0 || pp > 16) pow2_depths = false;
         }
         nslots = std::max(nslots, s);
+        slots_of[p] = std::max(s, 1);
         for (int32_t m = 0; m < M; ++m)
             rmax_all = std::max<int64_t>(rmax_all, rl.off[(size_t)p * M + m + 1] - rl.off[(size_t)p * M + m]);
     }
@@ -265,9 +280,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
     std::vector<int32_t> lat_off(C + 1, 0);
     for (int c = 0; c < C; ++c) lat_off[c + 1] = lat_off[c] + (uniform_stages ? 1 : t->cfg_pp[c]);
-    const int32_t lat_row = lat_off[C];
-    if (lat_row > kMaxLatRow) return fail(MMSIM_E_UNSUPPORTED, "configurations have more than 1023 pipeline stages in total");
-    std::vector<float> lat((size_t)M * lat_row);
+    const int32_t lat_row = lat_off[C] + 1;  // one extra entry per model: +inf, the latency of "no such replica"
+    if (lat_row > kMaxLatRow) return fail(MMSIM_E_UNSUPPORTED, "configurations have more than 1022 pipeline stages in total");
+    std::vector<float> lat((size_t)M * lat_row, std::numeric_limits<float>::infinity());
     for (int32_t m = 0; m < M; ++m)
         for (int c = 0; c < C; ++c)
             for (int k = 0; k < (uniform_stages ? 1 : t->cfg_pp[c]); ++k) {
@@ -285,33 +300,31 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     int heap_cap = 0;
     // Wavefronts per workgroup: no more than it takes to give every CU its share of the
     // batch (a small batch is spread over the CUs, one wavefront per workgroup), and
-    // no more than fit in LDS.  MMSIM_MAX_WAVES_PER_BLOCK lowers the cap (tuning knob).
+    // no more than fit in LDS.  MMSIM_WAVES_PER_CU (1..8) sets the number instead (tuning knob).
     int wpb_cap = kMaxWavesPerBlock;
     {
-        const int64_t waves_total = (int64_t)b->tiles * n_seeds;
+        const int64_t waves_total = (int64_t)((B + kWave - 1) / kWave) * n_seeds;
         const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
         wpb_cap = (int)std::min<int64_t>(wpb_cap, std::max<int64_t>(1, (waves_total + cus - 1) / cus));
     }
-    if (const char *env = std::getenv("MMSIM_MAX_WAVES_PER_BLOCK")) wpb_cap = std::max(1, std::min(wpb_cap, std::atoi(env)));
+    if (const char *env = std::getenv("MMSIM_WAVES_PER_CU")) wpb_cap = std::max(1, std::min(kMaxWavesPerBlock, std::atoi(env)));
+    // plain simulator, per wavefront: request block | replica bounds | clocks (one extra row that stays +inf)
+    // | slot owners | group counters; the latency table is shared by the workgroup
+    auto mixed_wave_bytes = [&](int ns) {
+        return ((size_t)mixed_clock_offset(rmax_lds_bytes) + (size_t)(ns + 1) * kSlotBytes +
+                ((flags & MMSIM_WANT_GROUP_COUNTS)
+                     ? (((size_t)ns * kWave + 15) & ~(size_t)15) + (size_t)2 * Gmax * kWave * sizeof(uint32_t)
+                     : 0) + 15) & ~(size_t)15;
+    };
     if (!batching) {
-        // shared latency table + per-wavefront private region
-        // request block | replica bounds | clocks (one extra row that stays +inf) | slot owners | group counters
-        wave_bytes = ((size_t)mixed_clock_offset(rmax_lds_bytes) + (size_t)(nslots + 1) * kSlotBytes +
-                      ((flags & MMSIM_WANT_GROUP_COUNTS)
-                           ? (((size_t)nslots * kWave + 15) & ~(size_t)15) + (size_t)2 * Gmax * kWave * sizeof(uint32_t)
-                           : 0) + 15) & ~(size_t)15;
+        wave_bytes = mixed_wave_bytes(nslots);  // of the largest placement
         lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
-        if (lat_bytes + wave_bytes <= (size_t)ctx->max_lds)
-            wpb = (int)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / wave_bytes);
-        if (wpb == 0) {
+        if (lat_bytes + wave_bytes > (size_t)ctx->max_lds) {
             lat_in_lds = 0;
-            wpb = (int)std::min<size_t>(wpb_cap, (size_t)ctx->max_lds / wave_bytes);
+            lat_bytes = 0;
         }
-        if (wpb == 0) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
-        wpb = std::min(wpb, b->tiles);
-        if (!lat_in_lds) lat_bytes = 0;
-        b->lds_bytes = lat_bytes + (size_t)wpb * wave_bytes;
-        if (b->lds_bytes > (size_t)kRepAddrMask) return fail(MMSIM_E_UNSUPPORTED, "LDS layout exceeds the descriptor's address field");
+        if (wave_bytes > (size_t)ctx->max_lds) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
+        if ((size_t)ctx->max_lds > (size_t)kRepAddrMask) return fail(MMSIM_E_UNSUPPORTED, "LDS is larger than the descriptor's address field");
     } else {
         // per wavefront: descriptors | clocks | event times | queue heads | event groups | arrivals per model.
         // Events: the reference's heap holds about one entry per group plus a few stale ones;
@@ -323,10 +336,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
         if (heap_cap < Gmax + 4) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: per-wavefront state does not fit in LDS (too many models/stages/groups)");
         wpb = (int)std::min<size_t>(kMaxWavesPerBlockBatching, (size_t)ctx->max_lds / wave_bytes);
-        wpb = std::min(wpb, b->tiles);
-        b->lds_bytes = (size_t)wpb * wave_bytes;
     }
-    b->waves_per_block = wpb;
 
     // ---- lane assignment.  A wavefront walks as many pipeline stages as its deepest
     //      lane needs, so placements are ordered by depth before they are cut into
@@ -352,14 +362,65 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 expected[p] += weight[m] * depth_of[m];
             }
         }
+        // Plain simulator: a placement's clock slots decide how many wavefronts like it fit a CU.
+        // Placements are grouped by that number ("class"), most wavefronts first; a class too small
+        // to fill one tile joins the next one.
+        // By default every placement is treated like the largest one (one class); with
+        // MMSIM_TILE_CLASSES=1 the classes are formed (measured no faster on the mixes tried: the
+        // classes' launches do not pack the chip evenly enough to pay for the smaller ones' gain).
+        const char *tc_env = std::getenv("MMSIM_TILE_CLASSES");
+        const bool by_class = tc_env && std::atoi(tc_env) != 0;
+        std::vector<int32_t> fit(B, 1);
+        if (!batching)
+            for (int32_t p = 0; p < B; ++p) {
+                int32_t f = (int32_t)std::max<size_t>(1, std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / mixed_wave_bytes(by_class ? slots_of[p] : nslots)));
+                while (f & (f - 1)) f &= f - 1;  // 1, 2, 4 or 8: the same number of wavefronts on every SIMD
+                fit[p] = f;
+            }
         std::vector<int32_t> order(B);
         for (int32_t p = 0; p < B; ++p) order[p] = p;
         std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
+            if (fit[x] != fit[y]) return fit[x] > fit[y];
             if (deepest[x] != deepest[y]) return deepest[x] < deepest[y];
             return expected[x] < expected[y];
         });
         b->pos.assign(B, 0);
-        for (int32_t i = 0; i < B; ++i) b->pos[order[i]] = i;
+        int32_t tile_at = 0;
+        for (int32_t i = 0; i < B;) {
+            int32_t j = i, f = fit[order[i]];
+            while (j < B && (fit[order[j]] == f || j - i < kWave)) {  // less than a tile: take in the next class
+                f = std::min(f, fit[order[j]]);
+                ++j;
+            }
+            while (j < B && fit[order[j]] >= f) ++j;
+            mmsim_batch::TileClass c;
+            c.tile0 = tile_at;
+            c.tile1 = tile_at + (j - i + kWave - 1) / kWave;
+            for (int32_t k = i; k < j; ++k) {
+                c.nslots = std::max(c.nslots, slots_of[order[k]]);
+                b->pos[order[k]] = c.tile0 * kWave + (k - i);
+            }
+            if (batching) {
+                c.nslots = nslots;
+                c.wpb = std::min(wpb, c.tile1 - c.tile0);
+                c.wave_bytes = wave_bytes;
+                c.lds_bytes = (size_t)c.wpb * wave_bytes;
+            } else {
+                c.wave_bytes = mixed_wave_bytes(c.nslots);
+                c.wpb = (int32_t)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / c.wave_bytes);
+                while (c.wpb & (c.wpb - 1)) c.wpb &= c.wpb - 1;
+                c.wpb = std::min(c.wpb, c.tile1 - c.tile0);
+                c.lds_bytes = lat_bytes + (size_t)c.wpb * c.wave_bytes;
+            }
+            b->classes.push_back(c);
+            tile_at = c.tile1;
+            i = j;
+        }
+        b->tiles = tile_at;
+        b->waves = b->tiles * n_seeds;
+        b->lds_bytes = 0;
+        for (const auto &c : b->classes) b->lds_bytes = std::max(b->lds_bytes, c.lds_bytes);
+        b->waves_per_block = b->classes.front().wpb;
     }
 
     // ---- per lane group descriptors [tiles][Gmax+1][64]; row Gmax stays empty
@@ -389,22 +450,26 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         repx32.resize((size_t)b->tiles * M * RX * kWave);
     }
     // LDS byte address of clock slot `slot` of the lane that simulates position `ps` (plain simulator);
-    // slot == nslots is the lane's +inf clock.
+    // slot < 0 names the lane's +inf clock.
     auto clock_addr = [&](int ps, int slot) {
-        const int wv = (ps / kWave) % wpb, lane = ps % kWave;
-        return (uint32_t)(lat_bytes + (size_t)wv * wave_bytes + mixed_clock_offset(rmax_lds_bytes) + (size_t)slot * kSlotBytes +
-                          (size_t)lane * sizeof(double));
+        const int tile = ps / kWave, lane = ps % kWave;
+        const mmsim_batch::TileClass *c = &b->classes.front();
+        for (const auto &x : b->classes)
+            if (tile >= x.tile0 && tile < x.tile1) c = &x;
+        const int wv = (tile - c->tile0) % c->wpb;
+        return (uint32_t)(lat_bytes + (size_t)wv * c->wave_bytes + mixed_clock_offset(rmax_lds_bytes) +
+                          (size_t)(slot < 0 ? c->nslots : slot) * kSlotBytes + (size_t)lane * sizeof(double));
     };
     if (!batching) {  // missing replicas: the +inf clock, flagged empty
         for (size_t i = 0; i < rep32.size(); ++i) {
             const int lane = (int)((i / 4) % kWave);
             const int tile = (int)(i / ((size_t)M * 2 * kWave * 4));
-            rep32[i] = kEmpty | clock_addr(tile * kWave + lane, nslots);
+            rep32[i] = kEmpty | clock_addr(tile * kWave + lane, -1) | ((uint32_t)lat_off[C] << 18);
         }
         for (size_t i = 0; i < repx32.size(); ++i) {
             const int lane = (int)(i % kWave);
             const int tile = (int)(i / ((size_t)M * RX * kWave));
-            repx32[i] = kEmpty | clock_addr(tile * kWave + lane, nslots);
+            repx32[i] = kEmpty | clock_addr(tile * kWave + lane, -1) | ((uint32_t)lat_off[C] << 18);
         }
     }
     std::vector<uint8_t> slot_group;
@@ -595,7 +660,32 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     HIP_TRY(hipEventCreate(&b->ev_stop));
     HIP_TRY(hipStreamSynchronize(st));  // host staging vectors go out of scope below
 
+    // ---- segments.  When the workgroups of a run do not all fit on the chip at once, the streams are
+    //      simulated in nseg launches per class (clocks parked in `state` in between), so that classes
+    //      with different workgroup sizes keep every CU busy instead of leaving a ragged last round.
+    //      MMSIM_SEGMENTS overrides the choice (tuning knob).
+    if (!batching) {
+        int64_t blocks = 0, rmin = b->Rmax;
+        for (const auto &c : b->classes) blocks += (int64_t)((c.tile1 - c.tile0 + c.wpb - 1) / c.wpb) * n_seeds;
+        for (int s = 0; s < n_seeds; ++s) rmin = std::min<int64_t>(rmin, wls[s]->R);
+        const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
+        int64_t nseg = 1;
+        if (blocks > cus && b->classes.size() > 1) nseg = std::min<int64_t>(32, (16 * cus + blocks - 1) / blocks);
+        nseg = std::min<int64_t>(nseg, rmin / 4096);  // a segment is at least 4096 requests
+        if (const char *env = std::getenv("MMSIM_SEGMENTS")) nseg = std::min<int64_t>(std::atoi(env), rmin / kWave);
+        nseg = std::max<int64_t>(1, nseg);
+        b->nseg = (int32_t)nseg;
+        if (b->nseg > 1) HIP_TRY(b->state.alloc((size_t)b->waves * nslots * kWave));
+    }
+
     MixedArgs &a = b->args;
+    a.state = b->state.p;
+    a.state_rows = nslots;
+    a.slot_rows = nslots;
+    a.seg = 0;
+    a.nseg = b->nseg;
+    a.tile0 = 0;
+    a.tile1 = b->tiles;
     a.streams = b->streams.p;
     a.stream_off = b->stream_off.p;
     a.rep32 = reinterpret_cast<const uint4 *>(b->rep32.p);
@@ -699,7 +789,12 @@ int mmsim_ctx_create(int device, mmsim_ctx **out) {
     if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device) != hipSuccess || lds <= 0)
         lds = (int)c->prop.sharedMemPerBlock;
     c->max_lds = lds;
-    HIP_TRY(hipStreamCreate(&c->stream));  // default priority
+    HIP_TRY(hipStreamCreate(&c->stream));  // default priority, like every stream of the library
+    for (int i = 0; i < kSideStreams; ++i) {
+        HIP_TRY(hipStreamCreate(&c->side[i]));
+        HIP_TRY(hipEventCreateWithFlags(&c->ev_join[i], hipEventDisableTiming));
+    }
+    HIP_TRY(hipEventCreateWithFlags(&c->ev_fork, hipEventDisableTiming));
     *out = c.release();
     return MMSIM_OK;
 }
@@ -711,6 +806,14 @@ void mmsim_ctx_destroy(mmsim_ctx *ctx) {
         (void)hipStreamSynchronize(ctx->stream);
         (void)hipStreamDestroy(ctx->stream);
     }
+    for (int i = 0; i < kSideStreams; ++i) {
+        if (ctx->side[i]) {
+            (void)hipStreamSynchronize(ctx->side[i]);
+            (void)hipStreamDestroy(ctx->side[i]);
+        }
+        if (ctx->ev_join[i]) (void)hipEventDestroy(ctx->ev_join[i]);
+    }
+    if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
     delete ctx;
 }
 
@@ -812,10 +915,37 @@ int mmsim_batch_run(mmsim_batch *b) {
     }
     HIP_TRY(hipEventRecord(b->ev_start, ctx->stream));
     std::string err;
-    hipError_t e = (b->flags & MMSIM_BATCHING)
-                       ? launch_sim_batching(b->bargs, b->waves_per_block, b->lds_bytes, ctx->stream, &err)
-                       : launch_sim_mixed(b->args, b->smax_bucket, b->waves_per_block, b->lds_bytes, ctx->stream, &err);
-    if (e != hipSuccess) return fail(MMSIM_E_HIP, err);
+    b->launches = 0;
+    if (b->flags & MMSIM_BATCHING) {
+        if (launch_sim_batching(b->bargs, b->waves_per_block, b->lds_bytes, ctx->stream, &err) != hipSuccess) return fail(MMSIM_E_HIP, err);
+        b->launches = 1;
+    } else {
+        // One launch per (class, segment).  A single class runs on the context's stream; several
+        // classes run side by side on the side streams, each class in segment order on its own.
+        const int nc = (int)b->classes.size();
+        const int used = nc > 1 ? std::min(nc, kSideStreams) : 0;
+        if (used) {
+            HIP_TRY(hipEventRecord(ctx->ev_fork, ctx->stream));
+            for (int i = 0; i < used; ++i) HIP_TRY(hipStreamWaitEvent(ctx->side[i], ctx->ev_fork, 0));
+        }
+        for (int seg = 0; seg < b->nseg; ++seg)
+            for (int ci = 0; ci < nc; ++ci) {
+                const mmsim_batch::TileClass &c = b->classes[ci];
+                MixedArgs a = b->args;
+                a.tile0 = c.tile0;
+                a.tile1 = c.tile1;
+                a.nslots = c.nslots;
+                a.wave_lds_bytes = (int32_t)c.wave_bytes;
+                a.seg = seg;
+                if (launch_sim_mixed(a, b->smax_bucket, c.wpb, c.lds_bytes, used ? ctx->side[ci % used] : ctx->stream, &err) != hipSuccess)
+                    return fail(MMSIM_E_HIP, err);
+                ++b->launches;
+            }
+        for (int i = 0; i < used; ++i) {
+            HIP_TRY(hipEventRecord(ctx->ev_join[i], ctx->side[i]));
+            HIP_TRY(hipStreamWaitEvent(ctx->stream, ctx->ev_join[i], 0));
+        }
+    }
     HIP_TRY(hipEventRecord(b->ev_stop, ctx->stream));
     b->ran = true;
     return MMSIM_OK;
@@ -954,6 +1084,10 @@ int mmsim_batch_get_info(const mmsim_batch *b, mmsim_batch_info *out) {
     out->table_bytes = (int64_t)(b->rep32.bytes() + b->repx32.bytes() + b->rep8.bytes() + b->repx.bytes() + b->ginfo.bytes() +
                                  b->rmax.bytes() + b->lat.bytes() + b->lat_nb.bytes());
     out->stream_bytes = (int64_t)b->streams.bytes();
+    out->tile_classes = (int32_t)b->classes.size();
+    out->segments = b->nseg;
+    out->launches = (b->flags & MMSIM_BATCHING) ? 1 : (int32_t)b->classes.size() * b->nseg;
+    out->reserved = 0;
     return MMSIM_OK;
 }
 

@@ -81,6 +81,11 @@ struct MixedArgs {
     const float *lat;            // [M][lat_row] compact stage latencies (batch size 1)
     int32_t M, lat_row, rep_extra;
     int32_t n_seeds, B, tiles, nslots, Gmax;
+    int32_t tile0, tile1;        // this launch covers tiles [tile0, tile1); nslots and wave_lds_bytes are theirs
+    int32_t seg, nseg;           // this launch covers segment seg of nseg of every stream
+    int32_t slot_rows;           // row pitch of slot_group (most slots of any tile)
+    int32_t state_rows;          // row pitch of state
+    double *state;               // [waves][state_rows][64] clocks between segments (nseg > 1)
     int32_t lat_in_lds;          // 1: the block keeps a copy of lat in LDS
     int32_t uniform_stages;      // 1: all stages of a (model, config) have the same latency; lat is [M][C]
     int32_t pow2_depths;         // 1: every group of the batch has 1, 2, 4, 8 or 16 stages
@@ -105,8 +110,10 @@ struct MixedArgs {
 // LDS layout of the plain simulator, shared by the kernel and by the host code
 // that bakes LDS addresses into the replica descriptors:
 //   [latency table][wavefront 0][wavefront 1]...
-//   wavefront: [64 staged requests][replica bounds][clocks: nslots+1 rows of 64 f64][slot owners][group counters]
+//   wavefront: [64 staged requests][replica bounds u8[M]]
+//              [clocks: nslots+1 rows of 64 f64][slot owners][group counters]
 // Row nslots of the clocks is the +inf row that empty descriptors point at.
+// rmax_lds_bytes is M rounded up to 16.
 __host__ __device__ inline uint32_t mixed_clock_offset(int32_t rmax_lds_bytes) {
     return (uint32_t)(kStageBytes + rmax_lds_bytes);
 }

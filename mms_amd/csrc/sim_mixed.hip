@@ -164,8 +164,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const int wv = uniform((int)(threadIdx.x >> 6));
     const int lane = (int)(threadIdx.x & 63);
     const int seed = (int)(blockIdx.x % (unsigned)a.n_seeds);
-    const int tile = (int)(blockIdx.x / (unsigned)a.n_seeds) * W + wv;
-    const bool live = tile < a.tiles;
+    const int tile = a.tile0 + (int)(blockIdx.x / (unsigned)a.n_seeds) * W + wv;
+    const bool live = tile < a.tile1;
     const bool want_model = (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
@@ -195,16 +195,39 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     __syncthreads();
     if (!live) return;  // padding wavefront of the last workgroup
 
-    for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
-    clk[a.nslots * kWave] = __builtin_inf();
-    if (want_group) {
-        for (int s = 0; s < a.nslots; ++s) owner[s * kWave + lane] = a.slot_group[((size_t)tile * a.nslots + s) * kWave + lane];
-        for (int g = 0; g < 2 * a.Gmax; ++g) gcnt[g * kWave] = 0u;
-    }
-
     const int wave = seed * a.tiles + tile;
+    const size_t out = (size_t)wave * kWave + lane;
     const int64_t off = a.stream_off[seed];
     const int64_t R = a.stream_off[seed + 1] - off;
+    // This launch simulates requests [r0, r1) of the stream: segment a.seg of a.nseg.  Segments other
+    // than the first pick up the lane's state where the previous launch left it.
+    const int64_t r0 = a.seg == 0 ? 0 : ((R * a.seg / a.nseg) & ~(int64_t)(kWave - 1));
+    const int64_t r1 = a.seg == a.nseg - 1 ? R : ((R * (a.seg + 1) / a.nseg) & ~(int64_t)(kWave - 1));
+    const bool resume = a.seg > 0;
+    double *saved = a.state + (size_t)wave * a.state_rows * kWave + lane;
+    int32_t *greq = a.group_req + (size_t)wave * a.Gmax * kWave + lane;
+    int32_t *ggood = a.group_good + (size_t)wave * a.Gmax * kWave + lane;
+
+    int32_t n_good = 0;
+    double lat_sum = 0.0;
+    int64_t fp_ops = 0;
+    if (resume) {
+        for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = saved[(size_t)s * kWave];
+        n_good = a.n_good[out];
+        lat_sum = a.lat_sum[out];
+        if (want_ops) fp_ops = a.fp_ops[out];
+    } else {
+        for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
+    }
+    clk[a.nslots * kWave] = __builtin_inf();
+    if (want_group) {
+        for (int s = 0; s < a.nslots; ++s) owner[s * kWave + lane] = a.slot_group[((size_t)tile * a.slot_rows + s) * kWave + lane];
+        for (int g = 0; g < a.Gmax; ++g) {
+            gcnt[g * kWave] = resume ? (uint32_t)greq[g * kWave] : 0u;
+            gcnt[(a.Gmax + g) * kWave] = resume ? (uint32_t)ggood[g * kWave] : 0u;
+        }
+    }
+
     const int4 *__restrict__ reqs4 = reinterpret_cast<const int4 *>(a.streams + off);
     const uint4 *__restrict__ rep_tile = a.rep32 + (size_t)tile * a.M * 2 * kWave + lane;
     const uint32_t *__restrict__ repx_tile = a.repx32 + (size_t)tile * a.M * a.rep_extra * kWave + lane;
@@ -214,17 +237,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + lane;
     const double overhead = a.fixed_overhead;
 
-    int32_t n_good = 0;
-    double lat_sum = 0.0;
-    int64_t fp_ops = 0;
-
     int4 ahead = make_int4(0, 0, -1, 0);  // this lane's request of the next block
-    if (R > 0) ahead = reqs4[lane < R ? lane : R - 1];
+    if (R > 0) ahead = reqs4[r0 + lane < R ? r0 + lane : R - 1];
 
-    for (int64_t blk = 0; blk < R; blk += kWave) {
+    for (int64_t blk = r0; blk < r1; blk += kWave) {
         {   // park this block's requests; the model word also carries the tile's replica bound
             int4 r = ahead;
-            const bool ok = blk + lane < R && r.z >= 0;
+            const bool ok = blk + lane < r1 && r.z >= 0;
             const int bound = (int)rmax_lds[ok ? r.z : 0];
             r.z = ok ? (r.z | (bound << 24)) : -1;
             stage4[lane] = r;
@@ -233,7 +252,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             const int64_t nx = blk + kWave + lane;
             ahead = reqs4[nx < R ? nx : R - 1];
         }
-        const int nblk = (int)(R - blk < kWave ? R - blk : kWave);  // requests in this block
+        const int nblk = (int)(r1 - blk < kWave ? r1 - blk : kWave);  // requests in this block
 
         // Always 2*CH loads per chunk, whatever the requests are.
         auto load_chunk = [&](Chunk<CH> &c, int cb) {
@@ -249,7 +268,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 const bool ok = w >= 0;
                 const int m = ok ? (w & 0xFFFFFF) : -1;
                 c.m[u] = m;
-                c.nrep[u] = ok ? (w >> 24) : 0;
+                c.nrep[u] = ok ? (w >> 24) : 0;  // 0: nothing to simulate (unknown model or no replica in the tile)
                 c.t[u] = __hiloint2double(r[u].y, r[u].x);
                 c.slo[u] = __int_as_float(r[u].w);
                 const uint4 *row = rep_tile + (size_t)(ok ? m : 0) * (2 * kWave);
@@ -316,7 +335,6 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                         consider(d, *reinterpret_cast<const double *>(lds_raw + rep_addr(d)), lrow_m[rep_lat_last(d)]);
                     }
                 }
-
                 const bool has = (int32_t)sel >= 0;
                 const int sm1 = has ? (int)rep_stages_m1(sel) : -1;  // stages - 1
                 const uint32_t last_addr = rep_addr(sel);            // the lane's +inf clock when there is no replica
@@ -452,13 +470,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         }
     }
 
-    const size_t out = (size_t)seed * a.tiles * kWave + (size_t)tile * kWave + lane;
     a.n_good[out] = n_good;
     a.lat_sum[out] = lat_sum;
     if (want_ops) a.fp_ops[out] = fp_ops;
+    if (a.seg < a.nseg - 1)
+        for (int s = 0; s < a.nslots; ++s) saved[(size_t)s * kWave] = clk[s * kWave];
     if (want_group) {
-        int32_t *greq = a.group_req + (size_t)wave * a.Gmax * kWave + lane;
-        int32_t *ggood = a.group_good + (size_t)wave * a.Gmax * kWave + lane;
         for (int g = 0; g < a.Gmax; ++g) {
             greq[g * kWave] = (int32_t)gcnt[g * kWave];
             ggood[g * kWave] = (int32_t)gcnt[(a.Gmax + g) * kWave];
@@ -474,7 +491,7 @@ hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStrea
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return e;
     }
-    const unsigned tile_groups = (unsigned)((args.tiles + wpb - 1) / wpb);
+    const unsigned tile_groups = (unsigned)((args.tile1 - args.tile0 + wpb - 1) / wpb);
     const dim3 grid(tile_groups * (unsigned)args.n_seeds);
     hipLaunchKernelGGL(kern, grid, dim3(wpb * kWave), lds_bytes, stream, args);
     return hipGetLastError();

@@ -123,6 +123,12 @@ def test_config4_subsample_counts_and_a_few_full_traces(eng):
     out, table, packed, streams, _ = _run_config(eng, cfg, cfg.placements[:4], [0], ALL)
     ref = oracle_batch(streams[0], table, packed, want_per_request=True)
     assert_batch_matches(out, ref, 0, packed[0], per_request=True, where="cfg4 traces")
+    # traces and model counts without group / operation counts, a full wavefront of placements
+    some_flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_PER_REQUEST
+    out, table, packed, streams, _ = _run_config(eng, cfg, cfg.placements[:64], [0], some_flags)
+    ref = oracle_batch(streams[0], table, packed, want_per_request=True)
+    assert_batch_matches(out, ref, 0, packed[0], per_request=True, where="cfg4 traces, 64 placements")
+    assert (~ref["good"]).all(axis=0).mean() > 0.2      # many requests are rejected by all 64 placements
 
 
 @pytest.mark.parametrize("depths", [(1, 2, 4), (1, 2, 4, 8, 16), (1, 2, 3, 4), (1, 3, 5, 8, 11, 16)])
@@ -171,6 +177,57 @@ def test_stage_walk_variants(eng, depths, uniform):
     ref = oracle_batch(st, table, packed, want_per_request=True)
     assert_batch_matches(out, ref, 0, packed[0], per_request=True, where=f"depths {depths} uniform {uniform}")
     assert 0.05 * R * 130 < ref["n_good"].sum() < 0.98 * R * 130    # both accepts and rejects are exercised
+
+
+@pytest.mark.parametrize("flags", [0, ALL])
+@pytest.mark.parametrize("segments", [1, 5])
+def test_tile_classes_and_stream_segments(eng, monkeypatch, flags, segments):
+    """Large batches are split into classes of tiles by clock-slot count (each launched with its own
+    LDS size, side by side) and their streams into segments with the clocks parked in between.
+    Forced here on a small batch: 420 placements using 4..56 devices, odd stream length."""
+    from types import SimpleNamespace
+    from mms_amd.profiling import ParallelConfig
+    from mms_amd.placement_policy.base_policy import ModelPlacement
+    from mms_amd.profiling import synthetic_profile
+    monkeypatch.setenv("MMSIM_WAVES_PER_CU", "8")
+    monkeypatch.setenv("MMSIM_TILE_CLASSES", "1")
+    monkeypatch.setenv("MMSIM_SEGMENTS", str(segments))
+    rng = np.random.default_rng(77)
+    M, R = 24, 3001
+    pcs = [ParallelConfig(1, 1, d) for d in (1, 2, 4, 8)]
+    profiles = [synthetic_profile(f"m{m}", float(rng.uniform(0.05, 0.3)), pcs) for m in range(M)]
+    sols = []
+    for i in range(420):
+        left, cfgs, models = int(rng.choice([4, 8, 12, 20, 28, 36, 44, 56])), [], []
+        while left > 0:
+            d = int(rng.choice([x for x in (1, 2, 4, 8) if x <= left]))
+            left -= d
+            cfgs.append(ParallelConfig(1, 1, d))
+            models.append([int(x) for x in rng.choice(M, size=int(rng.integers(1, 6)), replace=False)])
+        sols.append(ModelPlacement(cfgs, models))
+    streams = []
+    for seed in range(2):
+        gaps = rng.exponential(0.01, size=R + seed * 70)
+        streams.append(SimpleNamespace(tstamps=np.cumsum(gaps), model_ids=rng.integers(-1, M, len(gaps)).astype(np.int32),
+                                       slos=rng.uniform(0.2, 1.0, len(gaps)).astype(np.float32)))
+    table = E.LatencyTable(profiles, [1])
+    packed = E.pack_placements(sols, table)
+    dws = [E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, M) for st in streams]
+    batch = E.Batch(eng, dws, table, packed, flags)
+    info = batch.info()
+    print(info, flush=True)
+    assert info["tile_classes"] >= 2 and info["segments"] == segments
+    assert info["launches"] == info["tile_classes"] * segments
+    for _ in range(2):                      # a re-run starts from scratch again
+        batch.run()
+        batch.sync()
+    out = batch.fetch()
+    batch.close()
+    for s, st in enumerate(streams):
+        ref = oracle_batch(st, table, packed, want_per_request=bool(flags))
+        assert_batch_matches(out, ref, s, packed[0], per_request=bool(flags), where=f"seed {s}")
+        if flags:
+            assert out["fp_ops"][s].sum() == ref["fp_ops"]
 
 
 def test_scores_only_mode_equals_full_mode(eng):

@@ -47,7 +47,7 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.Tables) == 48
     assert ctypes.sizeof(_lib.Placements) == 40
     assert ctypes.sizeof(_lib.Result) == 10 * 8
-    assert ctypes.sizeof(_lib.BatchInfo) == 8 * 4 + 3 * 8
+    assert ctypes.sizeof(_lib.BatchInfo) == 8 * 4 + 3 * 8 + 4 * 4
 
 
 # ---- table build (controller.py:412-476) --------------------------------------------------
