@@ -82,6 +82,14 @@ __device__ __forceinline__ double vmin(double x, double y) {
     return r;
 }
 
+// LDS accesses by byte address (the replica descriptors carry addresses, not pointers).
+__device__ __forceinline__ double lds_f64(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) double *>(addr);
+}
+__device__ __forceinline__ void lds_set_f64(uint32_t addr, double v) {
+    *reinterpret_cast<__attribute__((address_space(3))) double *>(addr) = v;
+}
+
 // 32-bit LDS byte address of a pointer into shared memory (for ds_* in inline asm).
 __device__ __forceinline__ uint32_t lds_addr(const void *p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
@@ -318,7 +326,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     static_while<0, nj>([&](auto J) {
                         constexpr int j = decltype(J)::value;
                         const uint32_t d = pick_desc<j>(cur.da[u], cur.db[u]);
-                        cl[j] = *reinterpret_cast<const double *>(lds_raw + rep_addr(d));
+                        cl[j] = lds_f64(rep_addr(d));
                         ll[j] = lrow_m[rep_lat_last(d)];
                         return true;
                     });
@@ -336,7 +344,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
                     for (int j = RREG; j < n; ++j) {
                         const uint32_t d = row[(size_t)(j - RREG) * kWave];
-                        consider(d, *reinterpret_cast<const double *>(lds_raw + rep_addr(d)), lrow_m[rep_lat_last(d)]);
+                        consider(d, lds_f64(rep_addr(d)), lrow_m[rep_lat_last(d)]);
                     }
                 }
                 const bool has = (int32_t)sel >= 0;
@@ -355,17 +363,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     const double latency = finish_time - tstamp;
                     acc = has && latency <= slo;
                     if (acc) {
-                        *reinterpret_cast<double *>(lds_raw + last_addr) = t;
+                        lds_set_f64(last_addr, t);
                         n_good += 1;
                         lat_sum += latency;
                     }
                 } else {
                     // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
-                    int walk = -1;  // stages - 1 of lanes that walk
-                    if (has) {
-                        const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
-                        walk = bound > slo ? -1 : sm1;
-                    }
+                    const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
+                    const int walk = (has && !(bound > slo)) ? sm1 : -1;  // stages - 1 of lanes that walk
                     if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
                         // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
                         uint64_t saved_exec;
