@@ -151,6 +151,13 @@ def main():
     else:
         assert np.all(out["status"] == 0), "a lane ran out of idle-event slots"
 
+    # HBM bytes per launch from the committed rocprofv3 counter runs (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB,
+    # scaled by a 1 GiB device copy): only known for the workload those runs used.
+    traffic = None
+    if (cfg.index == 4 and args.placements is None and args.seeds is None and args.flags == "scores"):
+        traffic = {"bytes_per_launch": 1.438e11 + 1.5e6, "source": "profiles/sim_mixed_kernel_cfg4.md",
+                   "algorithmic_bytes": info["stream_bytes"] + info["table_bytes"] + 12 * lanes}
+
     result = {
         "metric": "simulated request x placement evals/sec",
         "value": value,
@@ -181,7 +188,7 @@ def main():
             "frac_of_published_fma_peak": None if achieved_tops is None else achieved_tops / FP64_VECTOR_PEAK_FMA_TFLOPS,
             "ops_per_launch": total_ops,
             "ops_per_eval": None if total_ops is None else total_ops / evals_per_step,
-            "traffic": None,
+            "traffic": traffic,
             "hbm_algorithmic_GBps": (info["stream_bytes"] * info["waves"] / max(len(seeds), 1)
                                      + info["table_bytes"] * len(seeds)) / kernel_s / 1e9,
             "note": "fp64 add/max/compare only (no FMA): peak = published 78.6 TFLOP/s / 2; "
