@@ -451,25 +451,26 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
     // LDS byte address of clock slot `slot` of the lane that simulates position `ps` (plain simulator);
     // slot < 0 names the lane's +inf clock.
+    std::vector<uint32_t> tile_clock0(b->tiles, 0);  // address of slot 0, lane 0 of each tile
+    std::vector<int32_t> tile_inf_slot(b->tiles, 0);
+    for (const auto &c : b->classes)
+        for (int32_t tile = c.tile0; tile < c.tile1; ++tile) {
+            tile_clock0[tile] = (uint32_t)(lat_bytes + (size_t)((tile - c.tile0) % c.wpb) * c.wave_bytes + mixed_clock_offset(rmax_lds_bytes));
+            tile_inf_slot[tile] = c.nslots;
+        }
     auto clock_addr = [&](int ps, int slot) {
         const int tile = ps / kWave, lane = ps % kWave;
-        const mmsim_batch::TileClass *c = &b->classes.front();
-        for (const auto &x : b->classes)
-            if (tile >= x.tile0 && tile < x.tile1) c = &x;
-        const int wv = (tile - c->tile0) % c->wpb;
-        return (uint32_t)(lat_bytes + (size_t)wv * c->wave_bytes + mixed_clock_offset(rmax_lds_bytes) +
-                          (size_t)(slot < 0 ? c->nslots : slot) * kSlotBytes + (size_t)lane * sizeof(double));
+        return tile_clock0[tile] + (uint32_t)(slot < 0 ? tile_inf_slot[tile] : slot) * kSlotBytes + (uint32_t)lane * (uint32_t)sizeof(double);
     };
-    if (!batching) {  // missing replicas: the +inf clock, flagged empty
-        for (size_t i = 0; i < rep32.size(); ++i) {
-            const int lane = (int)((i / 4) % kWave);
-            const int tile = (int)(i / ((size_t)M * 2 * kWave * 4));
-            rep32[i] = kEmpty | clock_addr(tile * kWave + lane, -1) | ((uint32_t)lat_off[C] << 18);
-        }
-        for (size_t i = 0; i < repx32.size(); ++i) {
-            const int lane = (int)(i % kWave);
-            const int tile = (int)(i / ((size_t)M * RX * kWave));
-            repx32[i] = kEmpty | clock_addr(tile * kWave + lane, -1) | ((uint32_t)lat_off[C] << 18);
+    if (!batching) {  // missing replicas: the +inf clock and the +inf latency, flagged empty
+        const uint32_t inf_lat = (uint32_t)lat_off[C] << 18;
+        for (int32_t tile = 0; tile < b->tiles; ++tile) {
+            uint32_t lane_word[kWave];
+            for (int lane = 0; lane < kWave; ++lane) lane_word[lane] = kEmpty | clock_addr(tile * kWave + lane, -1) | inf_lat;
+            uint32_t *dst = rep32.data() + (size_t)tile * M * 2 * kWave * 4;
+            for (size_t i = 0; i < (size_t)M * 2 * kWave * 4; ++i) dst[i] = lane_word[(i / 4) % kWave];
+            uint32_t *dx = repx32.data() + (size_t)tile * M * RX * kWave;
+            for (size_t i = 0; i < (size_t)M * RX * kWave; ++i) dx[i] = lane_word[i % kWave];
         }
     }
     std::vector<uint8_t> slot_group;
