@@ -374,7 +374,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (!batching)
             for (int32_t p = 0; p < B; ++p) {
                 int32_t f = (int32_t)std::max<size_t>(1, std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / mixed_wave_bytes(by_class ? slots_of[p] : nslots)));
-                while (f & (f - 1)) f &= f - 1;  // 1, 2, 4 or 8: the same number of wavefronts on every SIMD
+                if (f > 4) f = f == 8 ? 8 : 4;  // beyond one per SIMD only the same number on every SIMD pays
                 fit[p] = f;
             }
         std::vector<int32_t> order(B);
@@ -408,7 +408,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             } else {
                 c.wave_bytes = mixed_wave_bytes(c.nslots);
                 c.wpb = (int32_t)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / c.wave_bytes);
-                while (c.wpb & (c.wpb - 1)) c.wpb &= c.wpb - 1;
+                if (c.wpb > 4) c.wpb = c.wpb == 8 ? 8 : 4;
                 c.wpb = std::min(c.wpb, c.tile1 - c.tile0);
                 c.lds_bytes = lat_bytes + (size_t)c.wpb * c.wave_bytes;
             }
