@@ -468,7 +468,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     }
                     if (has) fp_ops += 2 * (sm1 + 1) + nvalid + 3;
                 }
-                if (want_model && m >= 0) model_good[(size_t)m * kWave] += acc ? 1 : 0;
+                if (want_model && m >= 0 && acc)  // one owner per counter: a relaxed add that nobody waits for
+                    __hip_atomic_fetch_add(&model_good[(size_t)m * kWave], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (want_req) {
                     fin_out[(blk + cb + u) * kWave] = acc ? finish_time : tstamp;
                     good_out[(blk + cb + u) * kWave] = acc ? 1 : 0;
