@@ -82,8 +82,7 @@ struct mmsim_workload {
     // arrivals regrouped by model (batching simulator): offsets per model, then per arrival
     // its time, its deadline time + (double)slo and its index in the stream
     std::vector<int64_t> mq_off;
-    DevBuf<double> mq_t, mq_dl;
-    DevBuf<int32_t> mq_idx;
+    DevBuf<MqEntry> mq;
 };
 
 // Ordered replica lists per (placement, model): the rows of m_id2g_id.
@@ -136,8 +135,8 @@ struct mmsim_batch {
     DevBuf<int64_t> fp_ops;
     // batching simulator
     DevBuf<int64_t> mq_off;
-    DevBuf<double> mq_t, mq_dl;
-    DevBuf<int32_t> mq_idx, status, batch_sizes;
+    DevBuf<MqEntry> mq;
+    DevBuf<int32_t> status, batch_sizes;
     DevBuf<uint16_t> g2m_off, g2m_idx;
     DevBuf<float> lat_nb;
     std::vector<uint8_t> hosted;  // [B][M] model has a replica (batching: decides model_num_requests)
@@ -326,11 +325,11 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (wave_bytes > (size_t)ctx->max_lds) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
         if ((size_t)ctx->max_lds > (size_t)kRepAddrMask) return fail(MMSIM_E_UNSUPPORTED, "LDS is larger than the descriptor's address field");
     } else {
-        // per wavefront: descriptors | clocks | event times | queue heads | event groups | arrivals per model.
-        // Events: the reference's heap holds about one entry per group plus a few stale ones;
-        // provision 2*G+8 if that fits, never less than G+4.
-        const size_t fixed = (size_t)(Gmax + 1) * kWave * 4 + (size_t)nslots * kWave * 8 + (size_t)M * kWave * 4 + (size_t)M * 4 + 16;
-        for (heap_cap = 2 * Gmax + 8; heap_cap >= Gmax + 4; --heap_cap) {
+        // per wavefront: descriptors | clocks | event times | queue heads | head ranks | event groups |
+        // arrivals per model.  Events: the reference's heap holds about one entry per group plus a few
+        // stale ones (most seen: G+3); provision min(2*G+8, G+16) if that fits, never less than G+4.
+        const size_t fixed = (size_t)(Gmax + 1) * kWave * 4 + (size_t)nslots * kWave * 8 + (size_t)2 * M * kWave * 4 + (((size_t)M * 4 + 15) & ~(size_t)15);
+        for (heap_cap = std::min(2 * Gmax + 8, Gmax + 16); heap_cap >= Gmax + 4; --heap_cap) {
             wave_bytes = (fixed + (size_t)heap_cap * kWave * 12 + 15) & ~(size_t)15;
             if (wave_bytes <= (size_t)ctx->max_lds) break;
         }
@@ -570,6 +569,38 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                     }
     }
 
+    // ---- batching simulator: keep the latency table (per workgroup) and the models of each group (per
+    //      wavefront) in LDS when they fit; they are read in the innermost loops.  Fewer wavefronts per
+    //      workgroup are accepted for it: the loops are bound by the latency of these reads.
+    size_t batching_lat_lds = 0;
+    int batching_g2m_lds = 0;
+    if (batching) {
+        const size_t lat_b = (lat_nb.size() * sizeof(float) + 15) & ~(size_t)15;
+        const size_t g2m_b = ((size_t)(Gmax + 1) * kWave * 2 + (size_t)members_max * kWave * 2 + 15) & ~(size_t)15;
+        const size_t cap = (size_t)ctx->max_lds;
+        int w = wpb;
+        for (; w >= 1; --w)
+            if (lat_b + (size_t)w * (wave_bytes + g2m_b) <= cap) break;
+        if (w >= 1) {
+            batching_lat_lds = lat_b;
+            batching_g2m_lds = 1;
+            wpb = w;
+        } else if (lat_b + wave_bytes <= cap) {
+            batching_lat_lds = lat_b;
+            wpb = (int)std::min<size_t>(wpb, (cap - lat_b) / wave_bytes);
+        } else if (wave_bytes + g2m_b <= cap) {
+            batching_g2m_lds = 1;
+            wpb = (int)std::min<size_t>(wpb, cap / (wave_bytes + g2m_b));
+        }
+        if (batching_g2m_lds) wave_bytes += g2m_b;
+        mmsim_batch::TileClass &c = b->classes.front();
+        c.wpb = std::min(wpb, c.tile1 - c.tile0);
+        c.wave_bytes = wave_bytes;
+        c.lds_bytes = batching_lat_lds + (size_t)c.wpb * wave_bytes;
+        b->lds_bytes = c.lds_bytes;
+        b->waves_per_block = c.wpb;
+    }
+
     // ---- request streams back to back
     std::vector<int64_t> soff(n_seeds + 1, 0);
     for (int s = 0; s < n_seeds; ++s) {
@@ -619,16 +650,13 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             for (int32_t m = 0; m <= M; ++m) mqo[(size_t)s * (M + 1) + m] = total + wls[s]->mq_off[m];
             total += wls[s]->mq_off[M];
         }
-        HIP_TRY(b->mq_t.alloc((size_t)total));
-        HIP_TRY(b->mq_dl.alloc((size_t)total));
-        HIP_TRY(b->mq_idx.alloc((size_t)total));
+        HIP_TRY(b->mq.alloc((size_t)total + 1));  // one padding entry: the kernel looks one entry past a popped head
+        HIP_TRY(hipMemsetAsync(b->mq.p + total, 0, sizeof(MqEntry), st));
         int64_t at = 0;
         for (int s = 0; s < n_seeds; ++s) {
             const size_t n = (size_t)wls[s]->mq_off[M];
             if (n > 0) {
-                HIP_TRY(hipMemcpyAsync(b->mq_t.p + at, wls[s]->mq_t.p, sizeof(double) * n, hipMemcpyDeviceToDevice, st));
-                HIP_TRY(hipMemcpyAsync(b->mq_dl.p + at, wls[s]->mq_dl.p, sizeof(double) * n, hipMemcpyDeviceToDevice, st));
-                HIP_TRY(hipMemcpyAsync(b->mq_idx.p + at, wls[s]->mq_idx.p, sizeof(int32_t) * n, hipMemcpyDeviceToDevice, st));
+                HIP_TRY(hipMemcpyAsync(b->mq.p + at, wls[s]->mq.p, sizeof(MqEntry) * n, hipMemcpyDeviceToDevice, st));
             }
             at += (int64_t)n;
         }
@@ -725,9 +753,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         q.streams = b->streams.p;
         q.stream_off = b->stream_off.p;
         q.mq_off = b->mq_off.p;
-        q.mq_t = b->mq_t.p;
-        q.mq_dl = b->mq_dl.p;
-        q.mq_idx = b->mq_idx.p;
+        q.mq = b->mq.p;
         q.rep8 = b->rep8.p;
         q.repx = b->repx.p;
         q.ginfo = b->ginfo.p;
@@ -747,6 +773,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         q.nslots = nslots;
         q.Gmax = Gmax;
         q.wave_lds_bytes = (int32_t)wave_bytes;
+        q.lat_lds_bytes = (int32_t)batching_lat_lds;
+        q.g2m_in_lds = batching_g2m_lds;
         q.Rmax = b->Rmax;
         q.fixed_overhead = t->fixed_overhead;
         q.flags = flags;
@@ -854,30 +882,36 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
     w->mq_off.assign((size_t)M + 1, 0);
     for (int32_t m = 0; m < M; ++m) w->mq_off[m + 1] = w->mq_off[m] + w->model_num_requests[m];
     const size_t known = (size_t)w->mq_off[M];
-    std::vector<double> mq_t(known), mq_dl(known);
-    std::vector<int32_t> mq_idx(known);
+    std::vector<MqEntry> mq(known);
     {
+        // dense rank of every arrival time (streams are normally sorted; this does not rely on it)
+        std::vector<int32_t> order((size_t)R), rank((size_t)R, 0);
+        for (int64_t i = 0; i < R; ++i) order[(size_t)i] = (int32_t)i;
+        std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) { return tstamps[x] < tstamps[y]; });
+        int32_t r = 0;
+        for (int64_t k = 0; k < R; ++k) {
+            if (k > 0 && tstamps[order[(size_t)k]] != tstamps[order[(size_t)k - 1]]) ++r;
+            rank[(size_t)order[(size_t)k]] = r;
+        }
         std::vector<int64_t> fill(w->mq_off.begin(), w->mq_off.end() - 1);
         for (int64_t i = 0; i < R; ++i)
             if (model_ids[i] >= 0) {
-                const size_t q = (size_t)fill[model_ids[i]]++;
-                mq_t[q] = tstamps[i];
-                mq_dl[q] = tstamps[i] + (double)slos[i];  // controller.py:679
-                mq_idx[q] = (int32_t)i;
+                MqEntry &e = mq[(size_t)fill[model_ids[i]]++];
+                e.t = tstamps[i];
+                e.dl = tstamps[i] + (double)slos[i];  // controller.py:679
+                e.idx = (int32_t)i;
+                e.rank = rank[(size_t)i];
+                e.pad[0] = e.pad[1] = 0;
             }
     }
     if (R > 0x7FFFFFFF) return fail(MMSIM_E_UNSUPPORTED, "workload_create: more than 2^31-1 requests");
     HIP_TRY(hipSetDevice(ctx->device));
     HIP_TRY(w->reqs.alloc((size_t)R));
-    HIP_TRY(w->mq_t.alloc(known));
-    HIP_TRY(w->mq_dl.alloc(known));
-    HIP_TRY(w->mq_idx.alloc(known));
+    HIP_TRY(w->mq.alloc(known));
     if (R > 0) {
         HIP_TRY(hipMemcpyAsync(w->reqs.p, host.data(), sizeof(Req) * (size_t)R, hipMemcpyHostToDevice, ctx->stream));
         if (known > 0) {
-            HIP_TRY(hipMemcpyAsync(w->mq_t.p, mq_t.data(), sizeof(double) * known, hipMemcpyHostToDevice, ctx->stream));
-            HIP_TRY(hipMemcpyAsync(w->mq_dl.p, mq_dl.data(), sizeof(double) * known, hipMemcpyHostToDevice, ctx->stream));
-            HIP_TRY(hipMemcpyAsync(w->mq_idx.p, mq_idx.data(), sizeof(int32_t) * known, hipMemcpyHostToDevice, ctx->stream));
+            HIP_TRY(hipMemcpyAsync(w->mq.p, mq.data(), sizeof(MqEntry) * known, hipMemcpyHostToDevice, ctx->stream));
         }
         HIP_TRY(hipStreamSynchronize(ctx->stream));
     }

@@ -20,6 +20,19 @@ struct __attribute__((aligned(16))) Req {
 };
 static_assert(sizeof(Req) == 16, "Req must be 16 bytes");
 
+// One arrival in a seed's arrivals regrouped by model (batching simulator): a model's FIFO is always
+// a window of that list.  rank is the dense rank of the arrival time among the seed's arrival times,
+// so comparing ranks is comparing times (the reference compares times, ties keep the earlier-listed
+// model) without fetching them.
+struct __attribute__((aligned(32))) MqEntry {
+    double t;      // arrival time
+    double dl;     // deadline: arrival + (double)slo
+    int32_t idx;   // index in the seed's stream
+    int32_t rank;
+    int32_t pad[2];
+};
+static_assert(sizeof(MqEntry) == 32, "MqEntry must be 32 bytes");
+
 // Group descriptor of the batching simulator: one 32-bit word per (placement,
 // group), kept per lane in LDS; replicas are listed as group indices.
 //   bits  0..7   clock slot of the group's LAST pipeline stage (slots are the
@@ -125,10 +138,8 @@ __host__ __device__ inline uint32_t mixed_clock_offset(int32_t rmax_lds_bytes) {
 struct BatchingArgs {
     const Req *streams;          // all seeds' requests, back to back
     const int64_t *stream_off;   // [n_seeds+1]
-    const int64_t *mq_off;       // [n_seeds][M+1] offsets into mq_* of the arrivals of each model
-    const double *mq_t;          // arrival time of each model-ordered arrival
-    const double *mq_dl;         // its deadline: arrival + (double)slo
-    const int32_t *mq_idx;       // its index in the seed's stream
+    const int64_t *mq_off;       // [n_seeds][M+1] offsets into mq of the arrivals of each model
+    const MqEntry *mq;           // model-ordered arrivals of all seeds, plus one padding entry at the end
     const uint64_t *rep8;        // as in MixedArgs
     const uint8_t *repx;
     const uint32_t *ginfo;       // [tiles][Gmax+1][64]
@@ -139,6 +150,8 @@ struct BatchingArgs {
     int32_t M, lat_row, NB, rep_extra, members_max, heap_cap;
     int32_t n_seeds, B, tiles, nslots, Gmax;
     int32_t wave_lds_bytes;
+    int32_t lat_lds_bytes;       // > 0: the workgroup keeps a copy of lat in LDS (that many bytes, 16-aligned)
+    int32_t g2m_in_lds;          // 1: each wavefront keeps its g2m_off / g2m_idx rows in LDS
     int64_t Rmax;
     double fixed_overhead;
     uint32_t flags;

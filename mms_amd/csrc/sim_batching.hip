@@ -16,7 +16,9 @@
 //     of that model's arrivals, so it is a (head, tail) window into the
 //     seed's arrivals regrouped by model; tail is the number of arrivals so
 //     far (the same for every lane that hosts the model) and head[m][lane]
-//     lives in LDS;
+//     lives in LDS, together with the dense rank of the head request's
+//     arrival time (hrank[m][lane]) so that "whose head arrived first" is
+//     decided without touching global memory;
 //   * the pending idle events, a multiset of (time, group) that the
 //     reference keeps in a heap (:728, :739-740): a small unsorted array per
 //     lane in LDS, popped by lexicographic minimum.  If a lane would need
@@ -46,14 +48,19 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const int lane = (int)(threadIdx.x & 63);
     const int seed = (int)(blockIdx.x % (unsigned)a.n_seeds);
     const int tile = (int)(blockIdx.x / (unsigned)a.n_seeds) * W + wv;
-    if (tile >= a.tiles) return;  // no barriers in this kernel
     const bool want_model = (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const int M = a.M, Gmax = a.Gmax, NB = a.NB;
 
-    // ---- LDS of this wavefront: group descriptors | clocks | queue heads | event times | event groups | arrivals per model
-    unsigned char *mine = lds_raw + wv * a.wave_lds_bytes;
+    // ---- LDS: [latency table, shared, if it fits][per wavefront: group descriptors | clocks | event times |
+    //      queue heads | head ranks | event groups | arrivals per model | models of each group, if they fit]
+    float *lat_lds = reinterpret_cast<float *>(lds_raw);
+    if (a.lat_lds_bytes > 0) {
+        const int n = M * a.lat_row * NB;
+        for (int i = (int)threadIdx.x; i < n; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
+    }
+    unsigned char *mine = lds_raw + a.lat_lds_bytes + wv * a.wave_lds_bytes;
     uint32_t *ginfo = reinterpret_cast<uint32_t *>(mine) + lane;
     size_t o = (size_t)(Gmax + 1) * kWave * 4;
     double *clk = reinterpret_cast<double *>(mine + o) + lane;
@@ -62,19 +69,38 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     o += (size_t)a.heap_cap * kWave * 8;
     uint32_t *head = reinterpret_cast<uint32_t *>(mine + o) + lane;
     o += (size_t)M * kWave * 4;
+    int32_t *hrank = reinterpret_cast<int32_t *>(mine + o) + lane;  // rank of the arrival at head[m] (already known before it arrives)
+    o += (size_t)M * kWave * 4;
     uint32_t *ev_g = reinterpret_cast<uint32_t *>(mine + o) + lane;
     o += (size_t)a.heap_cap * kWave * 4;
     volatile uint32_t *arrived = reinterpret_cast<volatile uint32_t *>(mine + o);  // [M], same for all lanes
+    o += ((size_t)M * 4 + 15) & ~(size_t)15;
+    uint16_t *g2m_off_lds = reinterpret_cast<uint16_t *>(mine + o) + lane;  // [Gmax+1][64]
+    o += (size_t)(Gmax + 1) * kWave * 2;
+    uint16_t *g2m_idx_lds = reinterpret_cast<uint16_t *>(mine + o) + lane;  // [members_max][64]
 
-    {
+    const bool live = tile < a.tiles;
+    if (live) {
         const uint32_t *gsrc = a.ginfo + (size_t)tile * (Gmax + 1) * kWave + lane;
         for (int g = 0; g <= Gmax; ++g) ginfo[g * kWave] = gsrc[g * kWave];
         for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
-        for (int m = 0; m < M; ++m) head[m * kWave] = 0u;
+        {
+            const int64_t *mo = a.mq_off + (size_t)seed * (M + 1);
+            for (int m = 0; m < M; ++m) {
+                head[m * kWave] = 0u;
+                hrank[m * kWave] = a.mq[mo[m]].rank;  // of the model's first arrival (the padding entry if it has none)
+            }
+        }
         for (int m = lane; m < M; m += kWave) arrived[m] = 0u;
+        if (a.g2m_in_lds) {
+            const uint16_t *osrc = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
+            const uint16_t *isrc = a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
+            for (int g = 0; g <= Gmax; ++g) g2m_off_lds[g * kWave] = osrc[g * kWave];
+            for (int x = 0; x < a.members_max; ++x) g2m_idx_lds[x * kWave] = isrc[(size_t)x * kWave];
+        }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    __syncthreads();  // the latency table is complete; wavefronts run independently from here
+    if (!live) return;
 
     const int wave = seed * a.tiles + tile;
     const int64_t off = a.stream_off[seed];
@@ -83,8 +109,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const int64_t *__restrict__ mq_off = a.mq_off + (size_t)seed * (M + 1);
     const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * M * kWave + lane;
     const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * M * a.rep_extra * kWave + lane;
-    const uint16_t *__restrict__ g2m_off = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
-    const uint16_t *__restrict__ g2m_idx = a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
+    // generic pointers: LDS copies when they fit, else the tables in global memory
+    const uint16_t *g2m_off = a.g2m_in_lds ? g2m_off_lds : a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
+    const uint16_t *g2m_idx = a.g2m_in_lds ? g2m_idx_lds : a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
+    const float *lat_tab = a.lat_lds_bytes > 0 ? lat_lds : a.lat;
     int32_t *model_good = a.model_good + (size_t)wave * M * kWave + lane;
     int32_t *group_req = a.group_req + (size_t)wave * Gmax * kWave + lane;
     int32_t *group_good = a.group_good + (size_t)wave * Gmax * kWave + lane;
@@ -95,9 +123,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     int32_t n_good = 0;
     double lat_sum = 0.0;
     int hn = 0;          // pending idle events of this lane
+    double next_due = __builtin_inf();  // the earliest of them (+inf if none): arrivals before it skip the event list
     int dead = 0;        // nonzero status: this lane stopped (out of event slots / unsupported input)
 
     const uint32_t none = (uint32_t)Gmax;
+    Req blk_req = {0.0, -1, 0.0f};  // this lane's request of the current block of 64
 
     // queue length of a model this lane hosts
     auto qlen = [&](int m) -> int { return (int)(arrived[m] - head[m * kWave]); };
@@ -105,16 +135,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     // :654-664 -- among the models of group g with a waiting request, the one whose head arrived first
     auto select_model = [&](uint32_t g) -> int {
         const int lo = g2m_off[g * kWave], hi = g2m_off[(g + 1) * kWave];
-        double min_arrival = 1e100;
+        int min_rank = 0x7FFFFFFF;
         int pick = -1;
         for (int x = lo; x < hi; ++x) {
             const int m = g2m_idx[(size_t)x * kWave];
-            if (qlen(m) > 0) {
-                const double t = a.mq_t[mq_off[m] + head[m * kWave]];
-                if (t < min_arrival) {
-                    min_arrival = t;
-                    pick = m;
-                }
+            const int rk = hrank[m * kWave];
+            if (qlen(m) > 0 && rk < min_rank) {  // strictly earlier arrival; ties keep the earlier-listed model
+                min_rank = rk;
+                pick = m;
             }
         }
         return pick;
@@ -133,34 +161,46 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         const int stages = (int)desc_stages_m1(d) + 1;
         double *gclk = clk + (desc_last_slot(d) - desc_stages_m1(d)) * kWave;
         for (;;) {
-            const float *lat_mg = a.lat + ((size_t)m * a.lat_row + desc_lat_off(d)) * NB;
+            const float *lat_mg = lat_tab + ((size_t)m * a.lat_row + desc_lat_off(d)) * NB;
             const int64_t base = mq_off[m];
-            // drop heads that cannot meet their deadline even alone (:677-686)
+            // drop heads that cannot meet their deadline even alone (:677-686).  The finish time of a
+            // batch of one does not depend on which request it is, so it is computed once; the
+            // deadlines of up to four heads are fetched together.
+            double alone = t0;
+            for (int k = 0; k < stages; ++k) alone = dmax(gclk[k * kWave], alone) + (double)lat_mg[(size_t)k * NB];
+            alone += overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
             bool found = false;
             int64_t first = 0;
-            while (qlen(m) > 0) {
-                const int64_t q = base + head[m * kWave];
-                head[m * kWave] += 1u;
-                if (check_slo(t0, gclk, stages, lat_mg, 0, a.mq_dl[q])) {
-                    found = true;
-                    first = q;
-                    break;
-                }
-                if (want_group) group_req[g * kWave] += 1;
-                if (want_req) {
-                    const int32_t r = a.mq_idx[q];
-                    fin_out[(size_t)r * kWave] = a.mq_t[q];
-                    good_out[(size_t)r * kWave] = 0;
+            double deadline = 0.0;
+            while (!found && qlen(m) > 0) {
+                const int64_t q0 = base + head[m * kWave];
+                const int avail = qlen(m) < 4 ? qlen(m) : 4;
+                double dl[4];
+                for (int k = 0; k < 4; ++k) dl[k] = a.mq[q0 + (k < avail ? k : avail - 1)].dl;
+                for (int k = 0; k < avail; ++k) {
+                    head[m * kWave] += 1u;
+                    if (alone <= dl[k]) {
+                        found = true;
+                        first = q0 + k;
+                        deadline = dl[k];
+                        break;
+                    }
+                    if (want_group) group_req[g * kWave] += 1;
+                    if (want_req) {
+                        const MqEntry e = a.mq[q0 + k];
+                        fin_out[(size_t)e.idx * kWave] = e.t;
+                        good_out[(size_t)e.idx * kWave] = 0;
+                    }
                 }
             }
             if (!found) {  // :709-713
+                hrank[m * kWave] = a.mq[base + head[m * kWave]].rank;
                 m = select_model(g);
                 if (m < 0) return;
                 continue;
             }
             // grow the batch while the first request still meets its deadline (:693-702)
             int bs = 1;
-            const double deadline = a.mq_dl[first];
             for (int b = 1; b < NB; ++b) {
                 const int cand = a.batch_sizes[b];
                 if (cand - 1 > qlen(m)) break;
@@ -175,17 +215,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 gclk[k * kWave] = t;
             }
             const double idle_at = gclk[0];
+            head[m * kWave] += (uint32_t)(bs - 1);  // the batch is the arrivals first .. first+bs-1 of the model
+            hrank[m * kWave] = a.mq[first + bs].rank;
             for (int u = 0; u < bs; ++u) {
-                int64_t q = first;
-                if (u > 0) {
-                    q = base + head[m * kWave];
-                    head[m * kWave] += 1u;
-                }
-                lat_sum += t - a.mq_t[q];
+                const MqEntry e = a.mq[first + u];
+                lat_sum += t - e.t;
                 if (want_req) {
-                    const int32_t r = a.mq_idx[q];
-                    fin_out[(size_t)r * kWave] = t;
-                    good_out[(size_t)r * kWave] = 1;
+                    fin_out[(size_t)e.idx * kWave] = t;
+                    good_out[(size_t)e.idx * kWave] = 1;
                 }
             }
             n_good += bs;
@@ -201,6 +238,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             ev_t[hn * kWave] = idle_at;
             ev_g[hn * kWave] = g;
             hn += 1;
+            next_due = fmin(next_due, idle_at);
             return;
         }
     };
@@ -229,21 +267,36 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         ev_g[e * kWave] = ev_g[hn * kWave];
     };
 
+    auto refresh_due = [&]() {
+        double d = __builtin_inf();
+        for (int e = 0; e < hn; ++e) d = fmin(d, ev_t[e * kWave]);
+        next_due = d;
+    };
+
     for (int64_t i = 0; i < R; ++i) {
-        const Req r = reqs[i];
-        const double tstamp = r.t;
-        const int m = uniform_i(r.m);
+        // requests are fetched 64 at a time (one coalesced load) and handed out lane by lane
+        if ((i & (kWave - 1)) == 0) {
+            const int64_t at = i + lane < R ? i + lane : R - 1;
+            blk_req = reqs[at];
+        }
+        const int j = (int)(i & (kWave - 1));
+        const double tstamp = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(blk_req.t), j),
+                                               __builtin_amdgcn_readlane(__double2loint(blk_req.t), j));
+        const int m = __builtin_amdgcn_readlane(blk_req.m, j);
 
         // ---- idle events that are due (:739-744)
-        while (!dead && hn > 0) {
-            const int e = min_event();
-            if (!(ev_t[e * kWave] <= tstamp)) break;
-            double ti;
-            uint32_t g;
-            pop_event(e, ti, g);
-            const int m2 = select_model(g);
-            if (m2 < 0) break;  // the popped event is dropped, later due events stay (:742-743)
-            handle(ti, m2, g);
+        if (!dead && next_due <= tstamp) {
+            while (!dead && hn > 0) {
+                const int e = min_event();
+                if (!(ev_t[e * kWave] <= tstamp)) break;
+                double ti;
+                uint32_t g;
+                pop_event(e, ti, g);
+                const int m2 = select_model(g);
+                if (m2 < 0) break;  // the popped event is dropped, later due events stay (:742-743)
+                handle(ti, m2, g);
+            }
+            refresh_due();
         }
 
         // ---- the arrival (:746-778)
