@@ -27,6 +27,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 FP64_VECTOR_PEAK_FMA_TFLOPS = 78.6   # MI355X published fp64 vector peak, FMA counted as 2
 FP64_NON_FMA_PEAK_TOPS = 39.3        # the path has only add/max/compare: half of the above
+LDS_PEAK_GBPS = 256 * 128 * 2.4      # 256 CUs x 128 B/clk x 2.4 GHz
 
 
 def log(*a):
@@ -155,8 +156,21 @@ def main():
     # scaled by a 1 GiB device copy): only known for the workload those runs used.
     traffic = None
     if (cfg.index == 4 and args.placements is None and args.seeds is None and args.flags == "scores"):
-        traffic = {"bytes_per_launch": 1.438e11 + 1.5e6, "source": "profiles/sim_mixed_kernel_cfg4.md",
-                   "algorithmic_bytes": info["stream_bytes"] + info["table_bytes"] + 12 * lanes}
+        traffic = 1.438e11 + 1.5e6      # bytes; profiles/sim_mixed_kernel_cfg4.md
+
+    hbm_bytes = info["stream_bytes"] + info["table_bytes"] + 12 * lanes
+    # dispatched requests = evaluations whose model has a replica: every one costs 3 operations beyond clocks
+    dispatched = None
+    if total_ops is not None:
+        hosted = np.zeros((B, cfg.num_models), bool)
+        for p, pl in enumerate(cfg.placements):
+            for ms in pl.group_models:
+                hosted[p, list(ms)] = True
+        per_model = np.zeros(cfg.num_models)
+        for st in streams:
+            ids = st.model_ids[st.model_ids >= 0]
+            per_model += np.bincount(ids, minlength=cfg.num_models)
+        dispatched = float((hosted * per_model[None, :]).sum())
 
     result = {
         "metric": "simulated request x placement evals/sec",
@@ -189,10 +203,16 @@ def main():
             "ops_per_launch": total_ops,
             "ops_per_eval": None if total_ops is None else total_ops / evals_per_step,
             "traffic": traffic,
-            "hbm_algorithmic_GBps": (info["stream_bytes"] * info["waves"] / max(len(seeds), 1)
-                                     + info["table_bytes"] * len(seeds)) / kernel_s / 1e9,
             "note": "fp64 add/max/compare only (no FMA): peak = published 78.6 TFLOP/s / 2; "
                     "achieved counts 2*stages+replicas+3 per dispatched request",
+            # the two other ceilings of this path, for the record: compulsory HBM bytes (streams once per
+            # wavefront group + tables + results) and algorithmic LDS bytes (8 per clock read or written:
+            # 2*stages + replicas per dispatched request) against 8 TB/s and 256 CUs x 128 B/clk x 2.4 GHz
+            "hbm": {"achieved_GBps": hbm_bytes / kernel_s / 1e9, "peak_GBps": 8000.0,
+                    "frac": hbm_bytes / kernel_s / 8e12, "bytes_per_launch": hbm_bytes},
+            "lds": None if total_ops is None else {
+                "achieved_GBps": 8.0 * (total_ops - 3 * dispatched) / kernel_s / 1e9, "peak_GBps": LDS_PEAK_GBPS,
+                "frac": 8.0 * (total_ops - 3 * dispatched) / kernel_s / 1e9 / LDS_PEAK_GBPS},
         },
     }
 
