@@ -230,6 +230,19 @@ def test_tile_classes_and_stream_segments(eng, monkeypatch, flags, segments):
             assert out["fp_ops"][s].sum() == ref["fp_ops"]
 
 
+def test_eight_wavefronts_per_workgroup(eng, monkeypatch):
+    """Large batches of small placements run 8 wavefronts per workgroup (two per SIMD); forced here on
+    520 placements of configuration 2 (16 clock slots)."""
+    monkeypatch.setenv("MMSIM_WAVES_PER_CU", "8")
+    cfg = make_config(2, 520)
+    for flags in (0, ALL):
+        out, table, packed, streams, info = _run_config(eng, cfg, cfg.placements, [0, 3], flags)
+        assert info["tile_classes"] == 1 and info["waves"] == 18
+        for s, st in enumerate(streams):
+            ref = oracle_batch(st, table, packed, want_per_request=bool(flags))
+            assert_batch_matches(out, ref, s, packed[0], per_request=bool(flags), where=f"8 waves, seed {s}")
+
+
 def test_scores_only_mode_equals_full_mode(eng):
     cfg = make_config(2)
     a, *_ = _run_config(eng, cfg, cfg.placements, [0, 1], 0)
