@@ -173,6 +173,101 @@ def body_pow2(levels, flavour):
     return a
 
 
+F0 = 232      # f[i] = v[F0+2i : F0+2i+1]: finish time of a lane that ends at depth EXITS-like 1, 2, 4, 8, 16
+FSEL = 242    # v[FSEL:FSEL+1]: the lane's own finish time, selected from f[]
+
+
+def freg(i):
+    return f"v[{F0 + 2 * i}:{F0 + 2 * i + 1}]"
+
+
+def body_pow2_straight(levels):
+    """"PU" walk: one latency per (model, configuration), depths all powers of two.
+
+    EXEC is written seven times at most instead of once per phase and exit: which lanes reach depth
+    2, 4, 8, 16 is kept as four SGPR masks; the code is straight-line per wave depth D (the deepest
+    walking lane), every walking lane fetches and chains D levels (levels past a lane's own depth read
+    clocks that are not its group's and compute values nobody uses), the lane's own finish time is
+    selected with the masks, and only the commit narrows EXEC.  Clock reads are waited for one by one,
+    so the chain starts when the first arrives; the finish-time adds and selects sit in the issue slots
+    the dependent max/add chain leaves empty.
+    """
+    depths = [d for d in (1, 2, 4, 8, 16) if d <= levels]
+    masks = {1: "%[m1]", 2: "%[m2]", 4: "%[m4]", 8: "%[m8]"}     # lanes with depth > key
+    a = []
+    a.append("s_mov_b64 %[sv], exec")
+    a.append("v_mov_b32_e32 %[acc], 0")
+    a.append(narrow(0))
+    a.append("s_cbranch_execz .Lmmsim_end_%=")
+    for e in depths[:-1]:
+        a.append(f"v_cmp_le_i32_e64 {masks[e]}, {e}, %[walk]")
+    a.append(f"ds_read_b64 {creg(0)}, %[cb]")
+    for e in depths[:-1]:                       # the wave's depth is the first e nobody goes beyond
+        a.append(f"s_cmp_eq_u64 {masks[e]}, 0")
+        a.append(f"s_cbranch_scc1 .Lmmsim_d{e}_%=")
+    for D in reversed(depths):                  # deepest first: falls through from the dispatch
+        a.append(f".Lmmsim_d{D}_%=:")
+        reads = pairs(1, D) if D > 1 else []
+        for n, k in reads:
+            if n == 2:
+                a.append(f"ds_read2st64_b64 v[{C0 + 2 * k}:{C0 + 2 * k + 3}], %[cb] offset0:{k} offset1:{k + 1}")
+            else:
+                a.append(f"ds_read_b64 {creg(k)}, %[cb] offset:{512 * k}")
+        # reads return in order: level k is there when at most (reads after it) are outstanding
+        arrive = {0: len(reads)}
+        for i, (n, k) in enumerate(reads):
+            for kk in range(k, k + n):
+                arrive[kk] = len(reads) - 1 - i
+        fill = []                               # independent instructions to drop into the chain's gaps
+        waited = None
+        for k in range(D):
+            if arrive[k] != waited:
+                a.append(f"s_waitcnt lgkmcnt({arrive[k]})")
+                waited = arrive[k]
+            prev = "%[ts]" if k == 0 else creg(k - 1)
+            a.append(f"v_max_f64 {creg(k)}, {prev}, {creg(k)}")
+            if fill:
+                a.append(fill.pop(0))
+            a.append(f"v_add_f64 {creg(k)}, {creg(k)}, %[lc]")
+            if fill:
+                a.append(fill.pop(0))
+            if k + 1 in depths:                 # a lane of depth k+1 finishes here
+                i = depths.index(k + 1)
+                fill.append(f"v_add_f64 {freg(i)}, {creg(k)}, %[oh]")
+                if i > 0:
+                    prev_sel = freg(0) if i == 1 else f"v[{FSEL}:{FSEL + 1}]"
+                    lo_prev, hi_prev = (F0, F0 + 1) if i == 1 else (FSEL, FSEL + 1)
+                    m = masks[depths[i - 1]]
+                    fill.append(f"v_cndmask_b32_e64 v{FSEL}, v{lo_prev}, v{F0 + 2 * i}, {m}")
+                    fill.append(f"v_cndmask_b32_e64 v{FSEL + 1}, v{hi_prev}, v{F0 + 2 * i + 1}, {m}")
+        a.extend(fill)
+        sel = freg(0) if D == 1 else f"v[{FSEL}:{FSEL + 1}]"
+        a.append(f"v_add_f64 %[lat], {sel}, -%[ts]")
+        a.append(f"v_mov_b64_e32 %[fin], {sel}")
+        if D != depths[0]:
+            a.append("s_branch .Lmmsim_decide_%=")
+    # ---- decide
+    a.append(".Lmmsim_decide_%=:")
+    a.append("v_cmpx_le_f64_e32 vcc, %[lat], %[slo]")
+    a.append("s_cbranch_execz .Lmmsim_end_%=")
+    a.append("v_mov_b32_e32 %[acc], 1")
+    a.append("v_add_u32_e32 %[ng], 1, %[ng]")
+    a.append("v_add_f64 %[ls], %[ls], %[lat]")
+    # ---- commit: accepted lanes, each its own depth
+    a.append(f"ds_write_b64 %[cb], {creg(0)}")
+    for e in depths[:-1]:
+        a.append(f"s_and_b64 exec, exec, {masks[e]}")
+        a.append("s_cbranch_scc0 .Lmmsim_end_%=")
+        for n, k in pairs(e, 2 * e):
+            if n == 2:
+                a.append(f"ds_write2st64_b64 %[cb], {creg(k)}, {creg(k + 1)} offset0:{k} offset1:{k + 1}")
+            else:
+                a.append(f"ds_write_b64 %[cb], {creg(k)} offset:{512 * k}")
+    a.append(".Lmmsim_end_%=:")
+    a.append("s_mov_b64 exec, %[sv]")
+    return a
+
+
 def clobbers(levels, flavour):
     regs = [f"v{C0 + i}" for i in range(2 * levels)]
     if flavour == "N":
@@ -187,12 +282,18 @@ def main():
     for levels in (4, 16):
         for flavour in ("U", "N", "PU", "PN"):
             name = f"MMSIM_WALK_{flavour}{levels}"
-            lines = body_pow2(levels, flavour[1]) if flavour[0] == "P" else body(levels, flavour)
+            if flavour == "PU":
+                lines = body_pow2_straight(levels)
+            else:
+                lines = body_pow2(levels, flavour[1]) if flavour[0] == "P" else body(levels, flavour)
+            straight = flavour == "PU"
             flavour = flavour[-1]
             out.append(f"#define {name}_TEXT \\")
             out.extend(f'    "{l}\\n" \\' for l in lines[:-1])
             out.append(f'    "{lines[-1]}\\n"')
             regs = clobbers(levels, flavour)
+            if straight:
+                regs += [f"v{F0 + i}" for i in range(10)] + [f"v{FSEL}", f"v{FSEL + 1}"]
             out.append(f"#define {name}_CLOBBERS " + ", ".join(f'"{r}"' for r in regs))
             out.append("")
     with open(os.path.join(here, "walk_asm.inc"), "w") as f:

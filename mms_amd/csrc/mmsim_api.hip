@@ -293,7 +293,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
 
     // ---- LDS budget
     const int32_t rmax_lds_bytes = (M + 15) & ~15;
-    size_t wave_bytes = 0, lat_bytes = 0;
+    size_t wave_bytes = 0, lat_bytes = 0, lds_tail = 0;
     int lat_in_lds = 1;
     int wpb = 0;
     int heap_cap = 0;
@@ -324,6 +324,14 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
         if (wave_bytes > (size_t)ctx->max_lds) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
         if ((size_t)ctx->max_lds > (size_t)kRepAddrMask) return fail(MMSIM_E_UNSUPPORTED, "LDS is larger than the descriptor's address field");
+        // The walk for power-of-two depths lets every walking lane read as many clock rows as the deepest
+        // one (up to 15 past its own group); the rows after the last wavefront's clocks must exist.  If that
+        // tail does not fit beside even one wavefront, the general walk is used.
+        lds_tail = pow2_depths ? (size_t)(b->smax_bucket - 1) * kSlotBytes : 0;
+        if (lat_bytes + wave_bytes + lds_tail > (size_t)ctx->max_lds) {
+            lds_tail = 0;
+            pow2_depths = false;
+        }
     } else {
         // per wavefront: descriptors | clocks | event times | queue heads | head ranks | event groups |
         // arrivals per model.  Events: the reference's heap holds about one entry per group plus a few
@@ -372,7 +380,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         std::vector<int32_t> fit(B, 1);
         if (!batching)
             for (int32_t p = 0; p < B; ++p) {
-                int32_t f = (int32_t)std::max<size_t>(1, std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / mixed_wave_bytes(by_class ? slots_of[p] : nslots)));
+                int32_t f = (int32_t)std::max<size_t>(1, std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes - lds_tail) / mixed_wave_bytes(by_class ? slots_of[p] : nslots)));
                 if (f > 4) f = f == 8 ? 8 : 4;  // beyond one per SIMD only the same number on every SIMD pays
                 fit[p] = f;
             }
@@ -406,10 +414,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 c.lds_bytes = (size_t)c.wpb * wave_bytes;
             } else {
                 c.wave_bytes = mixed_wave_bytes(c.nslots);
-                c.wpb = (int32_t)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes) / c.wave_bytes);
+                c.wpb = (int32_t)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes - lds_tail) / c.wave_bytes);
                 if (c.wpb > 4) c.wpb = c.wpb == 8 ? 8 : 4;
                 c.wpb = std::min(c.wpb, c.tile1 - c.tile0);
-                c.lds_bytes = lat_bytes + (size_t)c.wpb * c.wave_bytes;
+                c.lds_bytes = lat_bytes + (size_t)c.wpb * c.wave_bytes + lds_tail;
             }
             b->classes.push_back(c);
             tile_at = c.tile1;

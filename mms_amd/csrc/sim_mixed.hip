@@ -373,17 +373,18 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     const int walk = (has && !(bound > slo)) ? sm1 : -1;  // stages - 1 of lanes that walk
                     if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
                         // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
-                        uint64_t saved_exec;
+                        uint64_t saved_exec, mask1, mask2, mask4, mask8;  // masks: scratch of the power-of-two walk
                         int accepted;
                         double latency;
                         const uint32_t cb_addr = first_addr;
 #define MMSIM_WALK(NAME, LATNAME, LATVAL)                                                                           \
     asm volatile(NAME##_TEXT                                                                                        \
                  : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [fin] "=&v"(finish_time), [lat] "=&v"(latency),   \
-                   [ng] "+v"(n_good), [ls] "+v"(lat_sum)                                                            \
+                   [ng] "+v"(n_good), [ls] "+v"(lat_sum), [m1] "=&s"(mask1), [m2] "=&s"(mask2), [m4] "=&s"(mask4),  \
+                   [m8] "=&s"(mask8)                                                                                \
                  : [walk] "v"(walk), [cb] "v"(cb_addr), [LATNAME] "v"(LATVAL), [ts] "v"(tstamp), [slo] "v"(slo),    \
                    [oh] "s"(overhead)                                                                               \
-                 : "vcc", "memory", NAME##_CLOBBERS)
+                 : "vcc", "scc", "memory", NAME##_CLOBBERS)
                         if constexpr (UNIFORM) {
                             if (pow2) {
                                 if constexpr (SMAX == 4)
