@@ -21,11 +21,8 @@ Two flavours: "U" (one latency per (model, config): operand lc) and "N"
 (per-stage latencies read from the LDS table at byte address lb).
 
 The "P" variants are for batches whose pipeline depths are all powers of two
-(the usual case: group sizes and their inter-op splits are 1, 2, 4, 8, 16).
-Lanes can then only leave at depths 1, 2, 4, 8, so EXEC is narrowed there and
-nowhere else, clock slots move two at a time (ds_read2st64_b64 /
-ds_write2st64_b64: the 512-byte slot pitch is exactly the st64 stride), and the
-finish time is formed at the four exits instead of tracking t per level.
+(the usual case: group sizes and their inter-op splits are 1, 2, 4, 8, 16);
+see body_pow2_straight.
 """
 import os
 
@@ -112,88 +109,25 @@ def pairs(lo, hi):
     return out
 
 
-def body_pow2(levels, flavour):
-    # depth blocks [0,1) [1,2) [2,4) [4,8) [8,16): lanes inside a block all stay to its end
-    blocks = [(0, 1)] + [(e, min(2 * e, levels)) for e in EXITS if e < levels]
-    a = []
-    a.append("s_mov_b64 %[sv], exec")
-    a.append("v_mov_b32_e32 %[acc], 0")
-    # ---- fetch
-    for lo, hi in blocks:
-        a.append(narrow(lo))
-        a.append("s_cbranch_execz " + (".Lmmsim_end_%=" if lo == 0 else ".Lmmsim_fetched_%="))
-        for n, k in pairs(lo, hi):
-            if n == 2:
-                a.append(f"ds_read2st64_b64 v[{C0 + 2 * k}:{C0 + 2 * k + 3}], %[cb] offset0:{k} offset1:{k + 1}")
-            else:
-                a.append(f"ds_read_b64 {creg(k)}, %[cb]" + (f" offset:{512 * k}" if k else ""))
-        if flavour == "N":
-            for k in range(lo, hi):
-                a.append(f"ds_read_b32 v{L0 + k}, %[lb]" + (f" offset:{4 * k}" if k else ""))
-    a.append(".Lmmsim_fetched_%=:")
-    a.append("s_mov_b64 exec, %[sv]")
-    # ---- chain
-    for lo, hi in blocks:
-        a.append(narrow(lo))
-        if lo == 0:
-            a.append("s_waitcnt lgkmcnt(0)")
-        else:
-            a.append("s_cbranch_execz .Lmmsim_chained_%=")
-        for k in range(lo, hi):
-            prev = "%[ts]" if k == 0 else creg(k - 1)
-            a.append(f"v_max_f64 {creg(k)}, {prev}, {creg(k)}")
-            if flavour == "N":
-                a.append(f"v_cvt_f64_f32_e32 v[{TMP}:{TMP + 1}], v{L0 + k}")
-                a.append(f"v_add_f64 {creg(k)}, {creg(k)}, v[{TMP}:{TMP + 1}]")
-            else:
-                a.append(f"v_add_f64 {creg(k)}, {creg(k)}, %[lc]")
-        a.append(f"v_add_f64 %[fin], {creg(hi - 1)}, %[oh]")
-    a.append(".Lmmsim_chained_%=:")
-    a.append("s_mov_b64 exec, %[sv]")
-    # ---- decide
-    a.append(narrow(0))
-    a.append("v_add_f64 %[lat], %[fin], -%[ts]")
-    a.append("v_cmpx_le_f64_e32 vcc, %[lat], %[slo]")
-    a.append("s_cbranch_execz .Lmmsim_end_%=")
-    a.append("v_mov_b32_e32 %[acc], 1")
-    a.append("v_add_u32_e32 %[ng], 1, %[ng]")
-    a.append("v_add_f64 %[ls], %[ls], %[lat]")
-    # ---- commit
-    for lo, hi in blocks:
-        if lo > 0:
-            a.append(narrow(lo))
-            a.append("s_cbranch_execz .Lmmsim_end_%=")
-        for n, k in pairs(lo, hi):
-            if n == 2:
-                a.append(f"ds_write2st64_b64 %[cb], {creg(k)}, {creg(k + 1)} offset0:{k} offset1:{k + 1}")
-            else:
-                a.append(f"ds_write_b64 %[cb], {creg(k)}" + (f" offset:{512 * k}" if k else ""))
-    a.append(".Lmmsim_end_%=:")
-    a.append("s_mov_b64 exec, %[sv]")
-    return a
+FT = 250      # v[FT:FT+1]: finish time of a lane that would end at the level just computed
+FSEL = 252    # v[FSEL:FSEL+1]: the lane's own finish time
 
 
-F0 = 232      # f[i] = v[F0+2i : F0+2i+1]: finish time of a lane that ends at depth EXITS-like 1, 2, 4, 8, 16
-FSEL = 242    # v[FSEL:FSEL+1]: the lane's own finish time, selected from f[]
-
-
-def freg(i):
-    return f"v[{F0 + 2 * i}:{F0 + 2 * i + 1}]"
-
-
-def body_pow2_straight(levels):
-    """"PU" walk: one latency per (model, configuration), depths all powers of two.
+def body_pow2_straight(levels, flavour):
+    """"P" walks: depths all powers of two.
 
     EXEC is written seven times at most instead of once per phase and exit: which lanes reach depth
     2, 4, 8, 16 is kept as four SGPR masks; the code is straight-line per wave depth D (the deepest
     walking lane), every walking lane fetches and chains D levels (levels past a lane's own depth read
-    clocks that are not its group's and compute values nobody uses), the lane's own finish time is
-    selected with the masks, and only the commit narrows EXEC.  Clock reads are waited for one by one,
-    so the chain starts when the first arrives; the finish-time adds and selects sit in the issue slots
-    the dependent max/add chain leaves empty.
+    clocks and latencies that are not its group's and compute values nobody uses), the lane's own
+    finish time is selected with the masks, and only the commit narrows EXEC.  LDS reads are waited for
+    one by one, so the chain starts when the first arrives; the finish-time adds and selects sit in the
+    issue slots the dependent max/add chain leaves empty.
     """
     depths = [d for d in (1, 2, 4, 8, 16) if d <= levels]
     masks = {1: "%[m1]", 2: "%[m2]", 4: "%[m4]", 8: "%[m8]"}     # lanes with depth > key
+    fsel = f"v[{FSEL}:{FSEL + 1}]"
+    ft = f"v[{FT}:{FT + 1}]"
     a = []
     a.append("s_mov_b64 %[sv], exec")
     a.append("v_mov_b32_e32 %[acc], 0")
@@ -202,48 +136,61 @@ def body_pow2_straight(levels):
     for e in depths[:-1]:
         a.append(f"v_cmp_le_i32_e64 {masks[e]}, {e}, %[walk]")
     a.append(f"ds_read_b64 {creg(0)}, %[cb]")
+    if flavour == "N":
+        a.append(f"ds_read_b32 v{L0}, %[lb]")
     for e in depths[:-1]:                       # the wave's depth is the first e nobody goes beyond
         a.append(f"s_cmp_eq_u64 {masks[e]}, 0")
         a.append(f"s_cbranch_scc1 .Lmmsim_d{e}_%=")
     for D in reversed(depths):                  # deepest first: falls through from the dispatch
         a.append(f".Lmmsim_d{D}_%=:")
-        reads = pairs(1, D) if D > 1 else []
-        for n, k in reads:
+        # reads in issue order, each with the levels it brings (clock k: ("c", k), latency k: ("l", k))
+        issued = [[("c", 0)]] + ([[("l", 0)]] if flavour == "N" else [])
+        for n, k in (pairs(1, D) if D > 1 else []):
             if n == 2:
                 a.append(f"ds_read2st64_b64 v[{C0 + 2 * k}:{C0 + 2 * k + 3}], %[cb] offset0:{k} offset1:{k + 1}")
             else:
                 a.append(f"ds_read_b64 {creg(k)}, %[cb] offset:{512 * k}")
-        # reads return in order: level k is there when at most (reads after it) are outstanding
-        arrive = {0: len(reads)}
-        for i, (n, k) in enumerate(reads):
-            for kk in range(k, k + n):
-                arrive[kk] = len(reads) - 1 - i
+            issued.append([("c", kk) for kk in range(k, k + n)])
+            if flavour == "N":
+                for kk in range(k, k + n):
+                    a.append(f"ds_read_b32 v{L0 + kk}, %[lb] offset:{4 * kk}")
+                    issued.append([("l", kk)])
+        # reads return in order: an item is there when at most (reads issued after it) are outstanding
+        arrive = {}
+        for i, items in enumerate(issued):
+            for it in items:
+                arrive[it] = len(issued) - 1 - i
         fill = []                               # independent instructions to drop into the chain's gaps
-        waited = None
+        waited = 99
         for k in range(D):
-            if arrive[k] != waited:
-                a.append(f"s_waitcnt lgkmcnt({arrive[k]})")
-                waited = arrive[k]
+            need = arrive[("c", k)] if flavour == "U" else min(arrive[("c", k)], arrive[("l", k)])
+            need = min(need, 15)                # the counter field has four bits; waiting for fewer is only stricter
+            if need < waited:
+                a.append(f"s_waitcnt lgkmcnt({need})")
+                waited = need
             prev = "%[ts]" if k == 0 else creg(k - 1)
             a.append(f"v_max_f64 {creg(k)}, {prev}, {creg(k)}")
-            if fill:
+            if flavour == "N":
+                a.append(f"v_cvt_f64_f32_e32 v[{TMP}:{TMP + 1}], v{L0 + k}")
+            elif fill:
                 a.append(fill.pop(0))
-            a.append(f"v_add_f64 {creg(k)}, {creg(k)}, %[lc]")
+            a.append(f"v_add_f64 {creg(k)}, {creg(k)}, " + (f"v[{TMP}:{TMP + 1}]" if flavour == "N" else "%[lc]"))
             if fill:
                 a.append(fill.pop(0))
             if k + 1 in depths:                 # a lane of depth k+1 finishes here
+                a.extend(fill)                  # the shared temporary is reused: flush what still reads it
+                fill = []
                 i = depths.index(k + 1)
-                fill.append(f"v_add_f64 {freg(i)}, {creg(k)}, %[oh]")
-                if i > 0:
-                    prev_sel = freg(0) if i == 1 else f"v[{FSEL}:{FSEL + 1}]"
-                    lo_prev, hi_prev = (F0, F0 + 1) if i == 1 else (FSEL, FSEL + 1)
+                if i == 0:
+                    fill.append(f"v_add_f64 {fsel}, {creg(k)}, %[oh]")
+                else:
                     m = masks[depths[i - 1]]
-                    fill.append(f"v_cndmask_b32_e64 v{FSEL}, v{lo_prev}, v{F0 + 2 * i}, {m}")
-                    fill.append(f"v_cndmask_b32_e64 v{FSEL + 1}, v{hi_prev}, v{F0 + 2 * i + 1}, {m}")
+                    fill.append(f"v_add_f64 {ft}, {creg(k)}, %[oh]")
+                    fill.append(f"v_cndmask_b32_e64 v{FSEL}, v{FSEL}, v{FT}, {m}")
+                    fill.append(f"v_cndmask_b32_e64 v{FSEL + 1}, v{FSEL + 1}, v{FT + 1}, {m}")
         a.extend(fill)
-        sel = freg(0) if D == 1 else f"v[{FSEL}:{FSEL + 1}]"
-        a.append(f"v_add_f64 %[lat], {sel}, -%[ts]")
-        a.append(f"v_mov_b64_e32 %[fin], {sel}")
+        a.append(f"v_add_f64 %[lat], {fsel}, -%[ts]")
+        a.append(f"v_mov_b64_e32 %[fin], {fsel}")
         if D != depths[0]:
             a.append("s_branch .Lmmsim_decide_%=")
     # ---- decide
@@ -282,18 +229,15 @@ def main():
     for levels in (4, 16):
         for flavour in ("U", "N", "PU", "PN"):
             name = f"MMSIM_WALK_{flavour}{levels}"
-            if flavour == "PU":
-                lines = body_pow2_straight(levels)
-            else:
-                lines = body_pow2(levels, flavour[1]) if flavour[0] == "P" else body(levels, flavour)
-            straight = flavour == "PU"
+            straight = flavour[0] == "P"
             flavour = flavour[-1]
+            lines = body_pow2_straight(levels, flavour) if straight else body(levels, flavour)
             out.append(f"#define {name}_TEXT \\")
             out.extend(f'    "{l}\\n" \\' for l in lines[:-1])
             out.append(f'    "{lines[-1]}\\n"')
             regs = clobbers(levels, flavour)
             if straight:
-                regs += [f"v{F0 + i}" for i in range(10)] + [f"v{FSEL}", f"v{FSEL + 1}"]
+                regs += [f"v{FT}", f"v{FT + 1}", f"v{FSEL}", f"v{FSEL + 1}"]
             out.append(f"#define {name}_CLOBBERS " + ", ".join(f'"{r}"' for r in regs))
             out.append("")
     with open(os.path.join(here, "walk_asm.inc"), "w") as f:
