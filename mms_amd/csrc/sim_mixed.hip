@@ -308,33 +308,35 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 // ---- choose the replica group: strictly smallest last-stage clock (:590-598).
                 //      One LDS round trip fetches, for every listed replica, the clock of its last
                 //      stage and the latency of its last stage (needed by the early-reject bound).
-                double best = 1e100;
-                uint32_t sel = kEmpty;
-                float lsel = 0.0f;
-                auto consider = [&](uint32_t d, double c, float l) {
-                    const bool better = c < best;  // empty entries read a clock that is +inf
-                    best = vmin(best, c);
-                    sel = better ? d : sel;
-                    lsel = better ? l : lsel;
+                // Strictly smallest clock, first listed wins ties: a tournament whose left side wins ties
+                // picks the same entry as the reference's left-to-right scan, in log2 dependent steps.
+                // Entries past a lane's own replicas are empty descriptors, whose clock reads +inf.
+                struct Cand {
+                    double c;
+                    uint32_t d;
+                    float l;
                 };
-                // Scan 4 or 8 list entries without branching: entries past a lane's own
-                // replicas are empty descriptors, whose reads are harmless and never win.
+                auto first_min = [](const Cand &x, const Cand &y) {
+                    const bool right = y.c < x.c;
+                    return Cand{vmin(x.c, y.c), right ? y.d : x.d, right ? y.l : x.l};
+                };
+                Cand win{__builtin_inf(), kEmpty, 0.0f};
                 auto scan = [&](auto NJ) {
                     constexpr int nj = decltype(NJ)::value;
-                    double cl[nj];
-                    float ll[nj];
+                    Cand k[nj];
                     static_while<0, nj>([&](auto J) {
                         constexpr int j = decltype(J)::value;
-                        const uint32_t d = pick_desc<j>(cur.da[u], cur.db[u]);
-                        cl[j] = lds_f64(rep_addr(d));
-                        ll[j] = lrow_m[rep_lat_last(d)];
+                        k[j].d = pick_desc<j>(cur.da[u], cur.db[u]);
+                        k[j].c = lds_f64(rep_addr(k[j].d));
+                        k[j].l = lrow_m[rep_lat_last(k[j].d)];
                         return true;
                     });
-                    static_while<0, nj>([&](auto J) {
-                        constexpr int j = decltype(J)::value;
-                        consider(pick_desc<j>(cur.da[u], cur.db[u]), cl[j], ll[j]);
-                        return true;
-                    });
+                    const Cand a01 = first_min(k[0], k[1]), a23 = first_min(k[2], k[3]);
+                    win = first_min(a01, a23);
+                    if constexpr (nj == 8) {
+                        const Cand a45 = first_min(k[4], k[5]), a67 = first_min(k[6], k[7]);
+                        win = first_min(win, first_min(a45, a67));
+                    }
                 };
                 if (n > 4)
                     scan(Idx<8>{});
@@ -344,9 +346,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
                     for (int j = RREG; j < n; ++j) {
                         const uint32_t d = row[(size_t)(j - RREG) * kWave];
-                        consider(d, lds_f64(rep_addr(d)), lrow_m[rep_lat_last(d)]);
+                        win = first_min(win, Cand{lds_f64(rep_addr(d)), d, lrow_m[rep_lat_last(d)]});
                     }
                 }
+                // a clock that is infinite (a group that served a request with infinite latency) is never
+                // chosen (:590-598: "tmp < min_device_clock" with min_device_clock starting at inf)
+                const double best = win.c;
+                const uint32_t sel = best < 1e100 ? win.d : kEmpty;
+                const float lsel = win.l;
                 const bool has = (int32_t)sel >= 0;
                 const int sm1 = has ? (int)rep_stages_m1(sel) : -1;  // stages - 1
                 const uint32_t last_addr = rep_addr(sel);            // the lane's +inf clock when there is no replica
