@@ -64,7 +64,7 @@ def main():
                     help="synthetic configuration 1..5 (4 is the headline; 5 runs the batching simulator)")
     ap.add_argument("--placements", type=int, default=None, help="truncate the candidate list")
     ap.add_argument("--seeds", type=int, default=None, help="use only the first N arrival seeds")
-    ap.add_argument("--cpu-sample", type=int, default=1024, help="placements timed on the CPU oracle")
+    ap.add_argument("--cpu-sample", type=int, default=2048, help="placements timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="also launch one plain device copy of BYTES (read BYTES, write BYTES) so that "

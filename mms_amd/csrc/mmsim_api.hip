@@ -388,8 +388,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         for (int32_t p = 0; p < B; ++p) order[p] = p;
         std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
             if (fit[x] != fit[y]) return fit[x] > fit[y];
-            if (deepest[x] != deepest[y]) return deepest[x] < deepest[y];
-            return expected[x] < expected[y];
+            // deepest first: their wavefronts take longest, so they are launched first and the short ones
+            // fill the CUs as they free up
+            if (deepest[x] != deepest[y]) return deepest[x] > deepest[y];
+            return expected[x] > expected[y];
         });
         b->pos.assign(B, 0);
         int32_t tile_at = 0;
