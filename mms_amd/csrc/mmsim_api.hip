@@ -334,9 +334,11 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
     } else {
         // per wavefront: descriptors | clocks | event times | queue heads | head ranks | event groups |
-        // arrivals per model.  Events: the reference's heap holds about one entry per group plus a few
+        // arrivals per model | offsets of the models' arrival lists | batch sizes.  Events: the reference's heap holds about one entry per group plus a few
         // stale ones (most seen: G+3); provision min(2*G+8, G+16) if that fits, never less than G+4.
-        const size_t fixed = (size_t)(Gmax + 1) * kWave * 4 + (size_t)nslots * kWave * 8 + (size_t)2 * M * kWave * 4 + (((size_t)M * 4 + 15) & ~(size_t)15);
+        const size_t fixed = (size_t)(Gmax + 1) * kWave * 4 + (size_t)nslots * kWave * 8 + (size_t)2 * M * kWave * 4 +
+                             (((size_t)M * 4 + 15) & ~(size_t)15) + (((size_t)(M + 1) * 8 + 15) & ~(size_t)15) +
+                             (((size_t)t->NB * 4 + 15) & ~(size_t)15);
         for (heap_cap = std::min(2 * Gmax + 8, Gmax + 16); heap_cap >= Gmax + 4; --heap_cap) {
             wave_bytes = (fixed + (size_t)heap_cap * kWave * 12 + 15) & ~(size_t)15;
             if (wave_bytes <= (size_t)ctx->max_lds) break;

@@ -75,6 +75,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     o += (size_t)a.heap_cap * kWave * 4;
     volatile uint32_t *arrived = reinterpret_cast<volatile uint32_t *>(mine + o);  // [M], same for all lanes
     o += ((size_t)M * 4 + 15) & ~(size_t)15;
+    int64_t *mq_off = reinterpret_cast<int64_t *>(mine + o);  // [M+1] this seed's offsets into mq
+    o += ((size_t)(M + 1) * 8 + 15) & ~(size_t)15;
+    int32_t *bsz = reinterpret_cast<int32_t *>(mine + o);  // [NB] batch sizes
+    o += ((size_t)NB * 4 + 15) & ~(size_t)15;
     uint16_t *g2m_off_lds = reinterpret_cast<uint16_t *>(mine + o) + lane;  // [Gmax+1][64]
     o += (size_t)(Gmax + 1) * kWave * 2;
     uint16_t *g2m_idx_lds = reinterpret_cast<uint16_t *>(mine + o) + lane;  // [members_max][64]
@@ -86,6 +90,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
         {
             const int64_t *mo = a.mq_off + (size_t)seed * (M + 1);
+            for (int m = lane; m <= M; m += kWave) mq_off[m] = mo[m];
+            for (int q = lane; q < NB; q += kWave) bsz[q] = a.batch_sizes[q];
             for (int m = 0; m < M; ++m) {
                 head[m * kWave] = 0u;
                 hrank[m * kWave] = a.mq[mo[m]].rank;  // of the model's first arrival (the padding entry if it has none)
@@ -106,7 +112,6 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const int64_t off = a.stream_off[seed];
     const int64_t R = a.stream_off[seed + 1] - off;
     const Req *__restrict__ reqs = a.streams + off;
-    const int64_t *__restrict__ mq_off = a.mq_off + (size_t)seed * (M + 1);
     const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * M * kWave + lane;
     const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * M * a.rep_extra * kWave + lane;
     // generic pointers: LDS copies when they fit, else the tables in global memory
@@ -128,6 +133,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 
     const uint32_t none = (uint32_t)Gmax;
     Req blk_req = {0.0, -1, 0.0f};  // this lane's request of the current block of 64
+    uint64_t g8_next = 0;          // replica list (eight group bytes) of the next request's model, fetched ahead
 
     // queue length of a model this lane hosts
     auto qlen = [&](int m) -> int { return (int)(arrived[m] - head[m * kWave]); };
@@ -165,7 +171,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             const int64_t base = mq_off[m];
             // drop heads that cannot meet their deadline even alone (:677-686).  The finish time of a
             // batch of one does not depend on which request it is, so it is computed once; the
-            // deadlines of up to four heads are fetched together.
+            // deadlines of up to eight heads are fetched together.
             double alone = t0;
             for (int k = 0; k < stages; ++k) alone = dmax(gclk[k * kWave], alone) + (double)lat_mg[(size_t)k * NB];
             alone += overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
@@ -174,9 +180,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             double deadline = 0.0;
             while (!found && qlen(m) > 0) {
                 const int64_t q0 = base + head[m * kWave];
-                const int avail = qlen(m) < 4 ? qlen(m) : 4;
-                double dl[4];
-                for (int k = 0; k < 4; ++k) dl[k] = a.mq[q0 + (k < avail ? k : avail - 1)].dl;
+                const int avail = qlen(m) < 8 ? qlen(m) : 8;
+                double dl[8];
+                for (int k = 0; k < 8; ++k) dl[k] = a.mq[q0 + (k < avail ? k : avail - 1)].dl;
                 for (int k = 0; k < avail; ++k) {
                     head[m * kWave] += 1u;
                     if (alone <= dl[k]) {
@@ -202,7 +208,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             // grow the batch while the first request still meets its deadline (:693-702)
             int bs = 1;
             for (int b = 1; b < NB; ++b) {
-                const int cand = a.batch_sizes[b];
+                const int cand = bsz[b];
                 if (cand - 1 > qlen(m)) break;
                 if (!check_slo(t0, gclk, stages, lat_mg, ilog2i(cand), deadline)) break;
                 bs = cand;
@@ -217,12 +223,16 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             const double idle_at = gclk[0];
             head[m * kWave] += (uint32_t)(bs - 1);  // the batch is the arrivals first .. first+bs-1 of the model
             hrank[m * kWave] = a.mq[first + bs].rank;
-            for (int u = 0; u < bs; ++u) {
-                const MqEntry e = a.mq[first + u];
-                lat_sum += t - e.t;
-                if (want_req) {
-                    fin_out[(size_t)e.idx * kWave] = t;
-                    good_out[(size_t)e.idx * kWave] = 1;
+            for (int u0 = 0; u0 < bs; u0 += 8) {  // arrival times of up to eight members fetched together
+                double at[8];
+                for (int k = 0; k < 8; ++k) at[k] = a.mq[first + (u0 + k < bs ? u0 + k : bs - 1)].t;
+                for (int k = 0; k < 8 && u0 + k < bs; ++k) {
+                    lat_sum += t - at[k];
+                    if (want_req) {
+                        const int32_t r = a.mq[first + u0 + k].idx;
+                        fin_out[(size_t)r * kWave] = t;
+                        good_out[(size_t)r * kWave] = 1;
+                    }
                 }
             }
             n_good += bs;
@@ -275,14 +285,22 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 
     for (int64_t i = 0; i < R; ++i) {
         // requests are fetched 64 at a time (one coalesced load) and handed out lane by lane
-        if ((i & (kWave - 1)) == 0) {
+        const int j = (int)(i & (kWave - 1));
+        if (j == 0) {
             const int64_t at = i + lane < R ? i + lane : R - 1;
             blk_req = reqs[at];
+            const int m0 = __builtin_amdgcn_readlane(blk_req.m, 0);
+            g8_next = rep_tile[(size_t)(m0 < 0 ? 0 : m0) * kWave];
         }
-        const int j = (int)(i & (kWave - 1));
         const double tstamp = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(blk_req.t), j),
                                                __builtin_amdgcn_readlane(__double2loint(blk_req.t), j));
         const int m = __builtin_amdgcn_readlane(blk_req.m, j);
+        // the replica list of this request's model was fetched during the previous request; start the next one's
+        const uint64_t g8 = g8_next;
+        if (j != kWave - 1) {  // the first request of a block gets its list when the block is fetched
+            const int mn = __builtin_amdgcn_readlane(blk_req.m, j + 1);
+            g8_next = rep_tile[(size_t)(mn < 0 ? 0 : mn) * kWave];
+        }
 
         // ---- idle events that are due (:739-744)
         if (!dead && next_due <= tstamp) {
@@ -303,7 +321,6 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         bool queued = false;
         uint32_t gsel = none;
         if (m >= 0) {
-            const uint64_t g8 = rep_tile[(size_t)m * kWave];
             const bool hosted = (uint32_t)(g8 & 0xFFu) != none;
             if (hosted && !dead) {
                 // group with the strictly smallest last-stage clock (:760-770)
