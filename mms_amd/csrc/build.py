@@ -23,16 +23,19 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # one wavefront per SIMD is the rule for these kernels (LDS-bound occupancy), so instruction-level
-    # parallelism inside a wavefront is what hides latency: schedule for it (measured -7 % kernel time)
-    "-mllvm", "-amdgpu-sched-strategy=iterative-ilp",
     "-Wall", "-Wno-unused-command-line-argument",
 ]
 
 
+# One wavefront per SIMD is the rule for the plain simulator's kernel (LDS-bound occupancy), so
+# instruction-level parallelism inside a wavefront is what hides latency: schedule for it (measured
+# -7 % kernel time).  The batching kernel is built with the default scheduler (this one fails on it).
+SOURCE_FLAGS = {"sim_mixed.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"]}
+
+
 def _compile(src, extra, src_dir=HERE, obj_dir=OBJ_DIR):
     obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(src_dir, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *SOURCE_FLAGS.get(src, []), *extra, "-c", os.path.join(src_dir, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{proc.stdout}\n{proc.stderr}")

@@ -221,6 +221,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             if (col >= t->NB) return fail(MMSIM_E_INVALID, "tables: floor(log2(batch size)) must index a latency column");
         }
         if (t->M > 65535) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: more than 65535 models");
+        if (t->NB > kMaxLatencyColumns) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: more than 16 batch sizes");
     }
     const int32_t M = t->M, C = t->C, B = rl.B, Gmax = rl.Gmax;
     if (n_seeds < 1 || !wls) return fail(MMSIM_E_INVALID, "need at least one workload");
@@ -297,6 +298,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     int lat_in_lds = 1;
     int wpb = 0;
     int heap_cap = 0;
+    int blanes = kWave;  // batching simulator: lanes of a wavefront that simulate
     // Wavefronts per workgroup: no more than it takes to give every CU its share of the
     // batch (a small batch is spread over the CUs, one wavefront per workgroup), and
     // no more than fit in LDS.  MMSIM_WAVES_PER_CU (1..8) sets the number instead (tuning knob).
@@ -336,13 +338,35 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         // per wavefront: descriptors | clocks | event times | queue heads | head ranks | event groups |
         // arrivals per model | offsets of the models' arrival lists | batch sizes.  Events: the reference's heap holds about one entry per group plus a few
         // stale ones (most seen: G+3); provision min(2*G+8, G+16) if that fits, never less than G+4.
-        const size_t fixed = (size_t)(Gmax + 1) * kWave * 4 + (size_t)nslots * kWave * 8 + (size_t)2 * M * kWave * 4 +
-                             (((size_t)M * 4 + 15) & ~(size_t)15) + (((size_t)(M + 1) * 8 + 15) & ~(size_t)15) +
-                             (((size_t)t->NB * 4 + 15) & ~(size_t)15);
-        for (heap_cap = std::min(2 * Gmax + 8, Gmax + 16); heap_cap >= Gmax + 4; --heap_cap) {
-            wave_bytes = (fixed + (size_t)heap_cap * kWave * 12 + 15) & ~(size_t)15;
-            if (wave_bytes <= (size_t)ctx->max_lds) break;
+        auto size_for = [&](int lanes) {
+            const size_t fixed = (size_t)(Gmax + 1) * lanes * 4 + (size_t)nslots * lanes * 8 + (size_t)2 * M * lanes * 4 +
+                                 (((size_t)M * 4 + 15) & ~(size_t)15) + (((size_t)(M + 1) * 8 + 15) & ~(size_t)15) +
+                                 (((size_t)t->NB * 4 + 15) & ~(size_t)15);
+            // (a multiple of four: the kernel scans the list four slots at a time)
+            for (heap_cap = std::min(2 * Gmax + 8, Gmax + 16) & ~3; heap_cap >= Gmax + 4; heap_cap -= 4) {
+                wave_bytes = (fixed + (size_t)heap_cap * lanes * 12 + 15) & ~(size_t)15;
+                if (wave_bytes <= (size_t)ctx->max_lds) break;
+            }
+        };
+        // Simulations per wavefront.  The loops between two arrivals run per lane, so a wavefront takes as
+        // long as its slowest lane at every step, and its LDS footprint grows with its lanes.  When 64-lane
+        // wavefronts leave SIMDs without one (their state fills the CU's LDS, or the batch is small),
+        // narrower tiles are used: 32 or 16 lanes simulate, the others only help fetching requests.
+        blanes = kWave;
+        if (const char *env = std::getenv("MMSIM_BATCHING_LANES")) {
+            const int v = std::atoi(env);
+            if (v == 16 || v == 32 || v == 64) blanes = v;
+        } else {
+            const int64_t simds = 4 * (int64_t)std::max(1, ctx->prop.multiProcessorCount);
+            for (;;) {
+                size_for(blanes);
+                const int64_t per_cu = heap_cap >= Gmax + 4 ? std::min<int64_t>(4, (int64_t)ctx->max_lds / (int64_t)wave_bytes) : 0;
+                const int64_t waves = (int64_t)((B + blanes - 1) / blanes) * n_seeds;
+                if (blanes == 16 || (per_cu >= 4 && waves >= simds)) break;
+                blanes /= 2;
+            }
         }
+        size_for(blanes);
         if (heap_cap < Gmax + 4) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: per-wavefront state does not fit in LDS (too many models/stages/groups)");
         wpb = (int)std::min<size_t>(kMaxWavesPerBlockBatching, (size_t)ctx->max_lds / wave_bytes);
     }
@@ -406,10 +430,11 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             while (j < B && fit[order[j]] >= f) ++j;
             mmsim_batch::TileClass c;
             c.tile0 = tile_at;
-            c.tile1 = tile_at + (j - i + kWave - 1) / kWave;
+            const int32_t tl = batching ? blanes : kWave;  // placements per tile
+            c.tile1 = tile_at + (j - i + tl - 1) / tl;
             for (int32_t k = i; k < j; ++k) {
                 c.nslots = std::max(c.nslots, slots_of[order[k]]);
-                b->pos[order[k]] = c.tile0 * kWave + (k - i);
+                b->pos[order[k]] = (c.tile0 + (k - i) / tl) * kWave + (k - i) % tl;
             }
             if (batching) {
                 c.nslots = nslots;
@@ -588,7 +613,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     int batching_g2m_lds = 0;
     if (batching) {
         const size_t lat_b = (lat_nb.size() * sizeof(float) + 15) & ~(size_t)15;
-        const size_t g2m_b = ((size_t)(Gmax + 1) * kWave * 2 + (size_t)members_max * kWave * 2 + 15) & ~(size_t)15;
+        const size_t g2m_b = ((size_t)(Gmax + 1) * blanes * 2 + (size_t)members_max * blanes * 2 + 15) & ~(size_t)15;
         const size_t cap = (size_t)ctx->max_lds;
         int w = wpb;
         for (; w >= 1; --w)
@@ -787,6 +812,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         q.wave_lds_bytes = (int32_t)wave_bytes;
         q.lat_lds_bytes = (int32_t)batching_lat_lds;
         q.g2m_in_lds = batching_g2m_lds;
+        q.lane_stride = blanes;
         q.Rmax = b->Rmax;
         q.fixed_overhead = t->fixed_overhead;
         q.flags = flags;

@@ -152,6 +152,7 @@ struct BatchingArgs {
     int32_t wave_lds_bytes;
     int32_t lat_lds_bytes;       // > 0: the workgroup keeps a copy of lat in LDS (that many bytes, 16-aligned)
     int32_t g2m_in_lds;          // 1: each wavefront keeps its g2m_off / g2m_idx rows in LDS
+    int32_t lane_stride;         // 64, 32 or 16: lanes of a wavefront that simulate; pitch of the per-lane LDS arrays
     int64_t Rmax;
     double fixed_overhead;
     uint32_t flags;
@@ -175,5 +176,6 @@ hipError_t launch_sim_mixed(const MixedArgs &args, int smax_bucket, int waves_pe
 int smax_bucket_for(int smax);
 constexpr int kMaxWavesPerBlock = 8;          // plain simulator
 constexpr int kMaxWavesPerBlockBatching = 4;  // batching simulator
+constexpr int kMaxLatencyColumns = 16;       // batching simulator: batch sizes below 2^16
 
 }  // namespace mmsim

@@ -40,6 +40,16 @@ __device__ __forceinline__ int uniform_i(int v) { return __builtin_amdgcn_readfi
 __device__ __forceinline__ double dmax(double a, double b) { return b > a ? b : a; }
 __device__ __forceinline__ int ilog2i(int v) { return 31 - __clz(v); }
 
+typedef volatile __attribute__((address_space(3))) uint32_t lds_vu32;
+__device__ __forceinline__ lds_vu32 *as_lds_vu32(void *p) { return (lds_vu32 *)p; }
+
+// NBT: latency columns held in registers (the table's NB columns, rounded up to 4, 8 or 16).
+// LATLDS / G2MLDS: the latency table / the lists of each group's models are read from their LDS
+// copies.  These are compile-time choices so that every LDS access is a DS instruction: through a
+// generic pointer the compiler may fold a constant of the index (the 31 of 31 - clz(batch size)) into
+// the instruction's offset field, and the hardware picks the aperture from the base register alone,
+// which then lies below the LDS aperture for a table at the start of LDS.
+template <int NBT, bool LATLDS, bool G2MLDS>
 __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching_kernel(const BatchingArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
@@ -52,6 +62,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const int M = a.M, Gmax = a.Gmax, NB = a.NB;
+    const int LS = a.lane_stride;  // lanes of a wavefront that simulate (64, 32 or 16): pitch of the per-lane LDS arrays
 
     // ---- LDS: [latency table, shared, if it fits][per wavefront: group descriptors | clocks | event times |
     //      queue heads | head ranks | event groups | arrivals per model | models of each group, if they fit]
@@ -62,47 +73,54 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     }
     unsigned char *mine = lds_raw + a.lat_lds_bytes + wv * a.wave_lds_bytes;
     uint32_t *ginfo = reinterpret_cast<uint32_t *>(mine) + lane;
-    size_t o = (size_t)(Gmax + 1) * kWave * 4;
+    size_t o = (size_t)(Gmax + 1) * LS * 4;
     double *clk = reinterpret_cast<double *>(mine + o) + lane;
-    o += (size_t)a.nslots * kWave * 8;
+    o += (size_t)a.nslots * LS * 8;
     double *ev_t = reinterpret_cast<double *>(mine + o) + lane;
-    o += (size_t)a.heap_cap * kWave * 8;
+    o += (size_t)a.heap_cap * LS * 8;
     uint32_t *head = reinterpret_cast<uint32_t *>(mine + o) + lane;
-    o += (size_t)M * kWave * 4;
+    o += (size_t)M * LS * 4;
     int32_t *hrank = reinterpret_cast<int32_t *>(mine + o) + lane;  // rank of the arrival at head[m] (already known before it arrives)
-    o += (size_t)M * kWave * 4;
+    o += (size_t)M * LS * 4;
     uint32_t *ev_g = reinterpret_cast<uint32_t *>(mine + o) + lane;
-    o += (size_t)a.heap_cap * kWave * 4;
-    volatile uint32_t *arrived = reinterpret_cast<volatile uint32_t *>(mine + o);  // [M], same for all lanes
+    o += (size_t)a.heap_cap * LS * 4;
+    // [M], same for all lanes; written by lane 0 and read by all, hence volatile (and spelled as an LDS
+    // pointer: volatile accesses are not rewritten from generic to LDS by the compiler)
+    lds_vu32 *arrived = as_lds_vu32(mine + o);
     o += ((size_t)M * 4 + 15) & ~(size_t)15;
     int64_t *mq_off = reinterpret_cast<int64_t *>(mine + o);  // [M+1] this seed's offsets into mq
     o += ((size_t)(M + 1) * 8 + 15) & ~(size_t)15;
     int32_t *bsz = reinterpret_cast<int32_t *>(mine + o);  // [NB] batch sizes
     o += ((size_t)NB * 4 + 15) & ~(size_t)15;
     uint16_t *g2m_off_lds = reinterpret_cast<uint16_t *>(mine + o) + lane;  // [Gmax+1][64]
-    o += (size_t)(Gmax + 1) * kWave * 2;
+    o += (size_t)(Gmax + 1) * LS * 2;
     uint16_t *g2m_idx_lds = reinterpret_cast<uint16_t *>(mine + o) + lane;  // [members_max][64]
 
     const bool live = tile < a.tiles;
-    if (live) {
+    const bool sim = lane < LS;  // the other lanes of a narrow tile only help fetching requests
+    if (live && sim) {
         const uint32_t *gsrc = a.ginfo + (size_t)tile * (Gmax + 1) * kWave + lane;
-        for (int g = 0; g <= Gmax; ++g) ginfo[g * kWave] = gsrc[g * kWave];
-        for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
+        for (int g = 0; g <= Gmax; ++g) ginfo[g * LS] = gsrc[g * kWave];
+        for (int s = 0; s < a.nslots; ++s) clk[s * LS] = 0.0;
+        for (int e = 0; e < a.heap_cap; ++e) {  // unused event slots never win the minimum scan
+            ev_t[e * LS] = __builtin_inf();
+            ev_g[e * LS] = 0xFFFFFFFFu;
+        }
         {
             const int64_t *mo = a.mq_off + (size_t)seed * (M + 1);
-            for (int m = lane; m <= M; m += kWave) mq_off[m] = mo[m];
-            for (int q = lane; q < NB; q += kWave) bsz[q] = a.batch_sizes[q];
+            for (int m = lane; m <= M; m += LS) mq_off[m] = mo[m];
+            for (int q = lane; q < NB; q += LS) bsz[q] = a.batch_sizes[q];
             for (int m = 0; m < M; ++m) {
-                head[m * kWave] = 0u;
-                hrank[m * kWave] = a.mq[mo[m]].rank;  // of the model's first arrival (the padding entry if it has none)
+                head[m * LS] = 0u;
+                hrank[m * LS] = a.mq[mo[m]].rank;  // of the model's first arrival (the padding entry if it has none)
             }
         }
-        for (int m = lane; m < M; m += kWave) arrived[m] = 0u;
+        for (int m = lane; m < M; m += LS) arrived[m] = 0u;
         if (a.g2m_in_lds) {
             const uint16_t *osrc = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
             const uint16_t *isrc = a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
-            for (int g = 0; g <= Gmax; ++g) g2m_off_lds[g * kWave] = osrc[g * kWave];
-            for (int x = 0; x < a.members_max; ++x) g2m_idx_lds[x * kWave] = isrc[(size_t)x * kWave];
+            for (int g = 0; g <= Gmax; ++g) g2m_off_lds[g * LS] = osrc[g * kWave];
+            for (int x = 0; x < a.members_max; ++x) g2m_idx_lds[x * LS] = isrc[(size_t)x * kWave];
         }
     }
     __syncthreads();  // the latency table is complete; wavefronts run independently from here
@@ -114,10 +132,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const Req *__restrict__ reqs = a.streams + off;
     const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * M * kWave + lane;
     const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * M * a.rep_extra * kWave + lane;
-    // generic pointers: LDS copies when they fit, else the tables in global memory
-    const uint16_t *g2m_off = a.g2m_in_lds ? g2m_off_lds : a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
-    const uint16_t *g2m_idx = a.g2m_in_lds ? g2m_idx_lds : a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
-    const float *lat_tab = a.lat_lds_bytes > 0 ? lat_lds : a.lat;
+    const uint16_t *g2m_off_glb = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
+    const uint16_t *g2m_idx_glb = a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
+    auto g2m_off_at = [&](uint32_t g) -> int { return G2MLDS ? g2m_off_lds[g * LS] : g2m_off_glb[(size_t)g * kWave]; };
+    auto g2m_idx_at = [&](int x) -> int { return G2MLDS ? g2m_idx_lds[x * LS] : g2m_idx_glb[(size_t)x * kWave]; };
+    auto lat_at = [&](uint32_t i) -> float { return LATLDS ? lat_lds[i] : a.lat[i]; };
     int32_t *model_good = a.model_good + (size_t)wave * M * kWave + lane;
     int32_t *group_req = a.group_req + (size_t)wave * Gmax * kWave + lane;
     int32_t *group_good = a.group_good + (size_t)wave * Gmax * kWave + lane;
@@ -129,62 +148,91 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     double lat_sum = 0.0;
     int hn = 0;          // pending idle events of this lane
     double next_due = __builtin_inf();  // the earliest of them (+inf if none): arrivals before it skip the event list
-    int dead = 0;        // nonzero status: this lane stopped (out of event slots / unsupported input)
+    int dead = sim ? 0 : 1;  // nonzero: this lane simulates nothing (more): out of event slots, unsupported input, or a spare lane of a narrow tile
 
     const uint32_t none = (uint32_t)Gmax;
     Req blk_req = {0.0, -1, 0.0f};  // this lane's request of the current block of 64
     uint64_t g8_next = 0;          // replica list (eight group bytes) of the next request's model, fetched ahead
 
-    // queue length of a model this lane hosts
-    auto qlen = [&](int m) -> int { return (int)(arrived[m] - head[m * kWave]); };
-
     // :654-664 -- among the models of group g with a waiting request, the one whose head arrived first
     auto select_model = [&](uint32_t g) -> int {
-        const int lo = g2m_off[g * kWave], hi = g2m_off[(g + 1) * kWave];
+        const int lo = g2m_off_at(g), hi = g2m_off_at(g + 1u);
         int min_rank = 0x7FFFFFFF;
         int pick = -1;
-        for (int x = lo; x < hi; ++x) {
-            const int m = g2m_idx[(size_t)x * kWave];
-            const int rk = hrank[m * kWave];
-            if (qlen(m) > 0 && rk < min_rank) {  // strictly earlier arrival; ties keep the earlier-listed model
-                min_rank = rk;
-                pick = m;
+        for (int x0 = lo; x0 < hi; x0 += 4) {  // four models at a time: their reads overlap
+            int mm[4], rk[4];
+            uint32_t hd[4], ar[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) mm[u] = g2m_idx_at(x0 + u < hi ? x0 + u : hi - 1);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                rk[u] = hrank[mm[u] * LS];
+                hd[u] = head[mm[u] * LS];
+                ar[u] = arrived[mm[u]];
             }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                // strictly earlier arrival; ties keep the earlier-listed model
+                if (x0 + u < hi && (int)(ar[u] - hd[u]) > 0 && rk[u] < min_rank) {
+                    min_rank = rk[u];
+                    pick = mm[u];
+                }
         }
         return pick;
     };
 
-    // :666-672
-    auto check_slo = [&](double t0, const double *gclk, int stages, const float *lat_mg, int col, double deadline) -> bool {
-        double t = t0;
-        for (int k = 0; k < stages; ++k) t = dmax(gclk[k * kWave], t) + (double)lat_mg[(size_t)k * NB + col];
-        return (t + overhead) <= deadline;
+    // :666-672 without the final "+ overhead <= deadline": the time a batch started at t0 leaves the
+    // group's last stage, for every latency column at once (one pass over the stages, four stages per
+    // round of LDS reads)
+    auto batch_times = [&](double t0, const double *gclk, int stages, uint32_t lat_mg, double(&tb)[NBT]) {
+#pragma unroll
+        for (int b = 0; b < NBT; ++b) tb[b] = t0;
+        for (int k0 = 0; k0 < stages; k0 += 4) {
+            double c[4];
+            float l[4][NBT];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int k = k0 + u < stages ? k0 + u : stages - 1;
+                c[u] = gclk[k * LS];
+#pragma unroll
+                for (int b = 0; b < NBT; ++b) l[u][b] = lat_at(lat_mg + (uint32_t)(k * NB + (b < NB ? b : NB - 1)));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (k0 + u < stages) {
+#pragma unroll
+                    for (int b = 0; b < NBT; ++b) tb[b] = dmax(c[u], tb[b]) + (double)l[u][b];
+                }
+        }
     };
 
     // :706-732 with :674-704 inlined; the reference's recursion on "nothing servable" is the outer loop
     auto handle = [&](double t0, int m, uint32_t g) {
-        const uint32_t d = ginfo[g * kWave];
+        const uint32_t d = ginfo[g * LS];
         const int stages = (int)desc_stages_m1(d) + 1;
-        double *gclk = clk + (desc_last_slot(d) - desc_stages_m1(d)) * kWave;
+        double *gclk = clk + (desc_last_slot(d) - desc_stages_m1(d)) * LS;
         for (;;) {
-            const float *lat_mg = lat_tab + ((size_t)m * a.lat_row + desc_lat_off(d)) * NB;
+            const uint32_t lat_mg = ((uint32_t)m * (uint32_t)a.lat_row + desc_lat_off(d)) * (uint32_t)NB;  // the (model, group) rows of the table
             const int64_t base = mq_off[m];
+            const uint32_t arr = arrived[m];  // does not change while a lane is in here
+            uint32_t h = head[m * LS];        // arr - h > 0: the caller saw a waiting request
             // drop heads that cannot meet their deadline even alone (:677-686).  The finish time of a
             // batch of one does not depend on which request it is, so it is computed once; the
-            // deadlines of up to eight heads are fetched together.
-            double alone = t0;
-            for (int k = 0; k < stages; ++k) alone = dmax(gclk[k * kWave], alone) + (double)lat_mg[(size_t)k * NB];
-            alone += overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
+            // deadlines of up to eight heads are fetched together, the first eight ahead of that pass.
+            int64_t q0 = base + h;
+            int avail = (int)(arr - h) < 8 ? (int)(arr - h) : 8;
+            double dl[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) dl[k] = a.mq[q0 + (k < avail ? k : avail - 1)].dl;
+            double tb[NBT];
+            batch_times(t0, gclk, stages, lat_mg, tb);
+            const double alone = tb[0] + overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
             bool found = false;
             int64_t first = 0;
             double deadline = 0.0;
-            while (!found && qlen(m) > 0) {
-                const int64_t q0 = base + head[m * kWave];
-                const int avail = qlen(m) < 8 ? qlen(m) : 8;
-                double dl[8];
-                for (int k = 0; k < 8; ++k) dl[k] = a.mq[q0 + (k < avail ? k : avail - 1)].dl;
+            for (;;) {
                 for (int k = 0; k < avail; ++k) {
-                    head[m * kWave] += 1u;
+                    h += 1u;
                     if (alone <= dl[k]) {
                         found = true;
                         first = q0 + k;
@@ -198,9 +246,15 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                         good_out[(size_t)e.idx * kWave] = 0;
                     }
                 }
+                if (found || h == arr) break;
+                q0 = base + h;
+                avail = (int)(arr - h) < 8 ? (int)(arr - h) : 8;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) dl[k] = a.mq[q0 + (k < avail ? k : avail - 1)].dl;
             }
             if (!found) {  // :709-713
-                hrank[m * kWave] = a.mq[base + head[m * kWave]].rank;
+                head[m * LS] = h;
+                hrank[m * LS] = a.mq[base + h].rank;
                 m = select_model(g);
                 if (m < 0) return;
                 continue;
@@ -209,22 +263,40 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             int bs = 1;
             for (int b = 1; b < NB; ++b) {
                 const int cand = bsz[b];
-                if (cand - 1 > qlen(m)) break;
-                if (!check_slo(t0, gclk, stages, lat_mg, ilog2i(cand), deadline)) break;
+                if (cand - 1 > (int)(arr - h)) break;
+                const int col = ilog2i(cand);
+                double tc = tb[0];
+#pragma unroll
+                for (int x = 1; x < NBT; ++x) tc = col == x ? tb[x] : tc;
+                if (!((tc + overhead) <= deadline)) break;
                 bs = cand;
             }
             // run it (:715-732)
             const int col = ilog2i(bs);
             double t = t0 + overhead;
-            for (int k = 0; k < stages; ++k) {
-                t = dmax(t, gclk[k * kWave]) + (double)lat_mg[(size_t)k * NB + col];
-                gclk[k * kWave] = t;
+            double idle_at = 0.0;
+            for (int k0 = 0; k0 < stages; k0 += 4) {
+                double c[4];
+                float l[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int k = k0 + u < stages ? k0 + u : stages - 1;
+                    c[u] = gclk[k * LS];
+                    l[u] = lat_at(lat_mg + (uint32_t)(k * NB + col));
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (k0 + u < stages) {
+                        t = dmax(t, c[u]) + (double)l[u];
+                        gclk[(k0 + u) * LS] = t;
+                        if (k0 + u == 0) idle_at = t;
+                    }
             }
-            const double idle_at = gclk[0];
-            head[m * kWave] += (uint32_t)(bs - 1);  // the batch is the arrivals first .. first+bs-1 of the model
-            hrank[m * kWave] = a.mq[first + bs].rank;
+            head[m * LS] = h + (uint32_t)(bs - 1);  // the batch is the arrivals first .. first+bs-1 of the model
+            hrank[m * LS] = a.mq[first + bs].rank;
             for (int u0 = 0; u0 < bs; u0 += 8) {  // arrival times of up to eight members fetched together
                 double at[8];
+#pragma unroll
                 for (int k = 0; k < 8; ++k) at[k] = a.mq[first + (u0 + k < bs ? u0 + k : bs - 1)].t;
                 for (int k = 0; k < 8 && u0 + k < bs; ++k) {
                     lat_sum += t - at[k];
@@ -245,42 +317,48 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 dead = MMSIM_E_OVERFLOW;
                 return;
             }
-            ev_t[hn * kWave] = idle_at;
-            ev_g[hn * kWave] = g;
+            ev_t[hn * LS] = idle_at;
+            ev_g[hn * LS] = g;
             hn += 1;
             next_due = fmin(next_due, idle_at);
             return;
         }
     };
 
-    // index of the lexicographically smallest (time, group) event, hn > 0
-    auto min_event = [&]() -> int {
+    // index, time and group of the lexicographically smallest (time, group) event; time +inf if there is
+    // none.  Slots from hn on hold (+inf, all ones), so four are read per round without a bound check.
+    auto min_event = [&](double &bt, uint32_t &bg) -> int {
         int best = 0;
-        double bt = ev_t[0];
-        uint32_t bg = ev_g[0];
-        for (int e = 1; e < hn; ++e) {
-            const double t = ev_t[e * kWave];
-            const uint32_t g = ev_g[e * kWave];
-            if (t < bt || (t == bt && g < bg)) {
-                best = e;
-                bt = t;
-                bg = g;
+        bt = __builtin_inf();
+        bg = 0xFFFFFFFFu;
+        for (int e0 = 0; e0 < hn; e0 += 4) {
+            double t[4];
+            uint32_t g[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                t[u] = ev_t[(e0 + u) * LS];
+                g[u] = ev_g[(e0 + u) * LS];
             }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (t[u] < bt || (t[u] == bt && g[u] < bg)) {
+                    best = e0 + u;
+                    bt = t[u];
+                    bg = g[u];
+                }
         }
         return best;
     };
-    auto pop_event = [&](int e, double &t, uint32_t &g) {
-        t = ev_t[e * kWave];
-        g = ev_g[e * kWave];
+    auto pop_event = [&](int e) {  // the last event takes the place of event e
         hn -= 1;
-        ev_t[e * kWave] = ev_t[hn * kWave];
-        ev_g[e * kWave] = ev_g[hn * kWave];
-    };
-
-    auto refresh_due = [&]() {
-        double d = __builtin_inf();
-        for (int e = 0; e < hn; ++e) d = fmin(d, ev_t[e * kWave]);
-        next_due = d;
+        const double lt = ev_t[hn * LS];
+        const uint32_t lg = ev_g[hn * LS];
+        ev_t[hn * LS] = __builtin_inf();
+        ev_g[hn * LS] = 0xFFFFFFFFu;
+        if (e != hn) {
+            ev_t[e * LS] = lt;
+            ev_g[e * LS] = lg;
+        }
     };
 
     for (int64_t i = 0; i < R; ++i) {
@@ -304,17 +382,23 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 
         // ---- idle events that are due (:739-744)
         if (!dead && next_due <= tstamp) {
-            while (!dead && hn > 0) {
-                const int e = min_event();
-                if (!(ev_t[e * kWave] <= tstamp)) break;
+            for (;;) {
                 double ti;
                 uint32_t g;
-                pop_event(e, ti, g);
+                const int e = min_event(ti, g);
+                if (!(ti <= tstamp)) {  // also: no event left
+                    next_due = ti;
+                    break;
+                }
+                pop_event(e);
                 const int m2 = select_model(g);
-                if (m2 < 0) break;  // the popped event is dropped, later due events stay (:742-743)
+                if (m2 < 0) {  // the popped event is dropped, later due events stay (:742-743)
+                    (void)min_event(next_due, g);
+                    break;
+                }
                 handle(ti, m2, g);
+                if (dead) break;
             }
-            refresh_due();
         }
 
         // ---- the arrival (:746-778)
@@ -325,22 +409,32 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             if (hosted && !dead) {
                 // group with the strictly smallest last-stage clock (:760-770)
                 double best = 1e100;
-                int j = 0;
-                for (;;) {
-                    uint32_t g;
-                    if (j < kPackedReplicas)
-                        g = (uint32_t)(g8 >> (8 * j)) & 0xFFu;
-                    else if (j - kPackedReplicas < a.rep_extra)
-                        g = repx_tile[((size_t)m * a.rep_extra + (j - kPackedReplicas)) * kWave];
-                    else
-                        break;
+                bool more = true;  // the list may go on
+                for (int j0 = 0; j0 < kPackedReplicas && more; j0 += 4) {  // four replicas at a time: their reads overlap
+                    uint32_t g[4], d[4];
+                    double c[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) g[u] = (uint32_t)(g8 >> (8 * (j0 + u))) & 0xFFu;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) d[u] = ginfo[g[u] * LS];  // the empty row for unused bytes
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) c[u] = clk[desc_last_slot(d[u]) * LS];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        if (g[u] != none && c[u] < best) {
+                            best = c[u];
+                            gsel = g[u];
+                        }
+                    more = g[3] != none;
+                }
+                for (int j = 0; more && j < a.rep_extra; ++j) {
+                    const uint32_t g = repx_tile[((size_t)m * a.rep_extra + j) * kWave];
                     if (g == none) break;
-                    const double c = clk[desc_last_slot(ginfo[g * kWave]) * kWave];
+                    const double c = clk[desc_last_slot(ginfo[g * LS]) * LS];
                     if (c < best) {
                         best = c;
                         gsel = g;
                     }
-                    ++j;
                 }
                 queued = true;
             }
@@ -360,17 +454,17 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         } else if (gsel == none) {
             dead = MMSIM_E_UNSUPPORTED;  // every replica's clock is infinite; the reference indexes out of range here
         } else {
-            const uint32_t d = ginfo[gsel * kWave];
-            const double idle_since = clk[(desc_last_slot(d) - desc_stages_m1(d)) * kWave];
+            const uint32_t d = ginfo[gsel * LS];
+            const double idle_since = clk[(desc_last_slot(d) - desc_stages_m1(d)) * LS];
             if (tstamp >= idle_since) handle(tstamp, m, gsel);  // :776-778
         }
     }
     // ---- drain (:781-787)
     while (!dead && hn > 0) {
-        const int e = min_event();
         double ti;
         uint32_t g;
-        pop_event(e, ti, g);
+        const int e = min_event(ti, g);
+        pop_event(e);
         const int m2 = select_model(g);
         if (m2 < 0) continue;
         handle(ti, m2, g);
@@ -387,10 +481,21 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_bytes, hipStream_t stream,
                                std::string *err) {
     hipError_t e = hipSuccess;
-    if (wpb < 1 || wpb > kMaxWavesPerBlockBatching) {
+    if (wpb < 1 || wpb > kMaxWavesPerBlockBatching || args.NB > kMaxLatencyColumns || (args.heap_cap & 3) != 0) {
         e = hipErrorInvalidValue;
     } else {
-        auto kern = sim_batching_kernel;
+        const bool ll = args.lat_lds_bytes > 0, gl = args.g2m_in_lds != 0;
+        void (*kern)(const BatchingArgs) = nullptr;
+#define MMSIM_PICK(NBT)                                                                    \
+    kern = ll ? (gl ? sim_batching_kernel<NBT, true, true> : sim_batching_kernel<NBT, true, false>) \
+              : (gl ? sim_batching_kernel<NBT, false, true> : sim_batching_kernel<NBT, false, false>)
+        if (args.NB <= 4)
+            MMSIM_PICK(4);
+        else if (args.NB <= 8)
+            MMSIM_PICK(8);
+        else
+            MMSIM_PICK(16);
+#undef MMSIM_PICK
         if (lds_bytes > 64 * 1024)
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)lds_bytes);
