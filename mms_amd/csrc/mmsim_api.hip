@@ -348,21 +348,22 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 if (wave_bytes <= (size_t)ctx->max_lds) break;
             }
         };
-        // Simulations per wavefront.  The loops between two arrivals run per lane, so a wavefront takes as
-        // long as its slowest lane at every step, and its LDS footprint grows with its lanes.  When 64-lane
-        // wavefronts leave SIMDs without one (their state fills the CU's LDS, or the batch is small),
-        // narrower tiles are used: 32 or 16 lanes simulate, the others only help fetching requests.
+        // Simulations per wavefront.  The loops between two arrivals run per lane and are bound by
+        // latency (LDS and memory round trips), so a wavefront takes nearly as long with 8 simulations
+        // as with 64 while its LDS footprint grows with their number: narrow tiles (32, 16 or 8 lanes
+        // simulate, the others only help fetching requests) put more wavefronts on a CU, and that is
+        // what hides the latency.  The widest tile that still gives every SIMD two wavefronts is used.
         blanes = kWave;
         if (const char *env = std::getenv("MMSIM_BATCHING_LANES")) {
             const int v = std::atoi(env);
-            if (v == 16 || v == 32 || v == 64) blanes = v;
+            if (v == 8 || v == 16 || v == 32 || v == 64) blanes = v;
         } else {
-            const int64_t simds = 4 * (int64_t)std::max(1, ctx->prop.multiProcessorCount);
+            const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
             for (;;) {
                 size_for(blanes);
-                const int64_t per_cu = heap_cap >= Gmax + 4 ? std::min<int64_t>(4, (int64_t)ctx->max_lds / (int64_t)wave_bytes) : 0;
+                const int64_t per_cu = heap_cap >= Gmax + 4 ? (int64_t)ctx->max_lds / (int64_t)wave_bytes : 0;
                 const int64_t waves = (int64_t)((B + blanes - 1) / blanes) * n_seeds;
-                if (blanes == 16 || (per_cu >= 4 && waves >= simds)) break;
+                if (blanes == 8 || (per_cu >= 8 && waves >= 8 * cus)) break;
                 blanes /= 2;
             }
         }
@@ -607,28 +608,31 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
 
     // ---- batching simulator: keep the latency table (per workgroup) and the models of each group (per
-    //      wavefront) in LDS when they fit; they are read in the innermost loops.  Fewer wavefronts per
-    //      workgroup are accepted for it: the loops are bound by the latency of these reads.
+    //      wavefront) in LDS when they fit; they are read in the innermost loops.  Wavefronts per
+    //      workgroup (up to one per SIMD) come first: the loops are bound by latency, so a CU with an
+    //      idle SIMD loses more than one that reads these tables through the caches.
     size_t batching_lat_lds = 0;
     int batching_g2m_lds = 0;
     if (batching) {
         const size_t lat_b = (lat_nb.size() * sizeof(float) + 15) & ~(size_t)15;
         const size_t g2m_b = ((size_t)(Gmax + 1) * blanes * 2 + (size_t)members_max * blanes * 2 + 15) & ~(size_t)15;
         const size_t cap = (size_t)ctx->max_lds;
-        int w = wpb;
-        for (; w >= 1; --w)
-            if (lat_b + (size_t)w * (wave_bytes + g2m_b) <= cap) break;
-        if (w >= 1) {
-            batching_lat_lds = lat_b;
-            batching_g2m_lds = 1;
-            wpb = w;
-        } else if (lat_b + wave_bytes <= cap) {
-            batching_lat_lds = lat_b;
-            wpb = (int)std::min<size_t>(wpb, (cap - lat_b) / wave_bytes);
-        } else if (wave_bytes + g2m_b <= cap) {
-            batching_g2m_lds = 1;
-            wpb = (int)std::min<size_t>(wpb, cap / (wave_bytes + g2m_b));
-        }
+        const int tiles_here = std::max(1, b->classes.front().tile1 - b->classes.front().tile0);
+        int best_w = 0, best_total = 0;
+        for (int per_cu = 1; per_cu <= 2; ++per_cu)  // workgroups meant to share a CU (each gets that share of LDS)
+            for (int opt = 0; opt < 4; ++opt) {      // both, table only, lists only, neither: the first that gives most wavefronts
+                const bool want_lat = opt < 2, want_g2m = opt == 0 || opt == 2;
+                const size_t per = wave_bytes + (want_g2m ? g2m_b : 0), shared = want_lat ? lat_b : 0;
+                if (shared + per > cap / per_cu) continue;
+                const int w = (int)std::min<size_t>(std::min(wpb, tiles_here), (cap / per_cu - shared) / per);
+                if (per_cu * w > best_total) {
+                    best_total = per_cu * w;
+                    best_w = w;
+                    batching_lat_lds = shared;
+                    batching_g2m_lds = want_g2m ? 1 : 0;
+                }
+            }
+        wpb = std::max(1, best_w);
         if (batching_g2m_lds) wave_bytes += g2m_b;
         mmsim_batch::TileClass &c = b->classes.front();
         c.wpb = std::min(wpb, c.tile1 - c.tile0);

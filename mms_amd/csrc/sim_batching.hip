@@ -62,7 +62,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const int M = a.M, Gmax = a.Gmax, NB = a.NB;
-    const int LS = a.lane_stride;  // lanes of a wavefront that simulate (64, 32 or 16): pitch of the per-lane LDS arrays
+    const int LS = a.lane_stride;  // lanes of a wavefront that simulate (64, 32, 16 or 8): pitch of the per-lane LDS arrays
 
     // ---- LDS: [latency table, shared, if it fits][per wavefront: group descriptors | clocks | event times |
     //      queue heads | head ranks | event groups | arrivals per model | models of each group, if they fit]
@@ -325,11 +325,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         }
     };
 
-    // index, time and group of the lexicographically smallest (time, group) event; time +inf if there is
-    // none.  Slots from hn on hold (+inf, all ones), so four are read per round without a bound check.
-    auto min_event = [&](double &bt, uint32_t &bg) -> int {
+    // index, time and group of the lexicographically smallest (time, group) event (time +inf if there is
+    // none), and the earliest time among the other events.  Slots from hn on hold (+inf, all ones), so
+    // four are read per round without a bound check.
+    auto min_event = [&](double &bt, uint32_t &bg, double &rest) -> int {
         int best = 0;
         bt = __builtin_inf();
+        rest = __builtin_inf();
         bg = 0xFFFFFFFFu;
         for (int e0 = 0; e0 < hn; e0 += 4) {
             double t[4];
@@ -342,9 +344,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 #pragma unroll
             for (int u = 0; u < 4; ++u)
                 if (t[u] < bt || (t[u] == bt && g[u] < bg)) {
+                    rest = bt;  // the previous best is the earliest of the others so far
                     best = e0 + u;
                     bt = t[u];
                     bg = g[u];
+                } else {
+                    rest = fmin(rest, t[u]);
                 }
         }
         return best;
@@ -383,21 +388,19 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         // ---- idle events that are due (:739-744)
         if (!dead && next_due <= tstamp) {
             for (;;) {
-                double ti;
+                double ti, rest;
                 uint32_t g;
-                const int e = min_event(ti, g);
+                const int e = min_event(ti, g, rest);
                 if (!(ti <= tstamp)) {  // also: no event left
                     next_due = ti;
                     break;
                 }
                 pop_event(e);
+                next_due = rest;  // of what is left; handle() lowers it when it adds an earlier event
                 const int m2 = select_model(g);
-                if (m2 < 0) {  // the popped event is dropped, later due events stay (:742-743)
-                    (void)min_event(next_due, g);
-                    break;
-                }
+                if (m2 < 0) break;  // the popped event is dropped, later due events stay (:742-743)
                 handle(ti, m2, g);
-                if (dead) break;
+                if (dead || !(next_due <= tstamp)) break;
             }
         }
 
@@ -463,7 +466,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     while (!dead && hn > 0) {
         double ti;
         uint32_t g;
-        const int e = min_event(ti, g);
+        double rest;
+        const int e = min_event(ti, g, rest);
         pop_event(e);
         const int m2 = select_model(g);
         if (m2 < 0) continue;
