@@ -37,7 +37,13 @@ namespace mmsim {
 namespace {
 
 __device__ __forceinline__ int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
-__device__ __forceinline__ double dmax(double a, double b) { return b > a ? b : a; }
+// max of two doubles that are never NaN: one v_max_f64 without the input quieting that the generic
+// fmax lowering adds
+__device__ __forceinline__ double max_nn(double x, double y) {
+    double r;
+    asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y));
+    return r;
+}
 __device__ __forceinline__ int ilog2i(int v) { return 31 - __clz(v); }
 
 typedef volatile __attribute__((address_space(3))) uint32_t lds_vu32;
@@ -198,11 +204,17 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 for (int b = 0; b < NBT; ++b) l[u][b] = lat_at(lat_mg + (uint32_t)(k * NB + (b < NB ? b : NB - 1)));
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
-                if (k0 + u < stages) {
+            for (int u = 1; u < 4; ++u)
+                if (!(k0 + u < stages)) {  // past the last stage: max(-inf, t) + 0 leaves t as it is
+                    c[u] = -__builtin_inf();
 #pragma unroll
-                    for (int b = 0; b < NBT; ++b) tb[b] = dmax(c[u], tb[b]) + (double)l[u][b];
+                    for (int b = 0; b < NBT; ++b) l[u][b] = 0.0f;
                 }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int b = 0; b < NBT; ++b) tb[b] = max_nn(c[u], tb[b]) + (double)l[u][b];
+            }
         }
     };
 
@@ -287,7 +299,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 #pragma unroll
                 for (int u = 0; u < 4; ++u)
                     if (k0 + u < stages) {
-                        t = dmax(t, c[u]) + (double)l[u];
+                        t = max_nn(t, c[u]) + (double)l[u];
                         gclk[(k0 + u) * LS] = t;
                         if (k0 + u == 0) idle_at = t;
                     }
