@@ -11,6 +11,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <limits>
 #include <memory>
 #include <new>
@@ -297,7 +298,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     size_t wave_bytes = 0, lat_bytes = 0, lds_tail = 0;
     int lat_in_lds = 1;
     int wpb = 0;
-    int heap_cap = 0;
+    int heap_cap = 0, heap_min = 0, heap_pref = 0;  // batching simulator: event slots per lane (chosen, least, preferred)
+    std::function<size_t(int, int)> batching_bytes_for;
     int blanes = kWave;  // batching simulator: lanes of a wavefront that simulate
     // Wavefronts per workgroup: no more than it takes to give every CU its share of the
     // batch (a small batch is spread over the CUs, one wavefront per workgroup), and
@@ -335,16 +337,23 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             pow2_depths = false;
         }
     } else {
-        // per wavefront: descriptors | clocks | event times | queue heads | head ranks | event groups |
-        // arrivals per model | offsets of the models' arrival lists | batch sizes.  Events: the reference's heap holds about one entry per group plus a few
-        // stale ones (most seen: G+3); provision min(2*G+8, G+16) if that fits, never less than G+4.
+        // per wavefront: descriptors | clocks | event times | chunk minima | queue heads | head ranks | event
+        // groups | free slots | arrivals per model | offsets of the models' arrival lists | batch sizes.
+        // Event slots: the reference's heap holds about one entry per group plus a few stale ones (most
+        // seen: G+3); min(2*G+8, G+16) are provisioned if that fits, never less than G+4, always a multiple
+        // of eight (the kernel keeps them in chunks of eight).
+        auto bytes_for = [&](int lanes, int slots) {
+            const size_t nch8 = (size_t)((slots / 8 + 7) & ~7);
+            return ((size_t)(Gmax + 1) * lanes * 4 + (size_t)nslots * lanes * 8 + (size_t)2 * M * lanes * 4 +
+                    (size_t)slots * lanes * (8 + 4 + 2) + nch8 * lanes * 8 +
+                    (((size_t)M * 4 + 15) & ~(size_t)15) + (((size_t)(M + 1) * 8 + 15) & ~(size_t)15) +
+                    (((size_t)t->NB * 4 + 15) & ~(size_t)15) + 15) & ~(size_t)15;
+        };
+        heap_min = (Gmax + 4 + 7) & ~7;
+        heap_pref = std::max(heap_min, std::min(2 * Gmax + 8, Gmax + 16) & ~7);
         auto size_for = [&](int lanes) {
-            const size_t fixed = (size_t)(Gmax + 1) * lanes * 4 + (size_t)nslots * lanes * 8 + (size_t)2 * M * lanes * 4 +
-                                 (((size_t)M * 4 + 15) & ~(size_t)15) + (((size_t)(M + 1) * 8 + 15) & ~(size_t)15) +
-                                 (((size_t)t->NB * 4 + 15) & ~(size_t)15);
-            // (a multiple of four: the kernel scans the list four slots at a time)
-            for (heap_cap = std::min(2 * Gmax + 8, Gmax + 16) & ~3; heap_cap >= Gmax + 4; heap_cap -= 4) {
-                wave_bytes = (fixed + (size_t)heap_cap * lanes * 12 + 15) & ~(size_t)15;
+            for (heap_cap = heap_pref; heap_cap >= heap_min; heap_cap -= 8) {
+                wave_bytes = bytes_for(lanes, heap_cap);
                 if (wave_bytes <= (size_t)ctx->max_lds) break;
             }
         };
@@ -361,14 +370,15 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
             for (;;) {
                 size_for(blanes);
-                const int64_t per_cu = heap_cap >= Gmax + 4 ? (int64_t)ctx->max_lds / (int64_t)wave_bytes : 0;
+                const int64_t per_cu = heap_cap >= heap_min ? (int64_t)ctx->max_lds / (int64_t)wave_bytes : 0;
                 const int64_t waves = (int64_t)((B + blanes - 1) / blanes) * n_seeds;
                 if (blanes == 8 || (per_cu >= 8 && waves >= 8 * cus)) break;
                 blanes /= 2;
             }
         }
         size_for(blanes);
-        if (heap_cap < Gmax + 4) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: per-wavefront state does not fit in LDS (too many models/stages/groups)");
+        if (heap_cap < heap_min) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: per-wavefront state does not fit in LDS (too many models/stages/groups)");
+        batching_bytes_for = bytes_for;
         wpb = (int)std::min<size_t>(kMaxWavesPerBlockBatching, (size_t)ctx->max_lds / wave_bytes);
     }
 
@@ -618,20 +628,29 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         const size_t g2m_b = ((size_t)(Gmax + 1) * blanes * 2 + (size_t)members_max * blanes * 2 + 15) & ~(size_t)15;
         const size_t cap = (size_t)ctx->max_lds;
         const int tiles_here = std::max(1, b->classes.front().tile1 - b->classes.front().tile0);
-        int best_w = 0, best_total = 0;
-        for (int per_cu = 1; per_cu <= 2; ++per_cu)  // workgroups meant to share a CU (each gets that share of LDS)
-            for (int opt = 0; opt < 4; ++opt) {      // both, table only, lists only, neither: the first that gives most wavefronts
-                const bool want_lat = opt < 2, want_g2m = opt == 0 || opt == 2;
-                const size_t per = wave_bytes + (want_g2m ? g2m_b : 0), shared = want_lat ? lat_b : 0;
-                if (shared + per > cap / per_cu) continue;
-                const int w = (int)std::min<size_t>(std::min(wpb, tiles_here), (cap / per_cu - shared) / per);
-                if (per_cu * w > best_total) {
-                    best_total = per_cu * w;
-                    best_w = w;
-                    batching_lat_lds = shared;
-                    batching_g2m_lds = want_g2m ? 1 : 0;
+        // Fewer event slots (down to G+8) are accepted when that puts more wavefronts on a CU.
+        const int wpb_max = kMaxWavesPerBlockBatching;
+        const int heap_try_min = std::min(heap_cap, std::max(heap_min, (Gmax + 8 + 7) & ~7));
+        int best_w = 0, best_total = 0, best_heap = heap_cap;
+        for (int hc = heap_cap; hc >= heap_try_min; hc -= 8) {
+            const size_t wb = batching_bytes_for(blanes, hc);
+            for (int per_cu = 1; per_cu <= 2; ++per_cu)  // workgroups meant to share a CU (each gets that share of LDS)
+                for (int opt = 0; opt < 4; ++opt) {      // both, table only, lists only, neither: the first that gives most wavefronts
+                    const bool want_lat = opt < 2, want_g2m = opt == 0 || opt == 2;
+                    const size_t per = wb + (want_g2m ? g2m_b : 0), shared = want_lat ? lat_b : 0;
+                    if (shared + per > cap / per_cu) continue;
+                    const int w = (int)std::min<size_t>(std::min(wpb_max, tiles_here), (cap / per_cu - shared) / per);
+                    if (per_cu * w > best_total) {
+                        best_total = per_cu * w;
+                        best_w = w;
+                        best_heap = hc;
+                        batching_lat_lds = shared;
+                        batching_g2m_lds = want_g2m ? 1 : 0;
+                    }
                 }
-            }
+        }
+        heap_cap = best_heap;
+        wave_bytes = batching_bytes_for(blanes, heap_cap);
         wpb = std::max(1, best_w);
         if (batching_g2m_lds) wave_bytes += g2m_b;
         mmsim_batch::TileClass &c = b->classes.front();

@@ -20,10 +20,13 @@
 //     arrival time (hrank[m][lane]) so that "whose head arrived first" is
 //     decided without touching global memory;
 //   * the pending idle events, a multiset of (time, group) that the
-//     reference keeps in a heap (:728, :739-740): a small unsorted array per
-//     lane in LDS, popped by lexicographic minimum.  If a lane would need
-//     more entries than were provisioned it is flagged MMSIM_E_OVERFLOW and
-//     stops; its results are then reported as invalid.
+//     reference keeps in a heap (:728, :739-740): an unsorted array of slots
+//     per lane in LDS, in chunks of eight, with the earliest time of every
+//     chunk kept beside it and a stack of the free slots.  Popping the
+//     lexicographic minimum reads the chunk minima and then one chunk; adding
+//     an event takes a slot off the stack.  If a lane would need more slots
+//     than were provisioned it is flagged MMSIM_E_OVERFLOW and stops; its
+//     results are then reported as invalid.
 //
 // Arithmetic follows the reference: deadlines are arrival + (double)slo,
 // check_slo adds the fixed overhead last (:666-672) while a committed batch
@@ -71,7 +74,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const int LS = a.lane_stride;  // lanes of a wavefront that simulate (64, 32, 16 or 8): pitch of the per-lane LDS arrays
 
     // ---- LDS: [latency table, shared, if it fits][per wavefront: group descriptors | clocks | event times |
-    //      queue heads | head ranks | event groups | arrivals per model | models of each group, if they fit]
+    //      chunk minima | queue heads | head ranks | event groups | free slots | arrivals per model | offsets of
+    //      the models' arrival lists | batch sizes | models of each group, if they fit]
+    const int nch = a.heap_cap >> 3;         // chunks of eight event slots
+    const int nch8 = (nch + 7) & ~7;         // chunk minima are read eight at a time; the spare ones stay +inf
     float *lat_lds = reinterpret_cast<float *>(lds_raw);
     if (a.lat_lds_bytes > 0) {
         const int n = M * a.lat_row * NB;
@@ -84,12 +90,16 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     o += (size_t)a.nslots * LS * 8;
     double *ev_t = reinterpret_cast<double *>(mine + o) + lane;
     o += (size_t)a.heap_cap * LS * 8;
+    double *cm_t = reinterpret_cast<double *>(mine + o) + lane;  // earliest event time of each chunk
+    o += (size_t)nch8 * LS * 8;
     uint32_t *head = reinterpret_cast<uint32_t *>(mine + o) + lane;
     o += (size_t)M * LS * 4;
     int32_t *hrank = reinterpret_cast<int32_t *>(mine + o) + lane;  // rank of the arrival at head[m] (already known before it arrives)
     o += (size_t)M * LS * 4;
     uint32_t *ev_g = reinterpret_cast<uint32_t *>(mine + o) + lane;
     o += (size_t)a.heap_cap * LS * 4;
+    uint16_t *fstack = reinterpret_cast<uint16_t *>(mine + o) + lane;  // free event slots, the next one to use on top
+    o += (size_t)a.heap_cap * LS * 2;
     // [M], same for all lanes; written by lane 0 and read by all, hence volatile (and spelled as an LDS
     // pointer: volatile accesses are not rewritten from generic to LDS by the compiler)
     lds_vu32 *arrived = as_lds_vu32(mine + o);
@@ -108,10 +118,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         const uint32_t *gsrc = a.ginfo + (size_t)tile * (Gmax + 1) * kWave + lane;
         for (int g = 0; g <= Gmax; ++g) ginfo[g * LS] = gsrc[g * kWave];
         for (int s = 0; s < a.nslots; ++s) clk[s * LS] = 0.0;
-        for (int e = 0; e < a.heap_cap; ++e) {  // unused event slots never win the minimum scan
+        for (int e = 0; e < a.heap_cap; ++e) {  // free event slots never win a minimum scan
             ev_t[e * LS] = __builtin_inf();
             ev_g[e * LS] = 0xFFFFFFFFu;
+            fstack[e * LS] = (uint16_t)(a.heap_cap - 1 - e);  // slot 0 is used first, so events gather in the first chunks
         }
+        for (int c = 0; c < nch8; ++c) cm_t[c * LS] = __builtin_inf();
         {
             const int64_t *mo = a.mq_off + (size_t)seed * (M + 1);
             for (int m = lane; m <= M; m += LS) mq_off[m] = mo[m];
@@ -152,7 +164,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 
     int32_t n_good = 0;
     double lat_sum = 0.0;
-    int hn = 0;          // pending idle events of this lane
+    int nfree = a.heap_cap;  // free event slots of this lane (heap_cap - nfree events are pending)
     double next_due = __builtin_inf();  // the earliest of them (+inf if none): arrivals before it skip the event list
     int dead = sim ? 0 : 1;  // nonzero: this lane simulates nothing (more): out of event slots, unsupported input, or a spare lane of a narrow tile
 
@@ -325,57 +337,87 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 group_good[g * kWave] += bs;
             }
             if (want_model) model_good[(size_t)m * kWave] += bs;
-            if (hn >= a.heap_cap) {
+            if (nfree == 0) {
                 dead = MMSIM_E_OVERFLOW;
                 return;
             }
-            ev_t[hn * LS] = idle_at;
-            ev_g[hn * LS] = g;
-            hn += 1;
+            nfree -= 1;
+            const int slot = fstack[nfree * LS];
+            ev_t[slot * LS] = idle_at;
+            ev_g[slot * LS] = g;
+            double *cm = cm_t + (slot >> 3) * LS;
+            *cm = fmin(*cm, idle_at);
             next_due = fmin(next_due, idle_at);
             return;
         }
     };
 
-    // index, time and group of the lexicographically smallest (time, group) event (time +inf if there is
-    // none), and the earliest time among the other events.  Slots from hn on hold (+inf, all ones), so
-    // four are read per round without a bound check.
-    auto min_event = [&](double &bt, uint32_t &bg, double &rest) -> int {
-        int best = 0;
-        bt = __builtin_inf();
-        rest = __builtin_inf();
-        bg = 0xFFFFFFFFu;
-        for (int e0 = 0; e0 < hn; e0 += 4) {
-            double t[4];
-            uint32_t g[4];
+    // earliest event time (+inf if there is no event), the chunk that holds it (the first such chunk),
+    // and the earliest time among the other chunks
+    auto chunk_scan = [&](double &T, int &cj, double &others) {
+        T = __builtin_inf();
+        others = __builtin_inf();
+        cj = 0;
+        for (int c0 = 0; c0 < nch; c0 += 8) {
+            double v[8];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                t[u] = ev_t[(e0 + u) * LS];
-                g[u] = ev_g[(e0 + u) * LS];
-            }
+            for (int u = 0; u < 8; ++u) v[u] = cm_t[(c0 + u) * LS];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
-                if (t[u] < bt || (t[u] == bt && g[u] < bg)) {
-                    rest = bt;  // the previous best is the earliest of the others so far
-                    best = e0 + u;
-                    bt = t[u];
-                    bg = g[u];
+            for (int u = 0; u < 8; ++u)
+                if (v[u] < T) {
+                    others = T;  // the previous earliest is the earliest of the others so far
+                    T = v[u];
+                    cj = c0 + u;
                 } else {
-                    rest = fmin(rest, t[u]);
+                    others = v[u] < others ? v[u] : others;
                 }
         }
-        return best;
     };
-    auto pop_event = [&](int e) {  // the last event takes the place of event e
-        hn -= 1;
-        const double lt = ev_t[hn * LS];
-        const uint32_t lg = ev_g[hn * LS];
-        ev_t[hn * LS] = __builtin_inf();
-        ev_g[hn * LS] = 0xFFFFFFFFu;
-        if (e != hn) {
-            ev_t[e * LS] = lt;
-            ev_g[e * LS] = lg;
+    // removes the lexicographically smallest (time, group) event, whose time T and chunk cj chunk_scan
+    // found (others as returned by it); returns its group and sets next_due to the earliest time left
+    auto take_event = [&](double T, int cj, double others) -> uint32_t {
+        uint32_t bg = 0xFFFFFFFFu;
+        int be = cj << 3;
+        if (others == T) {
+            // several chunks hold an event at time T: the smallest group among all of them (rare)
+            for (int c = 0; c < nch; ++c) {
+                if (cm_t[c * LS] != T) continue;
+                for (int u = 0; u < 8; ++u) {
+                    const int e = (c << 3) + u;
+                    const uint32_t g = ev_g[e * LS];
+                    if (ev_t[e * LS] == T && g < bg) {
+                        bg = g;
+                        be = e;
+                    }
+                }
+            }
+            cj = be >> 3;
         }
+        double t[8];
+        uint32_t g[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            t[u] = ev_t[((cj << 3) + u) * LS];
+            g[u] = ev_g[((cj << 3) + u) * LS];
+        }
+        if (others != T) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (t[u] == T && g[u] < bg) {
+                    bg = g[u];
+                    be = (cj << 3) + u;
+                }
+        }
+        double left = __builtin_inf();  // earliest time left in the chunk
+#pragma unroll
+        for (int u = 0; u < 8; ++u) left = ((cj << 3) + u != be && t[u] < left) ? t[u] : left;
+        ev_t[be * LS] = __builtin_inf();
+        ev_g[be * LS] = 0xFFFFFFFFu;
+        cm_t[cj * LS] = left;
+        fstack[nfree * LS] = (uint16_t)be;
+        nfree += 1;
+        next_due = left < others ? left : others;
+        return bg;
     };
 
     for (int64_t i = 0; i < R; ++i) {
@@ -400,15 +442,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         // ---- idle events that are due (:739-744)
         if (!dead && next_due <= tstamp) {
             for (;;) {
-                double ti, rest;
-                uint32_t g;
-                const int e = min_event(ti, g, rest);
+                double ti, others;
+                int cj;
+                chunk_scan(ti, cj, others);
                 if (!(ti <= tstamp)) {  // also: no event left
                     next_due = ti;
                     break;
                 }
-                pop_event(e);
-                next_due = rest;  // of what is left; handle() lowers it when it adds an earlier event
+                const uint32_t g = take_event(ti, cj, others);  // sets next_due; handle() lowers it when it adds an earlier event
                 const int m2 = select_model(g);
                 if (m2 < 0) break;  // the popped event is dropped, later due events stay (:742-743)
                 handle(ti, m2, g);
@@ -475,12 +516,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         }
     }
     // ---- drain (:781-787)
-    while (!dead && hn > 0) {
-        double ti;
-        uint32_t g;
-        double rest;
-        const int e = min_event(ti, g, rest);
-        pop_event(e);
+    while (!dead && nfree < a.heap_cap) {
+        double ti, others;
+        int cj;
+        chunk_scan(ti, cj, others);
+        const uint32_t g = take_event(ti, cj, others);
         const int m2 = select_model(g);
         if (m2 < 0) continue;
         handle(ti, m2, g);
@@ -497,7 +537,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_bytes, hipStream_t stream,
                                std::string *err) {
     hipError_t e = hipSuccess;
-    if (wpb < 1 || wpb > kMaxWavesPerBlockBatching || args.NB > kMaxLatencyColumns || (args.heap_cap & 3) != 0) {
+    if (wpb < 1 || wpb > kMaxWavesPerBlockBatching || args.NB > kMaxLatencyColumns || (args.heap_cap & 7) != 0) {
         e = hipErrorInvalidValue;
     } else {
         const bool ll = args.lat_lds_bytes > 0, gl = args.g2m_in_lds != 0;

@@ -64,6 +64,36 @@ def test_random_cases_match_oracle(eng):
             assert np.array_equal(a, b), seed
 
 
+def test_groups_that_become_idle_at_the_same_instant(eng):
+    """Idle events with equal times are popped in group order (the reference's heap holds (time, group)
+    tuples, alpa_serve/simulator/controller.py:728-740).  Twelve identical one-stage groups all start a
+    request at the same arrival time, so twelve events share one time and span two chunks of the kernel's
+    event list; the queued requests they pick up afterwards keep the times equal."""
+    G = M = 12
+    rng = np.random.default_rng(7)
+    waves = 6
+    tst = np.repeat(np.arange(waves) * 0.05, M)          # M arrivals at each instant, one per model
+    mids = np.concatenate([rng.permutation(M) for _ in range(waves)]).astype(np.int32)
+    slos = np.full(tst.size, 5.0, np.float32)
+    m2g = np.full((M, G), -1, np.int32)                   # [M][G] and [G][M], unused entries -1
+    g2m = np.full((G, M), -1, np.int32)
+    for m in range(M):
+        m2g[m, 0] = (m * 5) % G                           # a permutation of the groups
+        g2m[(m * 5) % G, 0] = m
+    lat = np.full((M, G, 1, 2), 0.125, np.float32)        # same latency everywhere, both batch sizes
+    c = {"tstamps": tst, "model_ids": mids, "slos": slos, "m2g": m2g, "g2m": g2m,
+         "num_stages": np.ones(G, np.int32), "lat": lat}
+    bss = [1, 2]
+    f0, g0, c0, _ = oracle_c.simulate_requests_mixed_batching(
+        c["tstamps"], c["model_ids"], c["slos"], c["m2g"], c["g2m"], c["num_stages"], c["lat"], bss)
+    assert g0.sum() > M                                   # queued requests were served from idle events
+    fin, good, cnt = _single(eng, c, bss)
+    assert np.array_equal(good, g0)
+    assert np.array_equal(fin.view(np.uint64), f0.view(np.uint64))
+    for a, b in zip(cnt, c0):
+        assert np.array_equal(a, b)
+
+
 def _run(eng, cfg, sols, seeds, flags):
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
     packed = E.pack_placements(sols, table)
