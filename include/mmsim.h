@@ -58,6 +58,7 @@ enum {
 #define MMSIM_MAX_GROUPS 254       /* groups of one placement                     */
 #define MMSIM_MAX_SLOTS 255        /* sum of pipeline stages over a placement     */
 #define MMSIM_MAX_CONFIGS 255      /* distinct parallel configurations            */
+#define MMSIM_MAX_BATCH_SIZES 16   /* batch sizes (batching simulator)            */
 
 typedef struct mmsim_ctx mmsim_ctx;
 typedef struct mmsim_workload mmsim_workload;

@@ -222,7 +222,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             if (col >= t->NB) return fail(MMSIM_E_INVALID, "tables: floor(log2(batch size)) must index a latency column");
         }
         if (t->M > 65535) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: more than 65535 models");
-        if (t->NB > kMaxLatencyColumns) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: more than 16 batch sizes");
+        if (t->NB > MMSIM_MAX_BATCH_SIZES) return fail(MMSIM_E_UNSUPPORTED, "batching simulator: more than 16 batch sizes");
     }
     const int32_t M = t->M, C = t->C, B = rl.B, Gmax = rl.Gmax;
     if (n_seeds < 1 || !wls) return fail(MMSIM_E_INVALID, "need at least one workload");

@@ -176,6 +176,6 @@ hipError_t launch_sim_mixed(const MixedArgs &args, int smax_bucket, int waves_pe
 int smax_bucket_for(int smax);
 constexpr int kMaxWavesPerBlock = 8;          // plain simulator
 constexpr int kMaxWavesPerBlockBatching = 4;  // batching simulator
-constexpr int kMaxLatencyColumns = 16;       // batching simulator: batch sizes below 2^16
+constexpr int kMaxLatencyColumns = MMSIM_MAX_BATCH_SIZES;  // batching simulator: batch sizes below 2^16
 
 }  // namespace mmsim
