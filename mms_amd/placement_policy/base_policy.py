@@ -346,42 +346,67 @@ def replica_placement_round_robin(init_sol: ModelPlacement, model_datas: List[Mo
     return sol
 
 
+def _fast_greedy_step(sol, stats, weight_mem, cluster_env):
+    """One iteration of the greedy search (:339-372): the model with most unserved
+    requests gets a replica on the least loaded group that still has memory for it.
+    Returns the (group, model) to add or None when nothing fits."""
+    overall_goodput, goodputs, group_num_requests, fullstats = stats
+    unserved = [s.num_requests * (1 - gp) for s, gp in zip(fullstats.per_model_stats, goodputs)]
+    model_order = np.argsort(unserved)[::-1]
+    group_order = np.argsort(group_num_requests)
+    group_mem = _group_memory(sol, weight_mem)
+    for g_id in group_order:
+        cfg = sol.group_configs[g_id]
+        for m_id in model_order:
+            if m_id not in sol.group_models[g_id] and \
+                    weight_mem[cfg][m_id] + group_mem[g_id] <= cluster_env.mem_budget:
+                return g_id, m_id
+    return None
+
+
 def replica_placement_fast_greedy(init_sol: ModelPlacement, model_datas: List[ModelData],
                                   cluster_env: ClusterEnv, workload: Workload,
                                   evaluator: PlacementEvaluator, verbose: int):
     """Repeatedly give the model with most unserved requests a replica on the
     least loaded group that still has memory for it (:329-400)."""
+    return replica_placement_fast_greedy_lockstep([init_sol], model_datas, cluster_env, workload,
+                                                  evaluator, verbose)[0]
+
+
+def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], model_datas: List[ModelData],
+                                           cluster_env: ClusterEnv, workload: Workload,
+                                           evaluator: PlacementEvaluator, verbose: int):
+    """``replica_placement_fast_greedy`` for several initial placements at once.
+
+    The reference runs one greedy search per enumerated group layout, each
+    scoring one placement per iteration (model_parallelism.py:341-344,
+    :533-541).  The searches do not depend on each other, so they are advanced
+    together: every iteration evaluates the current placement of every search
+    that is still running in one evaluator call (one lane each on the GPU), and
+    each search takes exactly the step it would take alone.  Returns the final
+    placements in the order of ``init_sols``."""
     tic = time.time()
     if evaluator is None:
         evaluator = PlacementEvaluator(model_datas, cluster_env, workload, "fast_simulator", False)
-    weight_mem = weight_mem_table(init_sol.group_configs, model_datas)
-    sol = init_sol
+    sols = list(init_sols)
+    weight_mems = [weight_mem_table(sol.group_configs, model_datas) for sol in sols]
+    running = list(range(len(sols)))
     it = 0
-    while True:
-        overall_goodput, goodputs, group_num_requests, fullstats = evaluator.get_stats([sol])[0]
-        unserved = [s.num_requests * (1 - gp) for s, gp in zip(fullstats.per_model_stats, goodputs)]
-        model_order = np.argsort(unserved)[::-1]
-        group_order = np.argsort(group_num_requests)
-        group_mem = _group_memory(sol, weight_mem)
-
-        choice = None
-        for g_id in group_order:
-            cfg = sol.group_configs[g_id]
-            for m_id in model_order:
-                if m_id not in sol.group_models[g_id] and \
-                        weight_mem[cfg][m_id] + group_mem[g_id] <= cluster_env.mem_budget:
-                    choice = (g_id, m_id)
-                    break
-            if choice:
-                break
-        if not choice:
-            break
-        sol = sol.add_model(*choice).normalize()
-        if verbose >= 2:
-            print(f"iter: {it}, score: {overall_goodput:.4f}, elapsed: {time.time() - tic:.2f}, "
-                  f"best placement: {sol}, ")
+    while running:
+        all_stats = evaluator.get_stats([sols[i] for i in running])
+        still = []
+        for i, stats in zip(running, all_stats):
+            choice = _fast_greedy_step(sols[i], stats, weight_mems[i], cluster_env)
+            if choice is None:
+                continue
+            sols[i] = sols[i].add_model(*choice).normalize()
+            still.append(i)
+            if verbose >= 2:
+                print(f"iter: {it}, search: {i}, score: {stats[0]:.4f}, elapsed: {time.time() - tic:.2f}, "
+                      f"best placement: {sols[i]}, ")
+        running = still
         it += 1
-    return sol
+    return sols
 
 
 def _beam_loop(init_sol, evaluator, beam_size, verbose, expand, tic):

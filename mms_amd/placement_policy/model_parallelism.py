@@ -16,7 +16,7 @@ import numpy as np
 from mms_amd.placement_policy.base_policy import (
     BasePlacementPolicy, ClusterEnv, ModelData, ModelPlacement, PlacementEvaluator,
     evolutionary_search, gen_train_workload, replica_placement_fast_greedy,
-    replica_placement_round_robin)
+    replica_placement_fast_greedy_lockstep, replica_placement_round_robin)
 from mms_amd.profiling import ParallelConfig
 from mms_amd.simulator.workload import Workload
 from mms_amd.util import decompose2tok, get2tok, get_factors, get_partitions
@@ -107,9 +107,9 @@ class ModelParallelismSearch(BasePlacementPolicy):
         evaluator = PlacementEvaluator(model_datas, cluster_env, train_workload,
                                        self.evaluator_method, self.parallel_evaluator)
         sols = self.enumerate_group_configs_uneven(cluster_env)
-        for i in range(len(sols)):
-            sols[i] = replica_placement_fast_greedy(sols[i], model_datas, cluster_env, train_workload,
-                                                    evaluator, self.verbose)
+        # one greedy search per layout, advanced together (one evaluator call per iteration for all of them)
+        sols = replica_placement_fast_greedy_lockstep(sols, model_datas, cluster_env, train_workload,
+                                                      evaluator, self.verbose)
         scores = evaluator.get_scores(sols)
         return sols[int(np.argmax(scores))], {}
 
@@ -224,15 +224,16 @@ class ModelParallelismSearch(BasePlacementPolicy):
         n, per_node = cluster_env.num_devices, cluster_env.num_devices_per_node
         beams = [[ModelPlacement([], [])]]
         for cur in range(1, n + 1):
-            candidates = []
+            starts = []
             for last_size in range(1, (cur - 1) % per_node + 1 + 1):
                 for cfg in self._configs_for(last_size):
                     for sol in beams[cur - last_size]:
                         pre = sol.copy()
                         pre.group_configs.append(cfg)
                         pre.group_models = [[] for _ in range(len(pre.group_configs))]
-                        candidates.append(replica_placement_fast_greedy(
-                            pre, model_datas, cluster_env, train_workload, evaluator, self.verbose))
+                        starts.append(pre)
+            candidates = replica_placement_fast_greedy_lockstep(
+                starts, model_datas, cluster_env, train_workload, evaluator, self.verbose)
             scores = evaluator.get_scores(candidates)
             keep = np.argsort(scores)[::-1][:beam_size]
             beams.append([candidates[i] for i in keep])

@@ -213,6 +213,32 @@ def test_other_policies_and_searches_run(backend):
     placement.verify(mixed, ClusterEnv(4, 4.5 * GB))
 
 
+def test_greedy_searches_in_lockstep_take_the_steps_they_take_alone(backend):
+    """The greedy searches of the enumerated group layouts (model_parallelism.py:341-344) advanced together
+    end where each ends alone, with one evaluator call per iteration instead of one per search and iteration."""
+    from mms_amd.placement_policy.base_policy import (replica_placement_fast_greedy,
+                                                      replica_placement_fast_greedy_lockstep)
+    cluster_env = ClusterEnv(num_devices=4, mem_budget=4.5 * GB)
+    model_datas = four_models(0.5, 6, 2)
+    wl = gen_train_workload(model_datas, simulation_min_samples=2000)
+    starts = ModelParallelismSearch().enumerate_group_configs_uneven(cluster_env)
+    assert len(starts) >= 4
+
+    class Counting(PlacementEvaluator):
+        calls = 0
+
+        def get_stats(self, sols):
+            Counting.calls += 1
+            return super().get_stats(sols)
+
+    ev = Counting(model_datas, cluster_env, wl, "fast_simulator", False)
+    alone = [replica_placement_fast_greedy(s, model_datas, cluster_env, wl, ev, 0) for s in starts]
+    calls_alone, Counting.calls = Counting.calls, 0
+    together = replica_placement_fast_greedy_lockstep(starts, model_datas, cluster_env, wl, ev, 0)
+    assert [str(a) for a in alone] == [str(t) for t in together]
+    assert Counting.calls < calls_alone / 2
+
+
 def test_batching_evaluator(backend, monkeypatch):
     import mms_amd.util as U
     from mms_amd.profiling import synthetic_profile
