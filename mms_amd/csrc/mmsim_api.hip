@@ -632,11 +632,15 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         const int wpb_max = kMaxWavesPerBlockBatching;
         const int heap_try_min = std::min(heap_cap, std::max(heap_min, (Gmax + 8 + 7) & ~7));
         int best_w = 0, best_total = 0, best_heap = heap_cap;
+        // MMSIM_BATCHING_LDS_TABLES (bit 0: latency table, bit 1: group lists) fixes which tables may go to LDS
+        int allowed = 3;
+        if (const char *env = std::getenv("MMSIM_BATCHING_LDS_TABLES")) allowed = std::atoi(env) & 3;
         for (int hc = heap_cap; hc >= heap_try_min; hc -= 8) {
             const size_t wb = batching_bytes_for(blanes, hc);
             for (int per_cu = 1; per_cu <= 2; ++per_cu)  // workgroups meant to share a CU (each gets that share of LDS)
                 for (int opt = 0; opt < 4; ++opt) {      // both, table only, lists only, neither: the first that gives most wavefronts
                     const bool want_lat = opt < 2, want_g2m = opt == 0 || opt == 2;
+                    if ((want_lat && !(allowed & 1)) || (want_g2m && !(allowed & 2))) continue;
                     const size_t per = wb + (want_g2m ? g2m_b : 0), shared = want_lat ? lat_b : 0;
                     if (shared + per > cap / per_cu) continue;
                     const int w = (int)std::min<size_t>(std::min(wpb_max, tiles_here), (cap / per_cu - shared) / per);

@@ -21,7 +21,8 @@ def random_case(seed, max_m=4, max_g=3, max_s=3, max_r=50, nb=1, p_unknown=0.05,
         ms = [m for m in range(M) if member[g, m]]
         g2m[g, :len(ms)] = ms
     base = rng.uniform(0.01, 0.3, size=(M, G, S, 1))
-    growth = 1 + 0.15 * (np.array([1, 2, 4, 8, 16][:nb]) - 1).reshape(1, 1, 1, nb)
+    steps = [1, 2, 4, 8, 16] + [16 + k for k in range(1, 12)]   # slow growth past 16 so that large batches can form
+    growth = 1 + 0.15 * (np.array(steps[:nb]) - 1).reshape(1, 1, 1, nb)
     jitter = rng.uniform(0.9, 1.1, size=(M, G, S, nb))
     lat = (base * growth * jitter).astype(np.float32)
     for m in range(M):

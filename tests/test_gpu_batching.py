@@ -64,6 +64,27 @@ def test_random_cases_match_oracle(eng):
             assert np.array_equal(a, b), seed
 
 
+@pytest.mark.parametrize("lanes", [8, 16, 32, 64])
+@pytest.mark.parametrize("lds_tables", [0, 1, 2, 3])
+def test_every_kernel_variant(eng, monkeypatch, lanes, lds_tables):
+    """Tile width (simulating lanes per wavefront), which tables are read from LDS, and the number of latency
+    columns held in registers (4, 8 or 16) are picked from the input's size; here each is forced."""
+    monkeypatch.setenv("MMSIM_BATCHING_LANES", str(lanes))
+    monkeypatch.setenv("MMSIM_BATCHING_LDS_TABLES", str(lds_tables))
+    all_bss = [1 << k for k in range(16)]
+    for seed, nb in enumerate([1, 3, 4, 5, 8, 9, 16] * 4):
+        c = random_case(4_000_000 + 100 * lanes + 10 * lds_tables + seed, max_m=7, max_g=5, max_s=6, max_r=150,
+                        nb=nb, load=2.0 + seed % 7, inf_slo=False)
+        bss = all_bss[:nb]
+        f0, g0, c0, _ = oracle_c.simulate_requests_mixed_batching(
+            c["tstamps"], c["model_ids"], c["slos"], c["m2g"], c["g2m"], c["num_stages"], c["lat"], bss)
+        fin, good, cnt = _single(eng, c, bss)
+        assert np.array_equal(good, g0), (seed, nb)
+        assert np.array_equal(fin.view(np.uint64), f0.view(np.uint64)), (seed, nb)
+        for a, b in zip(cnt, c0):
+            assert np.array_equal(a, b), (seed, nb)
+
+
 def test_groups_that_become_idle_at_the_same_instant(eng):
     """Idle events with equal times are popped in group order (the reference's heap holds (time, group)
     tuples, alpa_serve/simulator/controller.py:728-740).  Twelve identical one-stage groups all start a
