@@ -245,15 +245,19 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             // deadlines of up to eight heads are fetched together, the first eight ahead of that pass.
             int64_t q0 = base + h;
             int avail = (int)(arr - h) < 8 ? (int)(arr - h) : 8;
-            double dl[8];
+            double dl[8], tq[8];  // deadlines and arrival times (one 16-byte load per head)
 #pragma unroll
-            for (int k = 0; k < 8; ++k) dl[k] = a.mq[q0 + (k < avail ? k : avail - 1)].dl;
+            for (int k = 0; k < 8; ++k) {
+                const double2 v = *reinterpret_cast<const double2 *>(&a.mq[q0 + (k < avail ? k : avail - 1)]);
+                tq[k] = v.x;
+                dl[k] = v.y;
+            }
             double tb[NBT];
             batch_times(t0, gclk, stages, lat_mg, tb);
             const double alone = tb[0] + overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
             bool found = false;
             int64_t first = 0;
-            double deadline = 0.0;
+            double deadline = 0.0, first_t = 0.0;
             for (;;) {
                 for (int k = 0; k < avail; ++k) {
                     h += 1u;
@@ -261,6 +265,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                         found = true;
                         first = q0 + k;
                         deadline = dl[k];
+                        first_t = tq[k];
                         break;
                     }
                     if (want_group) group_req[g * kWave] += 1;
@@ -274,7 +279,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 q0 = base + h;
                 avail = (int)(arr - h) < 8 ? (int)(arr - h) : 8;
 #pragma unroll
-                for (int k = 0; k < 8; ++k) dl[k] = a.mq[q0 + (k < avail ? k : avail - 1)].dl;
+                for (int k = 0; k < 8; ++k) {
+                    const double2 v = *reinterpret_cast<const double2 *>(&a.mq[q0 + (k < avail ? k : avail - 1)]);
+                    tq[k] = v.x;
+                    dl[k] = v.y;
+                }
             }
             if (!found) {  // :709-713
                 head[m * LS] = h;
@@ -318,7 +327,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             }
             head[m * LS] = h + (uint32_t)(bs - 1);  // the batch is the arrivals first .. first+bs-1 of the model
             hrank[m * LS] = a.mq[first + bs].rank;
-            for (int u0 = 0; u0 < bs; u0 += 8) {  // arrival times of up to eight members fetched together
+            lat_sum += t - first_t;  // the first member's arrival time came with its deadline
+            if (want_req) {
+                const int32_t r = a.mq[first].idx;
+                fin_out[(size_t)r * kWave] = t;
+                good_out[(size_t)r * kWave] = 1;
+            }
+            for (int u0 = 1; u0 < bs; u0 += 8) {  // arrival times of up to eight more members fetched together
                 double at[8];
 #pragma unroll
                 for (int k = 0; k < 8; ++k) at[k] = a.mq[first + (u0 + k < bs ? u0 + k : bs - 1)].t;
