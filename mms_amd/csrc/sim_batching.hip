@@ -58,7 +58,10 @@ __device__ __forceinline__ lds_vu32 *as_lds_vu32(void *p) { return (lds_vu32 *)p
 // generic pointer the compiler may fold a constant of the index (the 31 of 31 - clz(batch size)) into
 // the instruction's offset field, and the hardware picks the aperture from the base register alone,
 // which then lies below the LDS aperture for a table at the start of LDS.
-template <int NBT, bool LATLDS, bool G2MLDS>
+// OCT: tiles of eight simulations, each worked on by an octet of consecutive lanes (lane = 8 * simulation
+// + helper).  The lanes of an octet hold the same state and take the same branches; the scans (event
+// slots, models of a group, replicas, heads' deadlines, latency columns) are split among them.
+template <int NBT, bool LATLDS, bool G2MLDS, bool OCT>
 __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching_kernel(const BatchingArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
@@ -71,7 +74,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const int M = a.M, Gmax = a.Gmax, NB = a.NB;
-    const int LS = a.lane_stride;  // lanes of a wavefront that simulate (64, 32, 16 or 8): pitch of the per-lane LDS arrays
+    const int LS = a.lane_stride;  // simulations per wavefront (64, 32, 16 or 8): pitch of the per-simulation LDS arrays
+    const int sl = OCT ? lane >> 3 : lane;  // this lane's simulation within the tile
+    const int oj = OCT ? lane & 7 : 0;      // this lane's place in its octet
+    const int fill = OCT ? kWave : LS;      // lanes that fill the wavefront's shared LDS arrays
 
     // ---- LDS: [latency table, shared, if it fits][per wavefront: group descriptors | clocks | event times |
     //      chunk minima | queue heads | head ranks | event groups | free slots | arrivals per model | offsets of
@@ -84,21 +90,21 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         for (int i = (int)threadIdx.x; i < n; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
     }
     unsigned char *mine = lds_raw + a.lat_lds_bytes + wv * a.wave_lds_bytes;
-    uint32_t *ginfo = reinterpret_cast<uint32_t *>(mine) + lane;
+    uint32_t *ginfo = reinterpret_cast<uint32_t *>(mine) + sl;
     size_t o = (size_t)(Gmax + 1) * LS * 4;
-    double *clk = reinterpret_cast<double *>(mine + o) + lane;
+    double *clk = reinterpret_cast<double *>(mine + o) + sl;
     o += (size_t)a.nslots * LS * 8;
-    double *ev_t = reinterpret_cast<double *>(mine + o) + lane;
+    double *ev_t = reinterpret_cast<double *>(mine + o) + sl;
     o += (size_t)a.heap_cap * LS * 8;
-    double *cm_t = reinterpret_cast<double *>(mine + o) + lane;  // earliest event time of each chunk
+    double *cm_t = reinterpret_cast<double *>(mine + o) + sl;  // earliest event time of each chunk
     o += (size_t)nch8 * LS * 8;
-    uint32_t *head = reinterpret_cast<uint32_t *>(mine + o) + lane;
+    uint32_t *head = reinterpret_cast<uint32_t *>(mine + o) + sl;
     o += (size_t)M * LS * 4;
-    int32_t *hrank = reinterpret_cast<int32_t *>(mine + o) + lane;  // rank of the arrival at head[m] (already known before it arrives)
+    int32_t *hrank = reinterpret_cast<int32_t *>(mine + o) + sl;  // rank of the arrival at head[m] (already known before it arrives)
     o += (size_t)M * LS * 4;
-    uint32_t *ev_g = reinterpret_cast<uint32_t *>(mine + o) + lane;
+    uint32_t *ev_g = reinterpret_cast<uint32_t *>(mine + o) + sl;
     o += (size_t)a.heap_cap * LS * 4;
-    uint16_t *fstack = reinterpret_cast<uint16_t *>(mine + o) + lane;  // free event slots, the next one to use on top
+    uint16_t *fstack = reinterpret_cast<uint16_t *>(mine + o) + sl;  // free event slots, the next one to use on top
     o += (size_t)a.heap_cap * LS * 2;
     // [M], same for all lanes; written by lane 0 and read by all, hence volatile (and spelled as an LDS
     // pointer: volatile accesses are not rewritten from generic to LDS by the compiler)
@@ -108,14 +114,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     o += ((size_t)(M + 1) * 8 + 15) & ~(size_t)15;
     int32_t *bsz = reinterpret_cast<int32_t *>(mine + o);  // [NB] batch sizes
     o += ((size_t)NB * 4 + 15) & ~(size_t)15;
-    uint16_t *g2m_off_lds = reinterpret_cast<uint16_t *>(mine + o) + lane;  // [Gmax+1][64]
+    uint16_t *g2m_off_lds = reinterpret_cast<uint16_t *>(mine + o) + sl;  // [Gmax+1][64]
     o += (size_t)(Gmax + 1) * LS * 2;
-    uint16_t *g2m_idx_lds = reinterpret_cast<uint16_t *>(mine + o) + lane;  // [members_max][64]
+    uint16_t *g2m_idx_lds = reinterpret_cast<uint16_t *>(mine + o) + sl;  // [members_max][64]
 
     const bool live = tile < a.tiles;
-    const bool sim = lane < LS;  // the other lanes of a narrow tile only help fetching requests
+    const bool sim = sl < LS;  // the other lanes of a narrow tile only help fetching requests
     if (live && sim) {
-        const uint32_t *gsrc = a.ginfo + (size_t)tile * (Gmax + 1) * kWave + lane;
+        const uint32_t *gsrc = a.ginfo + (size_t)tile * (Gmax + 1) * kWave + sl;
         for (int g = 0; g <= Gmax; ++g) ginfo[g * LS] = gsrc[g * kWave];
         for (int s = 0; s < a.nslots; ++s) clk[s * LS] = 0.0;
         for (int e = 0; e < a.heap_cap; ++e) {  // free event slots never win a minimum scan
@@ -126,17 +132,17 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         for (int c = 0; c < nch8; ++c) cm_t[c * LS] = __builtin_inf();
         {
             const int64_t *mo = a.mq_off + (size_t)seed * (M + 1);
-            for (int m = lane; m <= M; m += LS) mq_off[m] = mo[m];
-            for (int q = lane; q < NB; q += LS) bsz[q] = a.batch_sizes[q];
+            for (int m = lane; m <= M; m += fill) mq_off[m] = mo[m];
+            for (int q = lane; q < NB; q += fill) bsz[q] = a.batch_sizes[q];
             for (int m = 0; m < M; ++m) {
                 head[m * LS] = 0u;
                 hrank[m * LS] = a.mq[mo[m]].rank;  // of the model's first arrival (the padding entry if it has none)
             }
         }
-        for (int m = lane; m < M; m += LS) arrived[m] = 0u;
+        for (int m = lane; m < M; m += fill) arrived[m] = 0u;
         if (a.g2m_in_lds) {
-            const uint16_t *osrc = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
-            const uint16_t *isrc = a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
+            const uint16_t *osrc = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + sl;
+            const uint16_t *isrc = a.g2m_idx + (size_t)tile * a.members_max * kWave + sl;
             for (int g = 0; g <= Gmax; ++g) g2m_off_lds[g * LS] = osrc[g * kWave];
             for (int x = 0; x < a.members_max; ++x) g2m_idx_lds[x * LS] = isrc[(size_t)x * kWave];
         }
@@ -148,18 +154,18 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const int64_t off = a.stream_off[seed];
     const int64_t R = a.stream_off[seed + 1] - off;
     const Req *__restrict__ reqs = a.streams + off;
-    const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * M * kWave + lane;
-    const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * M * a.rep_extra * kWave + lane;
-    const uint16_t *g2m_off_glb = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + lane;
-    const uint16_t *g2m_idx_glb = a.g2m_idx + (size_t)tile * a.members_max * kWave + lane;
+    const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * M * kWave + sl;
+    const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * M * a.rep_extra * kWave + sl;
+    const uint16_t *g2m_off_glb = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + sl;
+    const uint16_t *g2m_idx_glb = a.g2m_idx + (size_t)tile * a.members_max * kWave + sl;
     auto g2m_off_at = [&](uint32_t g) -> int { return G2MLDS ? g2m_off_lds[g * LS] : g2m_off_glb[(size_t)g * kWave]; };
     auto g2m_idx_at = [&](int x) -> int { return G2MLDS ? g2m_idx_lds[x * LS] : g2m_idx_glb[(size_t)x * kWave]; };
     auto lat_at = [&](uint32_t i) -> float { return LATLDS ? lat_lds[i] : a.lat[i]; };
-    int32_t *model_good = a.model_good + (size_t)wave * M * kWave + lane;
-    int32_t *group_req = a.group_req + (size_t)wave * Gmax * kWave + lane;
-    int32_t *group_good = a.group_good + (size_t)wave * Gmax * kWave + lane;
-    double *fin_out = a.finish + (size_t)wave * a.Rmax * kWave + lane;
-    uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + lane;
+    int32_t *model_good = a.model_good + (size_t)wave * M * kWave + sl;
+    int32_t *group_req = a.group_req + (size_t)wave * Gmax * kWave + sl;
+    int32_t *group_good = a.group_good + (size_t)wave * Gmax * kWave + sl;
+    double *fin_out = a.finish + (size_t)wave * a.Rmax * kWave + sl;
+    uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + sl;
     const double overhead = a.fixed_overhead;
 
     int32_t n_good = 0;
@@ -268,7 +274,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                         first_t = tq[k];
                         break;
                     }
-                    if (want_group) group_req[g * kWave] += 1;
+                    if (want_group && oj == 0) group_req[g * kWave] += 1;
                     if (want_req) {
                         const MqEntry e = a.mq[q0 + k];
                         fin_out[(size_t)e.idx * kWave] = e.t;
@@ -347,11 +353,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 }
             }
             n_good += bs;
-            if (want_group) {
+            if (want_group && oj == 0) {  // the lanes of an octet would all add
                 group_req[g * kWave] += bs;
                 group_good[g * kWave] += bs;
             }
-            if (want_model) model_good[(size_t)m * kWave] += bs;
+            if (want_model && oj == 0) model_good[(size_t)m * kWave] += bs;
             if (nfree == 0) {
                 dead = MMSIM_E_OVERFLOW;
                 return;
@@ -541,10 +547,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         handle(ti, m2, g);
     }
 
-    const size_t out = (size_t)seed * a.tiles * kWave + (size_t)tile * kWave + lane;
-    a.n_good[out] = n_good;
-    a.lat_sum[out] = lat_sum;
-    a.status[out] = dead;
+    if (oj == 0) {
+        const size_t out = (size_t)seed * a.tiles * kWave + (size_t)tile * kWave + sl;
+        a.n_good[out] = n_good;
+        a.lat_sum[out] = lat_sum;
+        a.status[out] = dead;
+    }
 }
 
 }  // namespace
@@ -556,10 +564,12 @@ hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_byt
         e = hipErrorInvalidValue;
     } else {
         const bool ll = args.lat_lds_bytes > 0, gl = args.g2m_in_lds != 0;
+        const bool oct = args.lane_stride == 8;
         void (*kern)(const BatchingArgs) = nullptr;
-#define MMSIM_PICK(NBT)                                                                    \
-    kern = ll ? (gl ? sim_batching_kernel<NBT, true, true> : sim_batching_kernel<NBT, true, false>) \
-              : (gl ? sim_batching_kernel<NBT, false, true> : sim_batching_kernel<NBT, false, false>)
+#define MMSIM_PICK2(NBT, O)                                                                         \
+    (ll ? (gl ? sim_batching_kernel<NBT, true, true, O> : sim_batching_kernel<NBT, true, false, O>) \
+        : (gl ? sim_batching_kernel<NBT, false, true, O> : sim_batching_kernel<NBT, false, false, O>))
+#define MMSIM_PICK(NBT) kern = oct ? MMSIM_PICK2(NBT, true) : MMSIM_PICK2(NBT, false)
         if (args.NB <= 4)
             MMSIM_PICK(4);
         else if (args.NB <= 8)
@@ -567,6 +577,7 @@ hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_byt
         else
             MMSIM_PICK(16);
 #undef MMSIM_PICK
+#undef MMSIM_PICK2
         if (lds_bytes > 64 * 1024)
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)lds_bytes);
