@@ -49,6 +49,67 @@ __device__ __forceinline__ double max_nn(double x, double y) {
 }
 __device__ __forceinline__ int ilog2i(int v) { return 31 - __clz(v); }
 
+// ---- octet primitives.  An octet is eight consecutive lanes that work on one simulation; its lanes are
+// always converged when they call these (they hold the same state and take the same branches).
+// <octet primitives>
+__device__ __forceinline__ int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+// bit j = the predicate of lane j of the octet
+__device__ __forceinline__ uint32_t oct_ballot(bool p) {
+    const uint64_t b = __builtin_amdgcn_ballot_w64(p);
+    return (uint32_t)(b >> (lane_id() & 56)) & 0xFFu;
+}
+// exchange with the lane whose index differs in bit 0, bit 1, or with the mirror lane of the octet:
+// three rounds of it reach all eight lanes
+template <int STEP>
+__device__ __forceinline__ uint32_t oct_swap(uint32_t v) {
+    constexpr int ctrl = STEP == 0 ? 0xB1 /* quad_perm 1,0,3,2 */ : STEP == 1 ? 0x4E /* quad_perm 2,3,0,1 */ : 0x141 /* row_half_mirror */;
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, ctrl, 0xF, 0xF, false);
+}
+template <int STEP>
+__device__ __forceinline__ double oct_swap(double v) {
+    return __hiloint2double((int)oct_swap<STEP>((uint32_t)__double2hiint(v)), (int)oct_swap<STEP>((uint32_t)__double2loint(v)));
+}
+template <int STEP>
+__device__ __forceinline__ uint64_t oct_swap(uint64_t v) {
+    return ((uint64_t)oct_swap<STEP>((uint32_t)(v >> 32)) << 32) | oct_swap<STEP>((uint32_t)v);
+}
+// the value of lane k of the octet (k may differ from lane to lane)
+__device__ __forceinline__ uint32_t oct_get(uint32_t v, int k) {
+    return (uint32_t)__builtin_amdgcn_ds_bpermute(((lane_id() & 56) | k) << 2, (int)v);
+}
+__device__ __forceinline__ double oct_get(double v, int k) {
+    return __hiloint2double((int)oct_get((uint32_t)__double2hiint(v), k), (int)oct_get((uint32_t)__double2loint(v), k));
+}
+// The lanes of an octet run in lockstep; this marks the places where that matters (all have read a
+// value before any of them overwrites it).  No instruction.
+__device__ __forceinline__ void oct_sync() { __builtin_amdgcn_wave_barrier(); }
+// </octet primitives>
+// minimum over the octet, in all of its lanes (doubles are never NaN here)
+__device__ __forceinline__ double oct_min(double v) {
+    double w = oct_swap<0>(v);
+    v = w < v ? w : v;
+    w = oct_swap<1>(v);
+    v = w < v ? w : v;
+    w = oct_swap<2>(v);
+    return w < v ? w : v;
+}
+__device__ __forceinline__ uint32_t oct_min(uint32_t v) {
+    uint32_t w = oct_swap<0>(v);
+    v = w < v ? w : v;
+    w = oct_swap<1>(v);
+    v = w < v ? w : v;
+    w = oct_swap<2>(v);
+    return w < v ? w : v;
+}
+__device__ __forceinline__ uint64_t oct_min(uint64_t v) {
+    uint64_t w = oct_swap<0>(v);
+    v = w < v ? w : v;
+    w = oct_swap<1>(v);
+    v = w < v ? w : v;
+    w = oct_swap<2>(v);
+    return w < v ? w : v;
+}
+
 typedef volatile __attribute__((address_space(3))) uint32_t lds_vu32;
 __device__ __forceinline__ lds_vu32 *as_lds_vu32(void *p) { return (lds_vu32 *)p; }
 
@@ -181,6 +242,21 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     // :654-664 -- among the models of group g with a waiting request, the one whose head arrived first
     auto select_model = [&](uint32_t g) -> int {
         const int lo = g2m_off_at(g), hi = g2m_off_at(g + 1u);
+        if constexpr (OCT) {
+            // one model per lane; the key orders by rank of the head's arrival, then by place in the list
+            uint64_t best = ~0ull;
+            for (int x0 = lo; x0 < hi; x0 += 8) {
+                const int x = x0 + oj;
+                const int mm = g2m_idx_at(x < hi ? x : hi - 1);
+                const uint32_t rk = (uint32_t)hrank[mm * LS];
+                const uint32_t hd = head[mm * LS], ar = arrived[mm];
+                const bool waiting = x < hi && (int)(ar - hd) > 0;
+                const uint64_t key = waiting ? ((uint64_t)rk << 32) | ((uint64_t)(uint32_t)(x - lo) << 16) | (uint32_t)mm : ~0ull;
+                const uint64_t k = oct_min(key);
+                best = k < best ? k : best;
+            }
+            return best == ~0ull ? -1 : (int)(best & 0xFFFFu);
+        }
         int min_rank = 0x7FFFFFFF;
         int pick = -1;
         for (int x0 = lo; x0 < hi; x0 += 4) {  // four models at a time: their reads overlap
@@ -236,6 +312,31 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         }
     };
 
+    // the same for one latency column (the octet's lanes take one column each)
+    auto batch_time_col = [&](double t0, const double *gclk, int stages, uint32_t lat_mg, int col) -> double {
+        double t = t0;
+        for (int k0 = 0; k0 < stages; k0 += 4) {
+            double c[4];
+            float l[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int k = k0 + u < stages ? k0 + u : stages - 1;
+                c[u] = gclk[k * LS];
+                l[u] = lat_at(lat_mg + (uint32_t)(k * NB + col));
+            }
+#pragma unroll
+            for (int u = 1; u < 4; ++u)
+                if (!(k0 + u < stages)) {
+                    c[u] = -__builtin_inf();
+                    l[u] = 0.0f;
+                }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t = max_nn(c[u], t) + (double)l[u];
+        }
+        return t;
+    };
+    constexpr bool COOP = OCT && NBT <= 8;  // batch attempts split over the octet (one latency column per lane)
+
     // :706-732 with :674-704 inlined; the reference's recursion on "nothing servable" is the outer loop
     auto handle = [&](double t0, int m, uint32_t g) {
         const uint32_t d = ginfo[g * LS];
@@ -246,11 +347,57 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             const int64_t base = mq_off[m];
             const uint32_t arr = arrived[m];  // does not change while a lane is in here
             uint32_t h = head[m * LS];        // arr - h > 0: the caller saw a waiting request
+            if constexpr (OCT) oct_sync();
             // drop heads that cannot meet their deadline even alone (:677-686).  The finish time of a
             // batch of one does not depend on which request it is, so it is computed once; the
             // deadlines of up to eight heads are fetched together, the first eight ahead of that pass.
             int64_t q0 = base + h;
             int avail = (int)(arr - h) < 8 ? (int)(arr - h) : 8;
+            bool found = false;
+            int64_t first = 0;
+            double deadline = 0.0, first_t = 0.0;
+            int bs = 1;
+            if constexpr (COOP) {
+                // lane j of the octet takes head j of the queue and latency column j
+                double2 hv = *reinterpret_cast<const double2 *>(&a.mq[q0 + (oj < avail ? oj : avail - 1)]);
+                const double tcol = batch_time_col(t0, gclk, stages, lat_mg, oj < NB ? oj : NB - 1);
+                const double alone = oct_get(tcol, 0) + overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
+                for (;;) {
+                    const uint32_t pass = oct_ballot(oj < avail && alone <= hv.y);
+                    const int k = pass ? __ffs((int)pass) - 1 : avail;  // the heads before k are dropped
+                    if (oj < k) {
+                        if (want_req) {
+                            const MqEntry e = a.mq[q0 + oj];
+                            fin_out[(size_t)e.idx * kWave] = e.t;
+                            good_out[(size_t)e.idx * kWave] = 0;
+                        }
+                    }
+                    if (want_group && oj == 0) group_req[g * kWave] += k;
+                    if (pass) {
+                        found = true;
+                        first = q0 + k;
+                        deadline = oct_get(hv.y, k);
+                        first_t = oct_get(hv.x, k);
+                        h += (uint32_t)(k + 1);
+                        break;
+                    }
+                    h += (uint32_t)avail;
+                    if (h == arr) break;
+                    q0 = base + h;
+                    avail = (int)(arr - h) < 8 ? (int)(arr - h) : 8;
+                    hv = *reinterpret_cast<const double2 *>(&a.mq[q0 + (oj < avail ? oj : avail - 1)]);
+                }
+                if (found) {
+                    // grow the batch while the first request still meets its deadline (:693-702): lane b tests
+                    // batch size b, the batch is the last size before the first one that fails
+                    const int cand = bsz[oj < NB ? oj : NB - 1];
+                    const double tc = oct_get(tcol, ilog2i(cand));
+                    const bool ok = oj == 0 || (oj < NB && cand - 1 <= (int)(arr - h) && (tc + overhead) <= deadline);
+                    const uint32_t fail = ~oct_ballot(ok) & 0xFFu;
+                    const int nb_ok = fail ? __ffs((int)fail) - 1 : 8;
+                    bs = bsz[nb_ok - 1];
+                }
+            } else {
             double dl[8], tq[8];  // deadlines and arrival times (one 16-byte load per head)
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
@@ -261,9 +408,6 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             double tb[NBT];
             batch_times(t0, gclk, stages, lat_mg, tb);
             const double alone = tb[0] + overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
-            bool found = false;
-            int64_t first = 0;
-            double deadline = 0.0, first_t = 0.0;
             for (;;) {
                 for (int k = 0; k < avail; ++k) {
                     h += 1u;
@@ -291,24 +435,26 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                     dl[k] = v.y;
                 }
             }
+            if (found) {
+                // grow the batch while the first request still meets its deadline (:693-702)
+                for (int b = 1; b < NB; ++b) {
+                    const int cand = bsz[b];
+                    if (cand - 1 > (int)(arr - h)) break;
+                    const int col = ilog2i(cand);
+                    double tc = tb[0];
+#pragma unroll
+                    for (int x = 1; x < NBT; ++x) tc = col == x ? tb[x] : tc;
+                    if (!((tc + overhead) <= deadline)) break;
+                    bs = cand;
+                }
+            }
+            }
             if (!found) {  // :709-713
                 head[m * LS] = h;
                 hrank[m * LS] = a.mq[base + h].rank;
                 m = select_model(g);
                 if (m < 0) return;
                 continue;
-            }
-            // grow the batch while the first request still meets its deadline (:693-702)
-            int bs = 1;
-            for (int b = 1; b < NB; ++b) {
-                const int cand = bsz[b];
-                if (cand - 1 > (int)(arr - h)) break;
-                const int col = ilog2i(cand);
-                double tc = tb[0];
-#pragma unroll
-                for (int x = 1; x < NBT; ++x) tc = col == x ? tb[x] : tc;
-                if (!((tc + overhead) <= deadline)) break;
-                bs = cand;
             }
             // run it (:715-732)
             const int col = ilog2i(bs);
@@ -323,6 +469,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                     c[u] = gclk[k * LS];
                     l[u] = lat_at(lat_mg + (uint32_t)(k * NB + col));
                 }
+                if constexpr (OCT) oct_sync();
 #pragma unroll
                 for (int u = 0; u < 4; ++u)
                     if (k0 + u < stages) {
@@ -379,6 +526,22 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         T = __builtin_inf();
         others = __builtin_inf();
         cj = 0;
+        if constexpr (OCT) {
+            for (int c0 = 0; c0 < nch; c0 += 8) {  // one chunk minimum per lane
+                const double v = cm_t[(c0 + oj) * LS];
+                const double mn = oct_min(v);
+                const int first = __ffs((int)oct_ballot(v == mn)) - 1;
+                const double rest = oct_min(oj == first ? __builtin_inf() : v);
+                if (mn < T) {
+                    others = T < rest ? T : rest;  // the previous earliest is now one of the others
+                    T = mn;
+                    cj = c0 + first;
+                } else {
+                    others = mn < others ? mn : others;
+                }
+            }
+            return;
+        }
         for (int c0 = 0; c0 < nch; c0 += 8) {
             double v[8];
 #pragma unroll
@@ -413,6 +576,24 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 }
             }
             cj = be >> 3;
+        }
+        if constexpr (OCT) {
+            // one slot of the chunk per lane
+            const int e = (cj << 3) + oj;
+            const double t = ev_t[e * LS];
+            if (others != T) {
+                const uint32_t g = ev_g[e * LS];
+                bg = oct_min(t == T ? g : 0xFFFFFFFFu);
+                be = (cj << 3) + __ffs((int)oct_ballot(t == T && g == bg)) - 1;
+            }
+            const double left = oct_min(e == be ? __builtin_inf() : t);  // earliest time left in the chunk
+            ev_t[be * LS] = __builtin_inf();
+            ev_g[be * LS] = 0xFFFFFFFFu;
+            cm_t[cj * LS] = left;
+            fstack[nfree * LS] = (uint16_t)be;
+            nfree += 1;
+            next_due = left < others ? left : others;
+            return bg;
         }
         double t[8];
         uint32_t g[8];
@@ -487,7 +668,19 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 // group with the strictly smallest last-stage clock (:760-770)
                 double best = 1e100;
                 bool more = true;  // the list may go on
-                for (int j0 = 0; j0 < kPackedReplicas && more; j0 += 4) {  // four replicas at a time: their reads overlap
+                if constexpr (OCT) {
+                    // one replica per lane; the first of the smallest clocks wins, as in a scan with "<"
+                    const uint32_t g = (uint32_t)(g8 >> (8 * oj)) & 0xFFu;
+                    const double c = clk[desc_last_slot(ginfo[g * LS]) * LS];  // the empty row for unused bytes
+                    const double mn = oct_min(g != none ? c : __builtin_inf());
+                    if (mn < best) {
+                        best = mn;
+                        const int first = __ffs((int)oct_ballot(g != none && c == mn)) - 1;
+                        gsel = (uint32_t)(g8 >> (8 * first)) & 0xFFu;
+                    }
+                    more = ((uint32_t)(g8 >> 56) & 0xFFu) != none;
+                }
+                for (int j0 = 0; !OCT && j0 < kPackedReplicas && more; j0 += 4) {  // four replicas at a time: their reads overlap
                     uint32_t g[4], d[4];
                     double c[4];
 #pragma unroll
