@@ -85,6 +85,71 @@ def solve_separation_placement(self, eco_separation: List[Tuple[List[ModelData],
     return sol
 
 
+def solve_separations_lockstep(self, separations, model_id_map, model_datas: List[ModelData],
+                               cluster_env: ClusterEnv, train_workload: Workload):
+    """``solve_separation_placement`` for every separation, with all greedy searches advanced together.
+
+    The reference solves each (model cluster, device share) of each separation with its own evaluator
+    over the full training workload, in which the other clusters' requests name unknown models and are
+    skipped (:244-255, :323-353).  A placement that hosts only the cluster's models, scored on the same
+    workload under the global model ids, gives the same counts for those models and the same score, so
+    one evaluator serves all sub-problems: every iteration scores the current placement of every search
+    (all layouts of all distinct sub-problems) in one call.  A sub-problem is a (cluster, device count)
+    pair; separations share them, so each is solved once.  Returns one stitched placement per separation,
+    equal to what solving them one by one returns."""
+    from types import SimpleNamespace
+    from mms_amd.placement_policy.base_policy import _fast_greedy_step, weight_mem_table
+    evaluator = PlacementEvaluator(model_datas, cluster_env, train_workload,
+                                   self.evaluator_method, self.parallel_evaluator)
+    subs = {}
+    for sep in separations:
+        for ci, (sub_model_datas, sub_env) in enumerate(sep):
+            key = (ci, sub_env.num_devices)
+            if key not in subs:
+                subs[key] = SimpleNamespace(
+                    model_datas=sub_model_datas, env=sub_env,
+                    gmap=[model_id_map[(ci, j)] for j in range(len(sub_model_datas))],
+                    sols=self.enumerate_group_configs_uneven(sub_env))
+
+    def to_global(sub, sol):
+        return ModelPlacement(list(sol.group_configs), [[sub.gmap[m] for m in ms] for ms in sol.group_models])
+
+    searches = [(sub, i) for sub in subs.values() for i in range(len(sub.sols))]
+    weight_mems = [weight_mem_table(sub.sols[i].group_configs, sub.model_datas) for sub, i in searches]
+    running = list(range(len(searches)))
+    while running:
+        all_stats = evaluator.get_stats([to_global(searches[r][0], searches[r][0].sols[searches[r][1]])
+                                         for r in running])
+        still = []
+        for r, (overall, goodputs, group_num_requests, full) in zip(running, all_stats):
+            sub, i = searches[r]
+            sol = sub.sols[i]
+            local = (overall, [goodputs[g] for g in sub.gmap], group_num_requests,
+                     SimpleNamespace(per_model_stats=[full.per_model_stats[g] for g in sub.gmap]))
+            choice = _fast_greedy_step(sol, local, weight_mems[r], sub.env)
+            if choice is not None:
+                sub.sols[i] = sol.add_model(*choice).normalize()
+                still.append(r)
+        running = still
+    # the best layout of every sub-problem (first of equal scores, as np.argmax in :353)
+    finals = [to_global(sub, sol) for sub in subs.values() for sol in sub.sols]
+    scores = evaluator.get_scores(finals)
+    at = 0
+    for sub in subs.values():
+        n = len(sub.sols)
+        sub.best = sub.sols[int(np.argmax(scores[at:at + n]))]
+        at += n
+    stitched = []
+    for sep in separations:
+        sol = ModelPlacement([], [])
+        for ci, (_, sub_env) in enumerate(sep):
+            sub = subs[(ci, sub_env.num_devices)]
+            sol.group_configs += list(sub.best.group_configs)
+            sol.group_models += [[sub.gmap[m] for m in group] for group in sub.best.group_models]
+        stitched.append(sol)
+    return stitched
+
+
 class ModelParallelismSearch(BasePlacementPolicy):
     """Enumerate group partitions, fill each greedily, keep the best score."""
 
@@ -165,7 +230,8 @@ class ModelParallelismSearch(BasePlacementPolicy):
         if self.use_separation:
             separations, model_id_map = self.enumerate_separations(model_datas, cluster_env)
             print("number of combinations: ", len(separations))
-            sols = [solve_separation_placement(self, sep, model_id_map, train_workload) for sep in separations]
+            sols = solve_separations_lockstep(self, separations, model_id_map, model_datas, cluster_env,
+                                              train_workload)
             evaluator = PlacementEvaluator(model_datas, cluster_env, train_workload,
                                            self.evaluator_method, self.parallel_evaluator)
             scores = evaluator.get_scores(sols)

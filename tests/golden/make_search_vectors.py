@@ -59,7 +59,14 @@ def main():
     cases = []
 
     def record(name, policy_name, kwargs, model_spec, cluster_spec):
-        model_datas = models(*model_spec)
+        # model_spec: (n, slo, rate, cv[, profile]) or a list of such tuples (models m0, m1, ... in that order)
+        if isinstance(model_spec, list):
+            model_datas = []
+            for n, slo, rate, cv, prof_name in model_spec:
+                model_datas += [pp.ModelData(f"m{len(model_datas) + i}", slo, rate, cv,
+                                             prof.load_test_prof_result(prof_name)) for i in range(n)]
+        else:
+            model_datas = models(*model_spec)
         cluster_env = pp.ClusterEnv(*cluster_spec)
         policy = getattr(pp, policy_name)(**kwargs)
         placement, _ = policy.solve_placement(model_datas, cluster_env)
@@ -68,10 +75,22 @@ def main():
         score = float(ev.get_scores([placement])[0])
         stats = ev.get_stats([placement])[0]
         cases.append({"name": name, "policy": policy_name, "kwargs": kwargs,
-                      "models": list(model_spec), "cluster": list(cluster_spec),
+                      "models": [list(x) for x in model_spec] if isinstance(model_spec, list) else list(model_spec),
+                      "cluster": list(cluster_spec),
                       "placement": dump(placement), "score": score,
                       "goodput": float(stats[0]),
                       "group_num_requests": [int(x) for x in stats[2]]})
+        if kwargs.get("use_separation"):
+            # the best of the separated solutions too (the search may prefer the unseparated one)
+            import alpa_serve.placement_policy.model_parallelism as mp
+            separations, model_id_map = policy.enumerate_separations(model_datas, cluster_env)
+            sols = [mp.solve_separation_placement(policy, sep, model_id_map, wl) for sep in separations]
+            # (a fresh evaluator: the sub-problems' evaluators replaced the workload's cached model ids)
+            ev2 = pp.base_policy.PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+            scores = [float(x) for x in ev2.get_scores(sols)]
+            best = int(np.argmax(scores))
+            cases[-1]["separations"] = {"count": len(separations), "scores": scores,
+                                        "best": dump(sols[best]), "best_score": scores[best]}
         print(name, dump(placement)["group_models"], score, flush=True)
 
     # the three situations of the reference's own test
@@ -83,6 +102,10 @@ def main():
     record("loaded_sr_greedy", "SelectiveReplicationGreedy", {}, (4, 0.5, 9, 4), (4, 4.5 * GB))
     record("loaded_mp_greedy", "ModelParallelismGreedy", {"group_size": 2}, (6, 0.4, 6, 4), (4, 6.5 * GB))
     record("loaded_mp_search", "ModelParallelismSearch", {}, (5, 0.5, 7, 6, "test-4GB-150ms"), (8, 8.5 * GB))
+
+    # two kinds of models: the search also splits the devices between them (model_parallelism.py:356-456)
+    record("separation_mp_search", "ModelParallelismSearch", {"use_separation": True},
+           [(3, 0.5, 5, 3, "test-2GB-100ms"), (2, 0.9, 3, 2, "test-4GB-150ms")], (6, 8.5 * GB))
 
     path = os.path.join(HERE, "search_vectors.json")
     with open(path, "w") as f:

@@ -51,9 +51,15 @@ def test_policies_return_what_the_reference_returns(backend, case):
     """Final placement, its score, goodput and per-group request counts as
     recorded from the reference's own policies (tests/golden/make_search_vectors.py)."""
     import mms_amd.placement_policy as pp
-    n, slo, rate, cv = case["models"][:4]
-    prof = case["models"][4] if len(case["models"]) > 4 else "test-2GB-100ms"
-    model_datas = [ModelData(f"m{i}", slo, rate, cv, load_test_prof_result(prof)) for i in range(n)]
+    if isinstance(case["models"][0], list):     # several kinds of models: [n, slo, rate, cv, profile] each
+        model_datas = []
+        for n, slo, rate, cv, prof in case["models"]:
+            model_datas += [ModelData(f"m{len(model_datas) + i}", slo, rate, cv, load_test_prof_result(prof))
+                            for i in range(n)]
+    else:
+        n, slo, rate, cv = case["models"][:4]
+        prof = case["models"][4] if len(case["models"]) > 4 else "test-2GB-100ms"
+        model_datas = [ModelData(f"m{i}", slo, rate, cv, load_test_prof_result(prof)) for i in range(n)]
     cluster_env = ClusterEnv(*case["cluster"])
     placement, _ = getattr(pp, case["policy"])(**case["kwargs"]).solve_placement(model_datas, cluster_env)
     assert [list(c) for c in placement.group_configs] == case["placement"]["group_configs"]
@@ -65,6 +71,19 @@ def test_policies_return_what_the_reference_returns(backend, case):
     goodput, _, group_num_requests, _ = ev.get_stats([placement])[0]
     assert goodput == case["goodput"]
     assert [int(x) for x in group_num_requests] == case["group_num_requests"]
+    if "separations" in case:
+        # the separated solutions the reference builds on the way (model_parallelism.py:430-440), their scores,
+        # and the best of them
+        from mms_amd.placement_policy.model_parallelism import solve_separations_lockstep
+        policy = getattr(pp, case["policy"])(**case["kwargs"])
+        separations, model_id_map = policy.enumerate_separations(model_datas, cluster_env)
+        assert len(separations) == case["separations"]["count"]
+        sols = solve_separations_lockstep(policy, separations, model_id_map, model_datas, cluster_env, wl)
+        scores = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False).get_scores(sols)
+        np.testing.assert_allclose(scores, case["separations"]["scores"], rtol=1e-12, atol=0)
+        best = sols[int(np.argmax(scores))]
+        assert [list(c) for c in best.group_configs] == case["separations"]["best"]["group_configs"]
+        assert [[int(m) for m in ms] for ms in best.group_models] == case["separations"]["best"]["group_models"]
 
 
 def test_assertions_of_the_reference_test_file(backend):
@@ -237,6 +256,25 @@ def test_greedy_searches_in_lockstep_take_the_steps_they_take_alone(backend):
     together = replica_placement_fast_greedy_lockstep(starts, model_datas, cluster_env, wl, ev, 0)
     assert [str(a) for a in alone] == [str(t) for t in together]
     assert Counting.calls < calls_alone / 2
+
+
+def test_separations_solved_together_equal_separations_solved_one_by_one(backend):
+    """model_parallelism.py:432-434 solves every separation on its own; here all their greedy searches
+    share one evaluator and advance together.  Same stitched placements."""
+    from mms_amd.placement_policy.model_parallelism import (solve_separation_placement,
+                                                            solve_separations_lockstep)
+    mixed = ([ModelData(f"a{i}", 0.5, 3 + i, 3, load_test_prof_result("test-2GB-100ms")) for i in range(3)] +
+             [ModelData(f"b{i}", 0.9, 2 + i, 2, load_test_prof_result("test-4GB-150ms")) for i in range(2)])
+    cluster_env = ClusterEnv(6, 8.5 * GB)
+    wl = gen_train_workload(mixed, simulation_min_samples=3000)
+    policy = ModelParallelismSearch(use_separation=True)
+    separations, model_id_map = policy.enumerate_separations(mixed, cluster_env)
+    assert len(separations) >= 3
+    one_by_one = [solve_separation_placement(policy, sep, model_id_map, wl) for sep in separations]
+    together = solve_separations_lockstep(policy, separations, model_id_map, mixed, cluster_env, wl)
+    assert [str(a) for a in one_by_one] == [str(b) for b in together]
+    for sol in together:
+        sol.verify(mixed, cluster_env)
 
 
 def test_batching_evaluator(backend, monkeypatch):
