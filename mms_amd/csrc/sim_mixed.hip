@@ -459,8 +459,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 }
                 if (want_group && has) {  // :611, :618
                     const uint32_t g = owner[(last_addr - clk_off) >> 3];  // (slot * 512 + lane * 8) / 8
-                    gcnt[g * kWave] += 1u;
-                    if (acc) gcnt[(a.Gmax + g) * kWave] += 1u;
+                    // LDS adds that return nothing: the wavefront does not wait for them
+                    __hip_atomic_fetch_add(&gcnt[g * kWave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+                    __hip_atomic_fetch_add(&gcnt[(a.Gmax + g) * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_WAVEFRONT);
                 }
                 if (want_ops) {
                     asm volatile("" ::: "memory");  // keep this a wave-uniform branch, off the common path
