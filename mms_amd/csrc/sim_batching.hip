@@ -451,12 +451,17 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             }
             if (!found) {  // :709-713
                 head[m * LS] = h;
-                hrank[m * LS] = a.mq[base + h].rank;
-                m = select_model(g);
+                // the rank of this model's next arrival is not needed to pick another model (this one has
+                // nothing waiting), so its fetch overlaps the selection
+                const int32_t next_rank = a.mq[base + h].rank;
+                const int m_next = select_model(g);
+                hrank[m * LS] = next_rank;
+                m = m_next;
                 if (m < 0) return;
                 continue;
             }
-            // run it (:715-732)
+            // run it (:715-732); the rank of the arrival after the batch is fetched meanwhile
+            const int32_t next_rank = a.mq[first + bs].rank;
             const int col = ilog2i(bs);
             double t = t0 + overhead;
             double idle_at = 0.0;
@@ -479,7 +484,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                     }
             }
             head[m * LS] = h + (uint32_t)(bs - 1);  // the batch is the arrivals first .. first+bs-1 of the model
-            hrank[m * LS] = a.mq[first + bs].rank;
+            hrank[m * LS] = next_rank;
             lat_sum += t - first_t;  // the first member's arrival time came with its deadline
             if (want_req) {
                 const int32_t r = a.mq[first].idx;
