@@ -18,6 +18,10 @@
  *   mmsim_simulate_requests_mixed_batching
  *       simulate_requests_mixed_batching, same argument list
  *       (alpa_serve/simulator/controller.py:631-798; called at :486-489).
+ *   mmsim_simulate_requests
+ *       the numba kernel simulate_requests (one clock per group), same
+ *       argument list (alpa_serve/simulator/controller.py:506-558; called at
+ *       :496-499 when mixed is False, which no caller of the reference passes).
  *   mmsim_workload_create
  *       the per-workload arrays approximate_one_case derives once and caches:
  *       arrivals, model_ids (int32) and slos (float32)
@@ -198,6 +202,15 @@ int mmsim_simulate_requests_mixed(
     const int32_t *model_ids, const float *slos, const int32_t *m_id2g_id,
     const int32_t *num_stages, const float *stage_latency, int64_t num_requests,
     int32_t M, int32_t G, int32_t Smax, double fixed_overhead,
+    int32_t *model_num_requests, int32_t *model_num_good_requests,
+    int32_t *group_num_requests, int32_t *group_num_good_requests);
+
+/* group_max_latency, group_sum_latency: [M][G] float32 (controller.py:433-443) */
+int mmsim_simulate_requests(
+    mmsim_ctx *ctx, double *finish, uint8_t *good, const double *tstamps,
+    const int32_t *model_ids, const float *slos, const int32_t *m_id2g_id,
+    const float *group_max_latency, const float *group_sum_latency, int64_t num_requests,
+    int32_t M, int32_t G, double fixed_overhead,
     int32_t *model_num_requests, int32_t *model_num_good_requests,
     int32_t *group_num_requests, int32_t *group_num_good_requests);
 

@@ -83,6 +83,9 @@ SIGNATURES = {
     "mmsim_simulate_requests_mixed": (C.c_int, [
         C.c_void_p, _p_f64, _p_u8, _p_f64, _p_i32, _p_f32, _p_i32, _p_i32, _p_f32, C.c_int64,
         C.c_int32, C.c_int32, C.c_int32, C.c_double, _p_i32, _p_i32, _p_i32, _p_i32]),
+    "mmsim_simulate_requests": (C.c_int, [
+        C.c_void_p, _p_f64, _p_u8, _p_f64, _p_i32, _p_f32, _p_i32, _p_f32, _p_f32, C.c_int64,
+        C.c_int32, C.c_int32, C.c_double, _p_i32, _p_i32, _p_i32, _p_i32]),
     "mmsim_simulate_requests_mixed_batching": (C.c_int, [
         C.c_void_p, _p_f64, _p_u8, _p_f64, _p_i32, _p_f32, _p_i32, _p_i32, _p_i32, _p_f32, _p_i32,
         C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_double,

@@ -16,7 +16,7 @@ PKG = os.path.dirname(HERE)
 OUT = os.path.join(PKG, "libmmsim.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["mmsim_api.hip", "sim_mixed.hip", "sim_batching.hip"]
+SOURCES = ["mmsim_api.hip", "sim_mixed.hip", "sim_batching.hip", "sim_scalar.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -1274,6 +1274,89 @@ int mmsim_simulate_requests_mixed(mmsim_ctx *ctx, double *finish, uint8_t *good,
     return rc;
 }
 
+int mmsim_simulate_requests(mmsim_ctx *ctx, double *finish, uint8_t *good, const double *tstamps,
+                            const int32_t *model_ids, const float *slos, const int32_t *m_id2g_id,
+                            const float *group_max_latency, const float *group_sum_latency, int64_t num_requests,
+                            int32_t M, int32_t G, double fixed_overhead,
+                            int32_t *model_num_requests, int32_t *model_num_good_requests,
+                            int32_t *group_num_requests, int32_t *group_num_good_requests) {
+    if (!ctx) return fail(MMSIM_E_INVALID, "simulate_requests: null context");
+    if (M < 1 || G < 1 || num_requests < 0) return fail(MMSIM_E_INVALID, "simulate_requests: bad size");
+    if (!m_id2g_id || !group_max_latency || !group_sum_latency || !model_num_requests || !model_num_good_requests ||
+        !group_num_requests || !group_num_good_requests ||
+        (num_requests > 0 && (!finish || !good || !tstamps || !model_ids || !slos)))
+        return fail(MMSIM_E_INVALID, "simulate_requests: null pointer");
+    if (G > MMSIM_MAX_GROUPS) return fail(MMSIM_E_UNSUPPORTED, "simulate_requests: more than 254 groups");
+    for (size_t i = 0; i < (size_t)M * G; ++i) {
+        if (m_id2g_id[i] >= G) return fail(MMSIM_E_INVALID, "simulate_requests: m_id2g_id names a group >= G");
+        if (group_max_latency[i] != group_max_latency[i] || group_sum_latency[i] != group_sum_latency[i] ||
+            group_max_latency[i] < 0.0f || group_sum_latency[i] < 0.0f)
+            return fail(MMSIM_E_INVALID, "simulate_requests: a latency is NaN or negative");
+    }
+    for (int64_t i = 0; i < num_requests; ++i) {
+        if (tstamps[i] != tstamps[i]) return fail(MMSIM_E_INVALID, "simulate_requests: an arrival time is NaN");
+        if (model_ids[i] >= M) return fail(MMSIM_E_INVALID, "simulate_requests: a request names a model >= M");
+    }
+    std::memset(model_num_requests, 0, sizeof(int32_t) * (size_t)M);
+    std::memset(model_num_good_requests, 0, sizeof(int32_t) * (size_t)M);
+    std::memset(group_num_requests, 0, sizeof(int32_t) * (size_t)G);
+    std::memset(group_num_good_requests, 0, sizeof(int32_t) * (size_t)G);
+    if (num_requests == 0) return MMSIM_OK;
+
+    HIP_TRY(hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    const size_t R = (size_t)num_requests, MG = (size_t)M * G;
+    DevBuf<double> d_t, d_fin;
+    DevBuf<int32_t> d_m, d_m2g, d_cnt;
+    DevBuf<float> d_slo, d_max, d_sum;
+    DevBuf<uint8_t> d_good;
+    HIP_TRY(d_t.alloc(R));
+    HIP_TRY(d_fin.alloc(R));
+    HIP_TRY(d_m.alloc(R));
+    HIP_TRY(d_slo.alloc(R));
+    HIP_TRY(d_good.alloc(R));
+    HIP_TRY(d_m2g.alloc(MG));
+    HIP_TRY(d_max.alloc(MG));
+    HIP_TRY(d_sum.alloc(MG));
+    HIP_TRY(d_cnt.alloc(2 * (size_t)M + 2 * (size_t)G));
+    HIP_TRY(hipMemcpyAsync(d_t.p, tstamps, sizeof(double) * R, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_m.p, model_ids, sizeof(int32_t) * R, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_slo.p, slos, sizeof(float) * R, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_m2g.p, m_id2g_id, sizeof(int32_t) * MG, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_max.p, group_max_latency, sizeof(float) * MG, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_sum.p, group_sum_latency, sizeof(float) * MG, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemsetAsync(d_cnt.p, 0, d_cnt.bytes(), st));
+    ScalarArgs a{};
+    a.tstamps = d_t.p;
+    a.model_ids = d_m.p;
+    a.slos = d_slo.p;
+    a.m_id2g_id = d_m2g.p;
+    a.group_max_latency = d_max.p;
+    a.group_sum_latency = d_sum.p;
+    a.R = num_requests;
+    a.M = M;
+    a.G = G;
+    a.fixed_overhead = fixed_overhead;
+    a.finish = d_fin.p;
+    a.good = d_good.p;
+    a.model_req = d_cnt.p;
+    a.model_good = d_cnt.p + M;
+    a.group_req = d_cnt.p + 2 * (size_t)M;
+    a.group_good = d_cnt.p + 2 * (size_t)M + G;
+    std::string err;
+    if (launch_sim_scalar(a, st, &err) != hipSuccess) return fail(MMSIM_E_HIP, err);
+    HIP_TRY(hipMemcpyAsync(finish, d_fin.p, sizeof(double) * R, hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipMemcpyAsync(good, d_good.p, R, hipMemcpyDeviceToHost, st));
+    std::vector<int32_t> cnt(2 * (size_t)M + 2 * (size_t)G);
+    HIP_TRY(hipMemcpyAsync(cnt.data(), d_cnt.p, d_cnt.bytes(), hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    std::memcpy(model_num_requests, cnt.data(), sizeof(int32_t) * (size_t)M);
+    std::memcpy(model_num_good_requests, cnt.data() + M, sizeof(int32_t) * (size_t)M);
+    std::memcpy(group_num_requests, cnt.data() + 2 * (size_t)M, sizeof(int32_t) * (size_t)G);
+    std::memcpy(group_num_good_requests, cnt.data() + 2 * (size_t)M + G, sizeof(int32_t) * (size_t)G);
+    return MMSIM_OK;
+}
+
 int mmsim_simulate_requests_mixed_batching(mmsim_ctx *ctx, double *finish, uint8_t *good, const double *tstamps,
                                            const int32_t *model_ids, const float *slos, const int32_t *m_id2g_id,
                                            const int32_t *g_id2m_id, const int32_t *num_stages,

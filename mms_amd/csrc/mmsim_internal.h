@@ -166,6 +166,24 @@ struct BatchingArgs {
     double *finish;              // [waves][Rmax][64]
     uint8_t *good;               // [waves][Rmax][64]
 };
+// Arguments of the scalar-clock request loop (one placement, device pointers).
+struct ScalarArgs {
+    const double *tstamps;            // [R]
+    const int32_t *model_ids;         // [R]
+    const float *slos;                // [R]
+    const int32_t *m_id2g_id;         // [M][G], -1 terminated rows
+    const float *group_max_latency;   // [M][G]
+    const float *group_sum_latency;   // [M][G]
+    int64_t R;
+    int32_t M, G;
+    double fixed_overhead;
+    double *finish;                   // [R]
+    uint8_t *good;                    // [R]
+    int32_t *model_req, *model_good;  // [M], zeroed by the caller
+    int32_t *group_req, *group_good;  // [G], zeroed by the caller
+};
+hipError_t launch_sim_scalar(const ScalarArgs &args, hipStream_t stream, std::string *err);
+
 hipError_t launch_sim_batching(const BatchingArgs &args, int waves_per_block, size_t lds_bytes, hipStream_t stream,
                                std::string *err);
 

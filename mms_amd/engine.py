@@ -289,6 +289,33 @@ def simulate_requests_mixed(engine: Engine, finish, good, tstamps, model_ids, sl
     return tuple(counts)
 
 
+def simulate_requests(engine: Engine, finish, good, tstamps, model_ids, slos, m_id2g_id,
+                      group_max_latency, group_sum_latency, num_requests=None,
+                      fixed_overhead: float = FIXED_OVERHEAD):
+    """Same call as the reference's scalar-clock kernel (controller.py:506-558):
+    fills ``finish``/``good`` in place and returns the four count arrays."""
+    ts = _lib.carray(tstamps, np.float64)
+    R = len(ts) if num_requests is None else int(num_requests)
+    mid = _lib.carray(model_ids, np.int32)
+    sl = _lib.carray(slos, np.float32)
+    m2g = _lib.carray(m_id2g_id, np.int32)
+    gmax = _lib.carray(group_max_latency, np.float32)
+    gsum = _lib.carray(group_sum_latency, np.float32)
+    M, G = m2g.shape
+    assert gmax.shape == (M, G) and gsum.shape == (M, G)
+    fin = np.empty(R, np.float64)
+    gd = np.empty(R, np.uint8)
+    counts = [np.zeros(M, np.int32), np.zeros(M, np.int32), np.zeros(G, np.int32), np.zeros(G, np.int32)]
+    _lib.check(engine.lib.mmsim_simulate_requests(
+        engine._h, _lib.ptr(fin, C.c_double), _lib.ptr(gd, C.c_uint8), _lib.ptr(ts, C.c_double),
+        _lib.ptr(mid, C.c_int32), _lib.ptr(sl, C.c_float), _lib.ptr(m2g, C.c_int32),
+        _lib.ptr(gmax, C.c_float), _lib.ptr(gsum, C.c_float), R, M, G, float(fixed_overhead),
+        *[_lib.ptr(c, C.c_int32) for c in counts]))
+    finish[:R] = fin
+    good[:R] = gd.astype(bool)
+    return tuple(counts)
+
+
 def simulate_requests_mixed_batching(engine: Engine, finish, good, tstamps, model_ids, slos, m_id2g_id,
                                      g_id2m_id, num_stages, stage_latency, batch_sizes,
                                      num_requests=None, fixed_overhead: float = FIXED_OVERHEAD):

@@ -82,10 +82,6 @@ def approximate_one_case_one_placement(placement, model_names, prof_ress, model_
     The stage-latency table follows :467-476 (and :451-461 with batching); the
     request loop runs on the GPU through the C ABI's single-placement calls.
     """
-    if not mixed:
-        raise NotImplementedError(
-            "the scalar-clock variant (mixed=False) is not reachable from any "
-            "public caller of the reference and is not built for the GPU")
     eng = _engine.Engine.default()
     group_configs = placement.group_configs
     num_groups = len(group_configs)
@@ -95,6 +91,25 @@ def approximate_one_case_one_placement(placement, model_names, prof_ress, model_
     arrivals = np.asarray(arrivals, dtype=np.float64)
     num_requests = len(arrivals)
     m_id2g_id = _placement_to_replica_table(placement, num_models)
+    if not mixed:
+        # one clock per group: largest and summed stage latency of every (model, group), with the
+        # pipeline penalty, rounded to float32 on assignment (:433-443, :496-499)
+        group_max_latency = np.empty((num_models, num_groups), dtype=np.float32)
+        group_sum_latency = np.empty((num_models, num_groups), dtype=np.float32)
+        for m_id in range(num_models):
+            for g_id in range(num_groups):
+                value = prof_ress[m_id].para_dict.get(group_configs[g_id], None)
+                if value:
+                    penalty = 0.009 * len(value.latency[1])
+                    group_max_latency[m_id][g_id] = max(value.latency[1]) * (1 + penalty)
+                    group_sum_latency[m_id][g_id] = sum(value.latency[1]) * (1 + penalty)
+                else:
+                    group_max_latency[m_id][g_id] = group_sum_latency[m_id][g_id] = np.inf
+        finish = np.empty(num_requests, dtype=np.float64)
+        good = np.empty(num_requests, dtype=bool)
+        counts = _engine.simulate_requests(eng, finish, good, arrivals, model_ids, slos, m_id2g_id,
+                                           group_max_latency, group_sum_latency, num_requests)
+        return (arrivals, finish, good) + tuple(counts)
     num_stages = np.array([c.pp for c in group_configs], dtype=np.int32)
     max_num_stages = int(np.max(num_stages))
     batch_sizes = list(batchsize_config) if enable_batching else [1]

@@ -61,6 +61,14 @@ def _simulate_requests_mixed(engine, finish, good, tstamps, model_ids, slos, m2g
     return cnt
 
 
+def _simulate_requests(engine, finish, good, tstamps, model_ids, slos, m2g, gmax, gsum,
+                       num_requests=None, fixed_overhead=0.011):
+    f, g, cnt = oracle_c.simulate_requests(tstamps, model_ids, slos, m2g, gmax, gsum, fixed_overhead)
+    finish[:] = f
+    good[:] = g
+    return cnt
+
+
 def _simulate_requests_mixed_batching(engine, finish, good, tstamps, model_ids, slos, m2g, g2m, num_stages,
                                       lat, batch_sizes, num_requests=None, fixed_overhead=0.011):
     f, g, cnt, _ = oracle_c.simulate_requests_mixed_batching(tstamps, model_ids, slos, m2g, g2m, num_stages,
@@ -76,4 +84,5 @@ def install(monkeypatch):
     monkeypatch.setattr(E, "DeviceWorkload", _HostWorkload)
     monkeypatch.setattr(E, "evaluate", _evaluate)
     monkeypatch.setattr(E, "simulate_requests_mixed", _simulate_requests_mixed)
+    monkeypatch.setattr(E, "simulate_requests", _simulate_requests)
     monkeypatch.setattr(E, "simulate_requests_mixed_batching", _simulate_requests_mixed_batching)

@@ -71,6 +71,34 @@ def _run_config(eng, cfg, sols, seeds, flags):
     return out, table, packed, streams, info
 
 
+def test_scalar_clock_variant_matches_oracle(eng):
+    """simulate_requests (alpa_serve/simulator/controller.py:506-558), the mixed=False loop: finish bits,
+    flags and all four count arrays against the oracle; closed form for a single group."""
+    F32 = np.float32
+    gsum, gmax = np.full((1, 1), 0.3, F32), np.full((1, 1), 0.1, F32)
+    R = 10
+    fin, good = np.empty(R), np.empty(R, bool)
+    E.simulate_requests(eng, fin, good, np.zeros(R), np.zeros(R, np.int32), np.full(R, np.inf, F32),
+                        np.zeros((1, 1), np.int32), gmax, gsum)
+    start, want = 0.0, []
+    for _ in range(R):                       # the next request may start 0.1 after the previous start
+        want.append(start + float(F32(0.3)) + 0.011)
+        start = start + float(F32(0.1))
+    assert fin.tolist() == want and good.all()
+    for seed in range(300):
+        c = random_case(5_000_000 + seed, max_m=6, max_g=5, max_s=4, max_r=300, load=1.0 + seed % 5)
+        gmax = c["lat"][..., 0].max(axis=2)
+        gsum = c["lat"][..., 0].sum(axis=2, dtype=np.float32)
+        f0, g0, c0 = oracle_c.simulate_requests(c["tstamps"], c["model_ids"], c["slos"], c["m2g"], gmax, gsum)
+        R = len(c["tstamps"])
+        fin, good = np.empty(R), np.empty(R, bool)
+        cnt = E.simulate_requests(eng, fin, good, c["tstamps"], c["model_ids"], c["slos"], c["m2g"], gmax, gsum)
+        assert np.array_equal(good, g0), seed
+        assert np.array_equal(fin.view(np.uint64), f0.view(np.uint64)), seed
+        for a, b in zip(cnt, c0):
+            assert np.array_equal(a, b), seed
+
+
 def test_config1_sanity_case(eng):
     cfg = make_config(1)
     out, table, packed, streams, _ = _run_config(eng, cfg, cfg.placements, [0], ALL)

@@ -277,6 +277,28 @@ def test_separations_solved_together_equal_separations_solved_one_by_one(backend
         sol.verify(mixed, cluster_env)
 
 
+def test_one_placement_with_scalar_group_clocks(backend):
+    """approximate_one_case_one_placement(mixed=False) (controller.py:433-443, :496-499): tables and loop of
+    the scalar-clock variant.  For single-stage groups it coincides with the default (mixed) simulation."""
+    from mms_amd.simulator.controller import approximate_one_case_one_placement
+    model_datas = four_models(0.4, 6, 3)
+    wl = gen_train_workload(model_datas, simulation_min_samples=2000)
+    names = [d.name for d in model_datas]
+    profs = [d.profiling_result for d in model_datas]
+    ids = np.array([names.index(r.model_name) for r in wl.requests], np.int32)
+    slos = np.array([r.slo for r in wl.requests], np.float32)
+    single = ModelPlacement([ParallelConfig(1, 1, 1)] * 3, [[0, 1], [1, 2, 3], [0, 3]])
+    a = approximate_one_case_one_placement(single, names, profs, ids, slos, wl.arrivals, mixed=False)
+    b = approximate_one_case_one_placement(single, names, profs, ids, slos, wl.arrivals, mixed=True)
+    for x, y in zip(a[1:], b[1:]):
+        assert np.array_equal(x, y)
+    deep = ModelPlacement([ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 2)], [[0, 1, 2], [1, 2, 3]])
+    start, finish, good, mreq, mgood, greq, ggood = approximate_one_case_one_placement(
+        deep, names, profs, ids, slos, wl.arrivals, mixed=False)
+    assert mreq.sum() == len(wl) and mgood.sum() == good.sum() == ggood.sum() and 0 < good.sum() < len(wl)
+    assert np.all(finish[~good] == start[~good]) and np.all(finish[good] - start[good] <= slos[good].astype(np.float64))
+
+
 def test_batching_evaluator(backend, monkeypatch):
     import mms_amd.util as U
     from mms_amd.profiling import synthetic_profile
