@@ -1,12 +1,18 @@
 // Batching request-loop simulation for gfx950.
 //
 // Restates the reference's simulate_requests_mixed_batching
-// (alpa_serve/simulator/controller.py:631-798) with one lane per
-// (placement, arrival seed) and the 64 lanes of a wavefront walking the same
+// (alpa_serve/simulator/controller.py:631-798) with one simulation per
+// (placement, arrival seed) and all simulations of a wavefront walking the same
 // request stream.  The outer loop over arrivals is in lockstep; what happens
 // between two arrivals (idle groups picking up queued requests, dropping
 // requests that can no longer meet their deadline, growing a batch) differs
-// per lane and runs as divergent per-lane loops.
+// per simulation and runs as divergent loops, so a wavefront pays for every
+// simulation's trips.  These loops are bound by latency and instruction issue,
+// not by lanes, and a simulation's state takes about 2 KB of LDS.  Hence narrow
+// tiles: a wavefront carries 64, 32, 16 or 8 simulations ("lanes" below),
+// whichever puts most wavefronts on a CU; with 8, each simulation is worked on
+// by an octet of lanes that hold the same state, take the same branches and
+// split the scans among them.
 //
 // State of a lane:
 //   * stage clocks clk[slot][lane] in LDS, as in the plain simulator; a
