@@ -3,7 +3,7 @@ import numpy as np
 
 
 def random_case(seed, max_m=4, max_g=3, max_s=3, max_r=50, nb=1, p_unknown=0.05,
-                p_inf_row=0.05, p_odd_slo=0.05, tie_prob=0.2, load=1.0, inf_slo=True):
+                p_inf_row=0.05, p_odd_slo=0.05, tie_prob=0.2, load=1.0, inf_slo=True, p_member=0.6):
     """Returns dict(tstamps, model_ids, slos, m2g, g2m, num_stages, lat[M][G][S][nb])."""
     rng = np.random.default_rng(seed)
     M = int(rng.integers(1, max_m + 1))
@@ -11,7 +11,7 @@ def random_case(seed, max_m=4, max_g=3, max_s=3, max_r=50, nb=1, p_unknown=0.05,
     num_stages = rng.integers(1, max_s + 1, size=G).astype(np.int32)
     S = int(num_stages.max())
     R = int(rng.integers(0, max_r + 1))
-    member = rng.random((G, M)) < 0.6
+    member = rng.random((G, M)) < p_member
     m2g = np.full((M, G), -1, np.int32)
     g2m = np.full((G, M), -1, np.int32)
     for m in range(M):

@@ -85,6 +85,26 @@ def test_every_kernel_variant(eng, monkeypatch, lanes, lds_tables):
             assert np.array_equal(a, b), (seed, nb)
 
 
+@pytest.mark.parametrize("lanes", [8, 16])
+def test_many_groups_many_pending_events(eng, monkeypatch, lanes):
+    """More than 64 groups busy at once: the idle events fill more than eight chunks of the event list, so
+    the scan of the chunk minima takes several rounds."""
+    monkeypatch.setenv("MMSIM_BATCHING_LANES", str(lanes))
+    for seed in (12, 19, 22, 44, 50, 70):      # 74 to 90 groups each, up to 23 replicas per model
+        c = random_case(6_000_000 + seed, max_m=40, max_g=90, max_s=2, max_r=1500, nb=3, load=60.0,
+                        inf_slo=False, tie_prob=0.1, p_member=0.15)
+        assert c["m2g"].shape[1] >= 70
+        bss = BSS[:3]
+        f0, g0, c0, max_heap = oracle_c.simulate_requests_mixed_batching(
+            c["tstamps"], c["model_ids"], c["slos"], c["m2g"], c["g2m"], c["num_stages"], c["lat"], bss)
+        assert max_heap > 64, max_heap
+        fin, good, cnt = _single(eng, c, bss)
+        assert np.array_equal(good, g0), seed
+        assert np.array_equal(fin.view(np.uint64), f0.view(np.uint64)), seed
+        for a, b in zip(cnt, c0):
+            assert np.array_equal(a, b), seed
+
+
 def test_groups_that_become_idle_at_the_same_instant(eng):
     """Idle events with equal times are popped in group order (the reference's heap holds (time, group)
     tuples, alpa_serve/simulator/controller.py:728-740).  Twelve identical one-stage groups all start a
