@@ -351,6 +351,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         };
         heap_min = (Gmax + 4 + 7) & ~7;
         heap_pref = std::max(heap_min, std::min(2 * Gmax + 8, Gmax + 16) & ~7);
+        // MMSIM_BATCHING_EVENT_SLOTS fixes the number of event slots per simulation (a multiple of eight; fewer than
+        // the simulation needs makes it stop with MMSIM_E_OVERFLOW: used to test that path)
+        if (const char *env = std::getenv("MMSIM_BATCHING_EVENT_SLOTS")) heap_pref = heap_min = std::max(8, std::atoi(env) & ~7);
         auto size_for = [&](int lanes) {
             for (heap_cap = heap_pref; heap_cap >= heap_min; heap_cap -= 8) {
                 wave_bytes = bytes_for(lanes, heap_cap);

@@ -105,6 +105,21 @@ def test_many_groups_many_pending_events(eng, monkeypatch, lanes):
             assert np.array_equal(a, b), seed
 
 
+@pytest.mark.parametrize("lanes", [8, 16])
+def test_a_simulation_that_runs_out_of_event_slots_is_reported(eng, monkeypatch, lanes):
+    """With fewer event slots than busy groups the simulation stops and the call fails with MMSIM_E_OVERFLOW
+    instead of returning numbers (the slots are provisioned from the group count; here they are forced down)."""
+    monkeypatch.setenv("MMSIM_BATCHING_LANES", str(lanes))
+    monkeypatch.setenv("MMSIM_BATCHING_EVENT_SLOTS", "8")
+    c = random_case(6_000_012, max_m=40, max_g=90, max_s=2, max_r=1500, nb=3, load=60.0,
+                    inf_slo=False, tie_prob=0.1, p_member=0.15)
+    with pytest.raises(_lib.MmsimError) as err:
+        _single(eng, c, BSS[:3])
+    assert err.value.code == _lib.E_OVERFLOW
+    monkeypatch.delenv("MMSIM_BATCHING_EVENT_SLOTS")
+    _single(eng, c, BSS[:3])                 # and the context is fine afterwards
+
+
 def test_groups_that_become_idle_at_the_same_instant(eng):
     """Idle events with equal times are popped in group order (the reference's heap holds (time, group)
     tuples, alpa_serve/simulator/controller.py:728-740).  Twelve identical one-stage groups all start a
