@@ -312,12 +312,13 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
     if (const char *env = std::getenv("MMSIM_WAVES_PER_CU")) wpb_cap = std::max(1, std::min(kMaxWavesPerBlock, std::atoi(env)));
     // plain simulator, per wavefront: request block | replica bounds | clocks (one extra row that stays +inf)
-    // | slot owners | group counters; the latency table is shared by the workgroup
+    // | slot owners | group counters | model counters; the latency table is shared by the workgroup
+    size_t model_lds_bytes = 0;  // per-model counters [M][64] in LDS (decided below)
     auto mixed_wave_bytes = [&](int ns) {
         return ((size_t)mixed_clock_offset(rmax_lds_bytes) + (size_t)(ns + 1) * kSlotBytes +
                 ((flags & MMSIM_WANT_GROUP_COUNTS)
                      ? (((size_t)ns * kWave + 15) & ~(size_t)15) + (size_t)2 * Gmax * kWave * sizeof(uint32_t)
-                     : 0) + 15) & ~(size_t)15;
+                     : 0) + model_lds_bytes + 15) & ~(size_t)15;
     };
     if (!batching) {
         wave_bytes = mixed_wave_bytes(nslots);  // of the largest placement
@@ -335,6 +336,18 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (lat_bytes + wave_bytes + lds_tail > (size_t)ctx->max_lds) {
             lds_tail = 0;
             pow2_depths = false;
+        }
+        // Per-model counters: one relaxed add to a global row per accepted (lane, request) costs a small
+        // batch (one wavefront per CU, nothing to hide behind) about 300 cycles per request, because later
+        // loads wait behind it; counters in LDS do not.  They take M * 256 bytes per wavefront, so they are
+        // used when that does not lower the wavefronts a CU gets.
+        if (flags & MMSIM_WANT_MODEL_COUNTS) {
+            const size_t room = (size_t)ctx->max_lds - lat_bytes - lds_tail, extra = (size_t)M * kWave * sizeof(uint32_t);
+            const size_t used_now = std::min<size_t>(wpb_cap, room / wave_bytes);
+            if (wave_bytes + extra <= room && std::min<size_t>(wpb_cap, room / (wave_bytes + extra)) >= used_now) {
+                model_lds_bytes = extra;
+                wave_bytes = mixed_wave_bytes(nslots);
+            }
         }
     } else {
         // per wavefront: descriptors | clocks | event times | chunk minima | queue heads | head ranks | event
@@ -810,6 +823,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.n_good = b->n_good.p;
     a.lat_sum = b->lat_sum.p;
     a.model_good = b->model_good.p;
+    a.model_lds = model_lds_bytes ? 1 : 0;
     a.group_req = b->group_req.p;
     a.group_good = b->group_good.p;
     a.finish = b->finish.p;

@@ -118,6 +118,8 @@ struct MixedArgs {
     uint8_t *good;               // [waves][Rmax][64]
     int64_t *fp_ops;             // [n_seeds][tiles*64]
     int32_t *error;              // set to 1 if the kernel finds its LDS layout assumption broken
+    int32_t model_lds;           // 1: per-model counters [M][64] live in LDS behind the group counters (small batches,
+                                 // where LDS is not what limits the wavefronts per CU); 0: relaxed adds to model_good
 };
 
 // LDS layout of the plain simulator, shared by the kernel and by the host code

@@ -200,6 +200,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const int own_bytes = want_group ? ((a.nslots * kWave + 15) & ~15) : 0;
     uint8_t *owner = lds_raw + clk_off + (a.nslots + 1) * kSlotBytes;  // owner[slot * 64 + lane]
     uint32_t *gcnt = reinterpret_cast<uint32_t *>(owner + own_bytes) + lane;
+    const bool model_lds = want_model && a.model_lds != 0;
+    uint32_t *mcnt = gcnt + (want_group ? 2 * a.Gmax * kWave : 0);  // [M][64] accepted requests per model
 
     for (int i = (int)threadIdx.x; i < lat_floats; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
     if (live)
@@ -240,11 +242,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         }
     }
 
+    int32_t *model_good = a.model_good + (size_t)wave * a.M * kWave + lane;
+    if (model_lds)
+        for (int m = 0; m < a.M; ++m) mcnt[m * kWave] = resume ? (uint32_t)model_good[(size_t)m * kWave] : 0u;
+
     const int4 *__restrict__ reqs4 = reinterpret_cast<const int4 *>(a.streams + off);
     const uint4 *__restrict__ rep_tile = a.rep32 + (size_t)tile * a.M * 2 * kWave + lane;
     const uint32_t *__restrict__ repx_tile = a.repx32 + (size_t)tile * a.M * a.rep_extra * kWave + lane;
     const float *lat_base = LATLDS ? lat_lds : a.lat;
-    int32_t *model_good = a.model_good + (size_t)wave * a.M * kWave + lane;
     double *fin_out = a.finish + (size_t)wave * a.Rmax * kWave + lane;
     uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + lane;
     const double overhead = a.fixed_overhead;
@@ -478,8 +483,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     }
                     if (has) fp_ops += 2 * (sm1 + 1) + nvalid + 3;
                 }
-                if (want_model && m >= 0 && acc)  // one owner per counter: a relaxed add that nobody waits for
+                if (model_lds) {  // an LDS add that returns nothing
+                    if (m >= 0)
+                        __hip_atomic_fetch_add(&mcnt[m * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+                } else if (want_model && m >= 0 && acc) {  // one owner per counter: a relaxed add that nobody waits for
                     __hip_atomic_fetch_add(&model_good[(size_t)m * kWave], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
                 if (want_req) {
                     fin_out[(blk + cb + u) * kWave] = acc ? finish_time : tstamp;
                     good_out[(blk + cb + u) * kWave] = acc ? 1 : 0;
@@ -495,6 +504,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     if (want_ops) a.fp_ops[out] = fp_ops;
     if (a.seg < a.nseg - 1)
         for (int s = 0; s < a.nslots; ++s) saved[(size_t)s * kWave] = clk[s * kWave];
+    if (model_lds)
+        for (int m = 0; m < a.M; ++m) model_good[(size_t)m * kWave] = (int32_t)mcnt[m * kWave];
     if (want_group) {
         for (int g = 0; g < a.Gmax; ++g) {
             greq[g * kWave] = (int32_t)gcnt[g * kWave];
