@@ -163,10 +163,11 @@ __device__ __forceinline__ uint32_t pick_desc(const uint4 &a, const uint4 &b) {
 }
 
 // SMAX: most stages of a group (bucket).  LATLDS: the latency table is kept in LDS.  UNIFORM: one
-// latency per (model, configuration).  POW2: every group has 1, 2, 4, 8 or 16 stages.  STATS: some
-// output beyond goodput and latency sum is wanted (a.flags says which); without it the per-request
-// path carries no trace of them.
-template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, bool STATS>
+// latency per (model, configuration).  POW2: every group has 1, 2, 4, 8 or 16 stages.  OUT: what the
+// request loop produces beyond goodput and latency sum (a.flags says which of it): 0 nothing, 1
+// per-model / per-group counts, 2 also per-request results and operation counts; a level's loop
+// carries no trace of the higher levels' outputs.
+template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(const MixedArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     constexpr int CH = ChunkFor<SMAX>::value;
@@ -178,10 +179,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const int seed = (int)(blockIdx.x % (unsigned)a.n_seeds);
     const int tile = a.tile0 + (int)(blockIdx.x / (unsigned)a.n_seeds) * W + wv;
     const bool live = tile < a.tile1;
+    constexpr bool STATS = OUT > 0;
     const bool want_model = STATS && (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
     const bool want_group = STATS && (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
-    const bool want_req = STATS && (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
-    const bool want_ops = STATS && (a.flags & MMSIM_WANT_OP_COUNT) != 0;
+    const bool want_req = OUT == 2 && (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
+    const bool want_ops = OUT == 2 && (a.flags & MMSIM_WANT_OP_COUNT) != 0;
     constexpr bool pow2 = POW2;
 
     // ---- LDS: [latency table][per wavefront: request block | replica bounds | clocks (+inf row last) |
@@ -514,9 +516,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     }
 }
 
-template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, bool STATS>
+template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT>
 hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
-    auto kern = sim_mixed_kernel<SMAX, LATLDS, UNIFORM, POW2, STATS>;
+    auto kern = sim_mixed_kernel<SMAX, LATLDS, UNIFORM, POW2, OUT>;
     if (lds_bytes > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -532,15 +534,19 @@ hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStrea
 // table in global memory only the general kernels exist.
 template <int SMAX, bool UNIFORM>
 hipError_t launch_u(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
-    const bool stats = (args.flags & (MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS | MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT)) != 0;
-    if (!args.lat_in_lds) return launch_one<SMAX, false, UNIFORM, false, true>(args, wpb, lds_bytes, stream);
+    // what the request loop has to produce: 0 scores only, 1 also per-model / per-group counts, 2 anything
+    const int out = (args.flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT)) ? 2
+                    : (args.flags & (MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) ? 1 : 0;
+    if (!args.lat_in_lds) return launch_one<SMAX, false, UNIFORM, false, 2>(args, wpb, lds_bytes, stream);
     if constexpr (SMAX == 4 || SMAX == 16) {  // the stage buckets with a hand-scheduled walk
         if (args.pow2_depths)
-            return stats ? launch_one<SMAX, true, UNIFORM, true, true>(args, wpb, lds_bytes, stream)
-                         : launch_one<SMAX, true, UNIFORM, true, false>(args, wpb, lds_bytes, stream);
+            return out == 2   ? launch_one<SMAX, true, UNIFORM, true, 2>(args, wpb, lds_bytes, stream)
+                   : out == 1 ? launch_one<SMAX, true, UNIFORM, true, 1>(args, wpb, lds_bytes, stream)
+                              : launch_one<SMAX, true, UNIFORM, true, 0>(args, wpb, lds_bytes, stream);
     }
-    return stats ? launch_one<SMAX, true, UNIFORM, false, true>(args, wpb, lds_bytes, stream)
-                 : launch_one<SMAX, true, UNIFORM, false, false>(args, wpb, lds_bytes, stream);
+    return out == 2   ? launch_one<SMAX, true, UNIFORM, false, 2>(args, wpb, lds_bytes, stream)
+           : out == 1 ? launch_one<SMAX, true, UNIFORM, false, 1>(args, wpb, lds_bytes, stream)
+                      : launch_one<SMAX, true, UNIFORM, false, 0>(args, wpb, lds_bytes, stream);
 }
 
 template <int SMAX>
