@@ -56,8 +56,14 @@
 // Workgroup = up to 4 wavefronts that share only the read-only latency
 // table; after the single barrier that publishes it, wavefronts run
 // independently (lanes never exchange data).
-// blockIdx.x = tile_group * n_seeds + seed: with n_seeds a multiple of 8 all
-// wavefronts that read one stream sit on one XCD and share its L2.
+// Workgroups go to the eight XCDs round-robin by blockIdx.x, and each XCD has
+// its own L2.  A request costs a wavefront 16 bytes of its stream but 2 KiB of
+// its tile's descriptor rows, so the mapping keeps the descriptors together:
+// blockIdx.x = ((tile_group / 8) * n_seeds + seed) * 8 + tile_group % 8, i.e.
+// all seeds of a tile group run on one XCD and an XCD sees one eighth of the
+// descriptor tables (a.xcd_map; the grid is padded to whole rounds of eight
+// tile groups, the padding workgroups leave at once).  With a.xcd_map == 0
+// blockIdx.x = tile_group * n_seeds + seed.
 
 #include "mmsim_internal.h"
 #include "walk_asm.inc"
@@ -176,8 +182,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const int W = (int)(blockDim.x >> 6);
     const int wv = uniform((int)(threadIdx.x >> 6));
     const int lane = (int)(threadIdx.x & 63);
-    const int seed = (int)(blockIdx.x % (unsigned)a.n_seeds);
-    const int tile = a.tile0 + (int)(blockIdx.x / (unsigned)a.n_seeds) * W + wv;
+    const unsigned bq = a.xcd_map ? blockIdx.x >> 3 : blockIdx.x;
+    const int seed = (int)(bq % (unsigned)a.n_seeds);
+    const int tgroup = a.xcd_map ? (int)(bq / (unsigned)a.n_seeds) * 8 + (int)(blockIdx.x & 7u) : (int)(bq / (unsigned)a.n_seeds);
+    const int tile = a.tile0 + tgroup * W + wv;
     const bool live = tile < a.tile1;
     constexpr bool STATS = OUT > 0;
     const bool want_model = STATS && (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
@@ -525,7 +533,7 @@ hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStrea
         if (e != hipSuccess) return e;
     }
     const unsigned tile_groups = (unsigned)((args.tile1 - args.tile0 + wpb - 1) / wpb);
-    const dim3 grid(tile_groups * (unsigned)args.n_seeds);
+    const dim3 grid((args.xcd_map ? ((tile_groups + 7u) & ~7u) : tile_groups) * (unsigned)args.n_seeds);
     hipLaunchKernelGGL(kern, grid, dim3(wpb * kWave), lds_bytes, stream, args);
     return hipGetLastError();
 }
