@@ -264,6 +264,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + lane;
     const double overhead = a.fixed_overhead;
 
+    // the group chosen for the last request, kept while it stays valid (see the request loop)
+    int ch_model = -2;        // wave-uniform: model the choice was made for
+    bool ch_stale = true;     // wave-uniform: some lane accepted a request since
+    double ch_best = __builtin_inf(), ch_l_last = 0.0;
+    uint32_t ch_sel = kEmpty;
+
     int4 ahead = make_int4(0, 0, -1, 0);  // this lane's request of the next block
     if (R > 0) ahead = reqs4[r0 + lane < R ? r0 + lane : R - 1];
 
@@ -335,8 +341,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     const bool right = y.c < x.c;
                     return Cand{vmin(x.c, y.c), right ? y.d : x.d, right ? y.l : x.l};
                 };
-                Cand win{__builtin_inf(), kEmpty, 0.0f};
-                auto scan = [&](auto NJ) {
+                auto scan = [&](Cand &win, auto NJ) {
                     constexpr int nj = decltype(NJ)::value;
                     Cand k[nj];
                     static_while<0, nj>([&](auto J) {
@@ -353,28 +358,38 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                         win = first_min(win, first_min(a45, a67));
                     }
                 };
-                if (n > 4)
-                    scan(Idx<8>{});
-                else if (n > 0)
-                    scan(Idx<4>{});
-                if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
-                    const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
-                    for (int j = RREG; j < n; ++j) {
-                        const uint32_t d = row[(size_t)(j - RREG) * kWave];
-                        win = first_min(win, Cand{lds_f64(rep_addr(d)), d, lrow_m[rep_lat_last(d)]});
+                // Clocks change only when a request is accepted, so while no lane of the wavefront has
+                // accepted anything since the last scan, a request for the same model finds the same group
+                // in every lane: the choice is kept from request to request (bursts make most requests
+                // repeat the model of the one before, and most of a burst is rejected).
+                if (m != ch_model || ch_stale) {
+                    Cand win{__builtin_inf(), kEmpty, 0.0f};
+                    if (n > 4)
+                        scan(win, Idx<8>{});
+                    else if (n > 0)
+                        scan(win, Idx<4>{});
+                    if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
+                        const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
+                        for (int j = RREG; j < n; ++j) {
+                            const uint32_t d = row[(size_t)(j - RREG) * kWave];
+                            win = first_min(win, Cand{lds_f64(rep_addr(d)), d, lrow_m[rep_lat_last(d)]});
+                        }
                     }
+                    // a clock that is infinite (a group that served a request with infinite latency) is never
+                    // chosen (:590-598: "tmp < min_device_clock" with min_device_clock starting at inf)
+                    ch_model = m;
+                    ch_best = win.c;
+                    ch_sel = win.c < 1e100 ? win.d : kEmpty;
+                    ch_l_last = (double)win.l;
                 }
-                // a clock that is infinite (a group that served a request with infinite latency) is never
-                // chosen (:590-598: "tmp < min_device_clock" with min_device_clock starting at inf)
-                const double best = win.c;
-                const uint32_t sel = best < 1e100 ? win.d : kEmpty;
-                const float lsel = win.l;
+                const double best = ch_best;
+                const uint32_t sel = ch_sel;
                 const bool has = (int32_t)sel >= 0;
                 const int sm1 = has ? (int)rep_stages_m1(sel) : -1;  // stages - 1
                 const uint32_t last_addr = rep_addr(sel);            // the lane's +inf clock when there is no replica
                 const uint32_t first_addr = last_addr - (uint32_t)(has ? sm1 : 0) * kSlotBytes;
                 const float *lrow = lrow_m + (has ? (int)rep_lat_last(sel) - sm1 : 0);
-                const double l_last = (double)lsel;
+                const double l_last = ch_l_last;
 
                 double finish_time;
                 bool acc;
@@ -472,6 +487,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                             });
                     }
                 }
+                ch_stale = __ballot(acc) != 0ull;
                 if (want_group && has) {  // :611, :618
                     const uint32_t g = owner[(last_addr - clk_off) >> 3];  // (slot * 512 + lane * 8) / 8
                     // LDS adds that return nothing: the wavefront does not wait for them
