@@ -825,6 +825,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.model_good = b->model_good.p;
     a.model_lds = model_lds_bytes ? 1 : 0;
     a.xcd_map = 1;
+    a.skip_ahead = 1;
+    if (const char *env = std::getenv("MMSIM_SKIP_AHEAD")) a.skip_ahead = std::atoi(env) ? 1 : 0;  // tuning knob
     if (const char *env = std::getenv("MMSIM_XCD_MAP")) a.xcd_map = std::atoi(env) ? 1 : 0;  // tuning knob
     a.group_req = b->group_req.p;
     a.group_good = b->group_good.p;

@@ -279,6 +279,68 @@ def test_scores_only_mode_equals_full_mode(eng):
     assert np.array_equal(a["latency_sum"], b["latency_sum"])
 
 
+@pytest.mark.parametrize("n_placements", [200, 640])
+def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placements):
+    """A scores-only run keeps the chosen group from request to request while no lane accepts, and does
+    not simulate requests that every lane of a wavefront must reject.  Configuration 4's bursts (nine in
+    ten requests repeat the model of the one before) exercise both: goodput and latency sums equal the
+    oracle's bit for bit, in full and ragged tiles, with the skipping and without it."""
+    cfg = make_config(4, n_placements)
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(cfg.placements, table)
+    st = cfg.stream(0)
+    assert np.mean(st.model_ids[1:] == st.model_ids[:-1]) > 0.8
+    ref = oracle_batch(st, table, packed)
+    dw = E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models)
+    for skip in ("1", "0"):
+        monkeypatch.setenv("MMSIM_SKIP_AHEAD", skip)
+        batch = E.Batch(eng, [dw], table, packed, 0)
+        batch.run()
+        batch.sync()
+        out = batch.fetch()
+        batch.close()
+        assert np.array_equal(out["n_good"][0], ref["n_good"]), f"n_good differs (skip {skip})"
+        assert np.array_equal(out["latency_sum"][0], ref["latency_sum"]), f"latency_sum differs (skip {skip})"
+    dw.close()
+
+
+def test_scores_only_on_runs_of_one_model_with_odd_requests(eng):
+    """Runs of equal models with tied arrival times, SLOs that change inside a run (also inf and NaN),
+    unknown models, streams that end inside a block of 64, several seeds: scores-only results equal the
+    oracle's for every placement of configuration 2."""
+    cfg = make_config(2)
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(cfg.placements, table)
+    base_slo = np.asarray(cfg.slos, np.float32)
+    M = cfg.num_models
+    streams = []
+    for seed, R in enumerate([1, 63, 64, 65, 5000, 20011]):
+        rng = np.random.default_rng(100 + seed)
+        runs = rng.geometric(0.12, size=R)
+        models = np.repeat(rng.integers(0, M, size=R), runs)[:R].astype(np.int32)
+        models[rng.random(R) < 0.02] = -1
+        gaps = rng.exponential(0.004, size=R)
+        gaps[rng.random(R) < 0.25] = 0.0
+        gaps[rng.random(R) < 0.01] += 2.0                      # pauses that let the queues drain
+        ts = np.cumsum(gaps)
+        slos = base_slo[np.maximum(models, 0)] * rng.choice([1.0, 1.0, 1.0, 0.5, 3.0], size=R).astype(np.float32)
+        slos[rng.random(R) < 0.01] = np.inf
+        slos[rng.random(R) < 0.01] = np.nan
+        streams.append((ts, models, slos.astype(np.float32)))
+    dws = [E.DeviceWorkload(eng, t, m, s, M) for t, m, s in streams]
+    batch = E.Batch(eng, dws, table, packed, 0)
+    batch.run()
+    batch.sync()
+    out = batch.fetch()
+    batch.close()
+    from mms_amd.synthetic import Stream
+    for k, (t, m, s) in enumerate(streams):
+        ref = oracle_batch(Stream(t, m, s), table, packed)
+        assert np.array_equal(out["n_good"][k], ref["n_good"]), f"n_good differs, stream {k}"
+        assert np.array_equal(out["latency_sum"][k], ref["latency_sum"]), f"latency_sum differs, stream {k}"
+        assert 0 < ref["n_good"].sum() < len(t) * len(cfg.placements) or len(t) < 64
+
+
 def test_rerunning_a_batch_gives_the_same_answer(eng):
     cfg = make_config(2)
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
