@@ -92,8 +92,8 @@ __device__ __forceinline__ double vmin(double x, double y) {
 // 16 lanes (DPP), then the four row results through scalar registers.  All lanes must be active.
 template <int CTRL>
 __device__ __forceinline__ double dpp_f64(double x) {
-    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(x), CTRL, 0xF, 0xF, false);
-    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(x), CTRL, 0xF, 0xF, false);
+    const int lo = __builtin_amdgcn_update_dpp(__double2loint(x), __double2loint(x), CTRL, 0xF, 0xF, false);
+    const int hi = __builtin_amdgcn_update_dpp(__double2hiint(x), __double2hiint(x), CTRL, 0xF, 0xF, false);
     return __hiloint2double(hi, lo);
 }
 __device__ __forceinline__ double lane_f64(double x, int l) {
@@ -415,7 +415,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             } else {
                 // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
                 const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
-                const int walk = (has && !(bound > slo)) ? sm1 : -1;  // stages - 1 of lanes that walk
+                const int walk = (int)(has & !(bound > slo)) != 0 ? sm1 : -1;  // stages - 1 of lanes that walk (no per-lane branch)
                 if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
                     // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
                     uint64_t saved_exec, mask1, mask2, mask4, mask8;  // masks: scratch of the power-of-two walk
