@@ -80,6 +80,7 @@ struct mmsim_workload {
     int32_t M = 0;
     DevBuf<Req> reqs;
     std::vector<int32_t> model_num_requests;  // requests per model id (placement independent)
+    int64_t repeats = 0;                      // requests with the model of the request before
     // arrivals regrouped by model (batching simulator): offsets per model, then per arrival
     // its time, its deadline time + (double)slo and its index in the stream
     std::vector<int64_t> mq_off;
@@ -825,6 +826,15 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.model_good = b->model_good.p;
     a.model_lds = model_lds_bytes ? 1 : 0;
     a.xcd_map = 1;
+    {   // bursty streams (most requests repeat the model of the one before) get the loop over runs
+        int64_t rep = 0, tot = 0;
+        for (int s = 0; s < n_seeds; ++s) {
+            rep += wls[s]->repeats;
+            tot += wls[s]->R;
+        }
+        a.runs = 5 * rep > 4 * tot ? 1 : 0;  // four in five (measured: at three in four the chunked loop is still ahead)
+        if (const char *env = std::getenv("MMSIM_RUNS")) a.runs = std::atoi(env) ? 1 : 0;  // tuning knob
+    }
     a.skip_ahead = 1;
     if (const char *env = std::getenv("MMSIM_SKIP_AHEAD")) a.skip_ahead = std::atoi(env) ? 1 : 0;  // tuning knob
     if (const char *env = std::getenv("MMSIM_XCD_MAP")) a.xcd_map = std::atoi(env) ? 1 : 0;  // tuning knob
@@ -964,6 +974,7 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
         host[i].m = model_ids[i] < 0 ? -1 : model_ids[i];
         host[i].slo = slos[i];
         if (model_ids[i] >= 0) w->model_num_requests[model_ids[i]] += 1;
+        if (i > 0 && host[i].m == host[i - 1].m) w->repeats += 1;
     }
     w->mq_off.assign((size_t)M + 1, 0);
     for (int32_t m = 0; m < M; ++m) w->mq_off[m + 1] = w->mq_off[m] + w->model_num_requests[m];

@@ -157,6 +157,19 @@ __device__ __forceinline__ void walk_blocks(C &&c, B &&b) {
     }
 }
 
+// Chunked request loop (streams whose requests rarely repeat the model of the one before): requests whose
+// descriptors and fields are fetched ahead together.  The fetch of a chunk has the time the previous
+// chunk takes to arrive; four requests cover the latency of the descriptor loads.
+constexpr int kChunk = 4;
+struct Chunk {
+    int m[kChunk];        // wave-uniform model id (or -1)
+    int nrep[kChunk];     // wave-uniform replica bound of the tile for that model
+    double t[kChunk];     // arrival time (same in every lane)
+    float slo[kChunk];    // SLO (same in every lane)
+    uint4 da[kChunk];     // per-lane descriptors of replicas 0..3
+    uint4 db[kChunk];     // per-lane descriptors of replicas 4..7
+};
+
 template <int J>
 __device__ __forceinline__ uint32_t pick_desc(const uint4 &a, const uint4 &b) {
     if constexpr (J == 0) return a.x;
@@ -173,8 +186,9 @@ __device__ __forceinline__ uint32_t pick_desc(const uint4 &a, const uint4 &b) {
 // latency per (model, configuration).  POW2: every group has 1, 2, 4, 8 or 16 stages.  OUT: what the
 // request loop produces beyond goodput and latency sum (a.flags says which of it): 0 nothing, 1
 // per-model / per-group counts, 2 also per-request results and operation counts; a level's loop
-// carries no trace of the higher levels' outputs.
-template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT>
+// carries no trace of the higher levels' outputs.  RUNS: the loop walks runs of equal models (bursty
+// streams) instead of fixed chunks of four requests.
+template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT, bool RUNS>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(const MixedArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     constexpr int RREG = kPackedReplicas;
@@ -268,294 +282,359 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     bool ch_stale = true;     // wave-uniform: some lane accepted a request since
     double ch_best = __builtin_inf(), ch_l_last = 0.0;
     uint32_t ch_sel = kEmpty;
-    constexpr bool SKIP = OUT == 0;
+    constexpr bool SKIP = RUNS && OUT == 0;
     bool ch_looked = false;   // wave-uniform: the block has been searched for requests that the current choice rejects
     uint64_t skip = 0;        // wave-uniform: requests of the block that every lane rejects while nobody accepts
+
+    // One request for the whole wavefront: `at` is its place in the stream, m / n the model and the tile's
+    // replica bound for it (wave-uniform), da / db this lane's descriptors of the model's replicas.
+    auto simulate = [&](int64_t at, int m, int n, const uint4 &da, const uint4 &db, double tstamp, double slo) {
+        const float *lrow_m = lat_base + (size_t)(m < 0 ? 0 : m) * a.lat_row;
+
+        // ---- choose the replica group: strictly smallest last-stage clock (:590-598).
+        //      One LDS round trip fetches, for every listed replica, the clock of its last
+        //      stage and the latency of its last stage (needed by the early-reject bound).
+        // Strictly smallest clock, first listed wins ties: a tournament whose left side wins ties
+        // picks the same entry as the reference's left-to-right scan, in log2 dependent steps.
+        // Entries past a lane's own replicas are empty descriptors, whose clock reads +inf.
+        struct Cand {
+            double c;
+            uint32_t d;
+            float l;
+        };
+        auto first_min = [](const Cand &x, const Cand &y) {
+            const bool right = y.c < x.c;
+            return Cand{vmin(x.c, y.c), right ? y.d : x.d, right ? y.l : x.l};
+        };
+        auto scan = [&](Cand &win, auto NJ) {
+            constexpr int nj = decltype(NJ)::value;
+            Cand k[nj];
+            static_while<0, nj>([&](auto J) {
+                constexpr int j = decltype(J)::value;
+                k[j].d = pick_desc<j>(da, db);
+                k[j].c = lds_f64(rep_addr(k[j].d));
+                k[j].l = lrow_m[rep_lat_last(k[j].d)];
+                return true;
+            });
+            const Cand a01 = first_min(k[0], k[1]), a23 = first_min(k[2], k[3]);
+            win = first_min(a01, a23);
+            if constexpr (nj == 8) {
+                const Cand a45 = first_min(k[4], k[5]), a67 = first_min(k[6], k[7]);
+                win = first_min(win, first_min(a45, a67));
+            }
+        };
+        // Clocks change only when a request is accepted, so while no lane of the wavefront has
+        // accepted anything since the last scan, a request for the same model finds the same group
+        // in every lane: the choice is kept from request to request (bursts make most requests
+        // repeat the model of the one before, and most of a burst is rejected).
+        if (!RUNS || m != ch_model || ch_stale) {  // the chunked loop always scans
+            Cand win{__builtin_inf(), kEmpty, 0.0f};
+            if (n > 4)
+                scan(win, Idx<8>{});
+            else if (n > 0)
+                scan(win, Idx<4>{});
+            if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
+                const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
+                for (int j = RREG; j < n; ++j) {
+                    const uint32_t d = row[(size_t)(j - RREG) * kWave];
+                    win = first_min(win, Cand{lds_f64(rep_addr(d)), d, lrow_m[rep_lat_last(d)]});
+                }
+            }
+            // a clock that is infinite (a group that served a request with infinite latency) is never
+            // chosen (:590-598: "tmp < min_device_clock" with min_device_clock starting at inf)
+            ch_model = m;
+            ch_looked = false;
+            ch_best = win.c;
+            ch_sel = win.c < 1e100 ? win.d : kEmpty;
+            ch_l_last = (double)win.l;
+        }
+        const double best = ch_best;
+        const uint32_t sel = ch_sel;
+        const bool has = (int32_t)sel >= 0;
+        const int sm1 = has ? (int)rep_stages_m1(sel) : -1;  // stages - 1
+        const uint32_t last_addr = rep_addr(sel);            // the lane's +inf clock when there is no replica
+        const uint32_t first_addr = last_addr - (uint32_t)(has ? sm1 : 0) * kSlotBytes;
+        const float *lrow = lrow_m + (has ? (int)rep_lat_last(sel) - sm1 : 0);
+        const double l_last = ch_l_last;
+
+        double finish_time;
+        bool acc;
+        if constexpr (SMAX == 1) {
+            // ---- single-stage groups: the clock read for the choice is the whole pipeline (:605-619)
+            const double t = vmax(tstamp, best) + l_last;
+            finish_time = t + overhead;
+            const double latency = finish_time - tstamp;
+            acc = has && latency <= slo;
+            if (acc) {
+                lds_set_f64(last_addr, t);
+                n_good += 1;
+                lat_sum += latency;
+            }
+        } else {
+            // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
+            const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
+            const int walk = (int)(has & !(bound > slo)) != 0 ? sm1 : -1;  // stages - 1 of lanes that walk (no per-lane branch)
+            if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
+                // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
+                uint64_t saved_exec, mask1, mask2, mask4, mask8;  // masks: scratch of the power-of-two walk
+                int accepted;
+                double latency;
+                const uint32_t cb_addr = first_addr;
+#define MMSIM_WALK(NAME, LATNAME, LATVAL)                                                                           \
+asm volatile(NAME##_TEXT                                                                                        \
+     : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [fin] "=&v"(finish_time), [lat] "=&v"(latency),   \
+       [ng] "+v"(n_good), [ls] "+v"(lat_sum), [m1] "=&s"(mask1), [m2] "=&s"(mask2), [m4] "=&s"(mask4),  \
+       [m8] "=&s"(mask8)                                                                                \
+     : [walk] "v"(walk), [cb] "v"(cb_addr), [LATNAME] "v"(LATVAL), [ts] "v"(tstamp), [slo] "v"(slo),    \
+       [oh] "s"(overhead)                                                                               \
+     : "vcc", "scc", "memory", NAME##_CLOBBERS)
+                if constexpr (UNIFORM) {
+                    if (pow2) {
+                        if constexpr (SMAX == 4)
+                            MMSIM_WALK(MMSIM_WALK_PU4, lc, l_last);
+                        else
+                            MMSIM_WALK(MMSIM_WALK_PU16, lc, l_last);
+                    } else {
+                        if constexpr (SMAX == 4)
+                            MMSIM_WALK(MMSIM_WALK_U4, lc, l_last);
+                        else
+                            MMSIM_WALK(MMSIM_WALK_U16, lc, l_last);
+                    }
+                } else {
+                    const uint32_t lb = lds_addr(lrow);
+                    if (pow2) {
+                        if constexpr (SMAX == 4)
+                            MMSIM_WALK(MMSIM_WALK_PN4, lb, lb);
+                        else
+                            MMSIM_WALK(MMSIM_WALK_PN16, lb, lb);
+                    } else {
+                        if constexpr (SMAX == 4)
+                            MMSIM_WALK(MMSIM_WALK_N4, lb, lb);
+                        else
+                            MMSIM_WALK(MMSIM_WALK_N16, lb, lb);
+                    }
+                }
+#undef MMSIM_WALK
+                acc = accepted != 0;
+            } else {
+                // ---- the same in plain C++ (other stage buckets, latency table in global memory):
+                //      fetch, then the dependent chain (:605-608)
+                double *gclk = reinterpret_cast<double *>(lds_raw + first_addr);
+                double cv[SMAX];
+                float lv[SMAX];
+                walk_blocks<0, 1, SMAX>(
+                    [&](auto K) { return decltype(K)::value <= walk; },
+                    [&](auto K) {
+                        constexpr int k = decltype(K)::value;
+                        cv[k] = gclk[k * kWave];
+                        if (!UNIFORM) lv[k] = lrow[k];
+                    });
+                double t = tstamp;
+                walk_blocks<0, 1, SMAX>(
+                    [&](auto K) { return decltype(K)::value <= walk; },
+                    [&](auto K) {
+                        constexpr int k = decltype(K)::value;
+                        t = vmax(t, cv[k]) + (UNIFORM ? l_last : (double)lv[k]);
+                        cv[k] = t;
+                    });
+                finish_time = t + overhead;  // :610
+                const double latency = finish_time - tstamp;
+                acc = walk >= 0 && latency <= slo;  // :613
+                if (acc) {  // :614-619
+                    n_good += 1;
+                    lat_sum += latency;
+                }
+                const int commit = acc ? walk : -1;
+                walk_blocks<0, 1, SMAX>(
+                    [&](auto K) { return decltype(K)::value <= commit; },
+                    [&](auto K) {
+                        constexpr int k = decltype(K)::value;
+                        gclk[k * kWave] = cv[k];
+                    });
+            }
+        }
+        if constexpr (RUNS) {
+            ch_stale = __ballot(acc) != 0ull;
+            if (ch_stale) skip = 0;
+        }
+        if (want_group && has) {  // :611, :618
+            const uint32_t g = owner[(last_addr - clk_off) >> 3];  // (slot * 512 + lane * 8) / 8
+            // LDS adds that return nothing: the wavefront does not wait for them
+            __hip_atomic_fetch_add(&gcnt[g * kWave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            __hip_atomic_fetch_add(&gcnt[(a.Gmax + g) * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WAVEFRONT);
+        }
+        if (want_ops) {
+            asm volatile("" ::: "memory");  // keep this a wave-uniform branch, off the common path
+            int nvalid = 0;
+            static_while<0, RREG>([&](auto J) {
+                constexpr int j = decltype(J)::value;
+                nvalid += (j < n && (int32_t)pick_desc<j>(da, db) >= 0) ? 1 : 0;
+                return true;
+            });
+            if (n > RREG) {
+                const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
+                for (int j = RREG; j < n; ++j) nvalid += (int32_t)row[(size_t)(j - RREG) * kWave] >= 0 ? 1 : 0;
+            }
+            if (has) fp_ops += 2 * (sm1 + 1) + nvalid + 3;
+        }
+        if (model_lds) {  // an LDS add that returns nothing
+            if (m >= 0)
+                __hip_atomic_fetch_add(&mcnt[m * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        } else if (want_model && m >= 0 && acc) {  // one owner per counter: a relaxed add that nobody waits for
+            __hip_atomic_fetch_add(&model_good[(size_t)m * kWave], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (want_req) {
+            fin_out[at * kWave] = acc ? finish_time : tstamp;
+            good_out[at * kWave] = acc ? 1 : 0;
+        }
+    };
 
     int4 ahead = make_int4(0, 0, -1, 0);  // this lane's request of the next block
     if (R > 0) ahead = reqs4[r0 + lane < R ? r0 + lane : R - 1];
 
-    // Descriptors of the run about to start (fetched while the run before it is simulated).
-    uint4 nda = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty), ndb = nda;
-    auto fetch_run = [&](int model) {  // model < 0: any row will do, nothing is simulated
-        const uint4 *row = rep_tile + (size_t)(model < 0 ? 0 : model) * (2 * kWave);
-        nda = row[0];
-        ndb = row[kWave];
-    };
-    {
-        const int z0 = __builtin_amdgcn_readlane(ahead.z, 0);
-        fetch_run(r0 < r1 ? z0 : -1);
-    }
-
-    for (int64_t blk = r0; blk < r1; blk += kWave) {
-        // Lane j holds request j of the block; the request being simulated is read out of these
-        // registers with v_readlane.  The model word also carries the tile's replica bound.
-        const int nblk = (int)(r1 - blk < kWave ? r1 - blk : kWave);  // requests in this block
-        int4 r = ahead;
+    if constexpr (RUNS) {
+        // Descriptors of the run about to start (fetched while the run before it is simulated).
+        uint4 nda = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty), ndb = nda;
+        auto fetch_run = [&](int model) {  // model < 0: any row will do, nothing is simulated
+            const uint4 *row = rep_tile + (size_t)(model < 0 ? 0 : model) * (2 * kWave);
+            nda = row[0];
+            ndb = row[kWave];
+        };
         {
-            const bool ok = lane < nblk && r.z >= 0;
-            const int bound = (int)rmax_lds[ok ? r.z : 0];
-            r.z = ok ? (r.z | (bound << 24)) : -1;
-        }
-        {
-            const int64_t nx = blk + kWave + lane;
-            ahead = reqs4[nx < R ? nx : R - 1];
-        }
-        // Bursts make most requests repeat the model of the one before: the block is cut into runs of
-        // equal model words, and descriptors are fetched once per run.
-        const int before = __builtin_amdgcn_ds_bpermute(((lane - 1) & 63) << 2, r.z);
-        const uint64_t starts = __ballot(lane < nblk && (lane == 0 || r.z != before)) | 1ull;
-        const uint64_t valid = nblk == kWave ? ~0ull : ((1ull << nblk) - 1ull);
-        if constexpr (SKIP) {
-            skip = 0;
-            ch_looked = false;
+            const int z0 = __builtin_amdgcn_readlane(ahead.z, 0);
+            fetch_run(r0 < r1 ? z0 : -1);
         }
 
-        for (int s0 = 0; s0 < nblk;) {
-            const uint64_t later = starts & (s0 >= 63 ? 0ull : (~0ull << (s0 + 1)));
-            const int s1 = later ? (int)__builtin_ctzll(later) : nblk;  // the run is requests [s0, s1)
-            const uint4 da = nda, db = ndb;
-            {   // the run after this one: of this block, or the first of the next block
-                int zn = -1;
-                if (s1 < nblk)
-                    zn = __builtin_amdgcn_readlane(r.z, s1);
-                else if (blk + kWave < r1)
-                    zn = __builtin_amdgcn_readlane(ahead.z, 0);
-                fetch_run(zn < 0 ? -1 : (zn & 0xFFFFFF));
+        for (int64_t blk = r0; blk < r1; blk += kWave) {
+            // Lane j holds request j of the block; the request being simulated is read out of these
+            // registers with v_readlane.  The model word also carries the tile's replica bound.
+            const int nblk = (int)(r1 - blk < kWave ? r1 - blk : kWave);  // requests in this block
+            int4 r = ahead;
+            {
+                const bool ok = lane < nblk && r.z >= 0;
+                const int bound = (int)rmax_lds[ok ? r.z : 0];
+                r.z = ok ? (r.z | (bound << 24)) : -1;
             }
-            const int w = __builtin_amdgcn_readlane(r.z, s0);
-            const int m = w >= 0 ? (w & 0xFFFFFF) : -1;  // wave-uniform model id (or -1)
-            const int n = w >= 0 ? (w >> 24) : 0;        // replica bound of the tile; 0: nothing to simulate
-            const uint64_t run = (s1 >= 64 ? ~0ull : ((1ull << s1) - 1ull)) & (~0ull << s0) & valid;
-
-            auto request = [&](int i) {
-                const double tstamp = __hiloint2double(__builtin_amdgcn_readlane(r.y, i), __builtin_amdgcn_readlane(r.x, i));
-                const double slo = (double)__int_as_float(__builtin_amdgcn_readlane(r.w, i));
-            const float *lrow_m = lat_base + (size_t)(m < 0 ? 0 : m) * a.lat_row;
-
-            // ---- choose the replica group: strictly smallest last-stage clock (:590-598).
-            //      One LDS round trip fetches, for every listed replica, the clock of its last
-            //      stage and the latency of its last stage (needed by the early-reject bound).
-            // Strictly smallest clock, first listed wins ties: a tournament whose left side wins ties
-            // picks the same entry as the reference's left-to-right scan, in log2 dependent steps.
-            // Entries past a lane's own replicas are empty descriptors, whose clock reads +inf.
-            struct Cand {
-                double c;
-                uint32_t d;
-                float l;
-            };
-            auto first_min = [](const Cand &x, const Cand &y) {
-                const bool right = y.c < x.c;
-                return Cand{vmin(x.c, y.c), right ? y.d : x.d, right ? y.l : x.l};
-            };
-            auto scan = [&](Cand &win, auto NJ) {
-                constexpr int nj = decltype(NJ)::value;
-                Cand k[nj];
-                static_while<0, nj>([&](auto J) {
-                    constexpr int j = decltype(J)::value;
-                    k[j].d = pick_desc<j>(da, db);
-                    k[j].c = lds_f64(rep_addr(k[j].d));
-                    k[j].l = lrow_m[rep_lat_last(k[j].d)];
-                    return true;
-                });
-                const Cand a01 = first_min(k[0], k[1]), a23 = first_min(k[2], k[3]);
-                win = first_min(a01, a23);
-                if constexpr (nj == 8) {
-                    const Cand a45 = first_min(k[4], k[5]), a67 = first_min(k[6], k[7]);
-                    win = first_min(win, first_min(a45, a67));
-                }
-            };
-            // Clocks change only when a request is accepted, so while no lane of the wavefront has
-            // accepted anything since the last scan, a request for the same model finds the same group
-            // in every lane: the choice is kept from request to request (bursts make most requests
-            // repeat the model of the one before, and most of a burst is rejected).
-            if (m != ch_model || ch_stale) {
-                Cand win{__builtin_inf(), kEmpty, 0.0f};
-                if (n > 4)
-                    scan(win, Idx<8>{});
-                else if (n > 0)
-                    scan(win, Idx<4>{});
-                if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
-                    const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
-                    for (int j = RREG; j < n; ++j) {
-                        const uint32_t d = row[(size_t)(j - RREG) * kWave];
-                        win = first_min(win, Cand{lds_f64(rep_addr(d)), d, lrow_m[rep_lat_last(d)]});
-                    }
-                }
-                // a clock that is infinite (a group that served a request with infinite latency) is never
-                // chosen (:590-598: "tmp < min_device_clock" with min_device_clock starting at inf)
-                ch_model = m;
-                ch_looked = false;
-                ch_best = win.c;
-                ch_sel = win.c < 1e100 ? win.d : kEmpty;
-                ch_l_last = (double)win.l;
+            {
+                const int64_t nx = blk + kWave + lane;
+                ahead = reqs4[nx < R ? nx : R - 1];
             }
-            const double best = ch_best;
-            const uint32_t sel = ch_sel;
-            const bool has = (int32_t)sel >= 0;
-            const int sm1 = has ? (int)rep_stages_m1(sel) : -1;  // stages - 1
-            const uint32_t last_addr = rep_addr(sel);            // the lane's +inf clock when there is no replica
-            const uint32_t first_addr = last_addr - (uint32_t)(has ? sm1 : 0) * kSlotBytes;
-            const float *lrow = lrow_m + (has ? (int)rep_lat_last(sel) - sm1 : 0);
-            const double l_last = ch_l_last;
-
-            double finish_time;
-            bool acc;
-            if constexpr (SMAX == 1) {
-                // ---- single-stage groups: the clock read for the choice is the whole pipeline (:605-619)
-                const double t = vmax(tstamp, best) + l_last;
-                finish_time = t + overhead;
-                const double latency = finish_time - tstamp;
-                acc = has && latency <= slo;
-                if (acc) {
-                    lds_set_f64(last_addr, t);
-                    n_good += 1;
-                    lat_sum += latency;
-                }
-            } else {
-                // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
-                const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
-                const int walk = (int)(has & !(bound > slo)) != 0 ? sm1 : -1;  // stages - 1 of lanes that walk (no per-lane branch)
-                if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
-                    // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
-                    uint64_t saved_exec, mask1, mask2, mask4, mask8;  // masks: scratch of the power-of-two walk
-                    int accepted;
-                    double latency;
-                    const uint32_t cb_addr = first_addr;
-#define MMSIM_WALK(NAME, LATNAME, LATVAL)                                                                           \
-asm volatile(NAME##_TEXT                                                                                        \
-             : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [fin] "=&v"(finish_time), [lat] "=&v"(latency),   \
-               [ng] "+v"(n_good), [ls] "+v"(lat_sum), [m1] "=&s"(mask1), [m2] "=&s"(mask2), [m4] "=&s"(mask4),  \
-               [m8] "=&s"(mask8)                                                                                \
-             : [walk] "v"(walk), [cb] "v"(cb_addr), [LATNAME] "v"(LATVAL), [ts] "v"(tstamp), [slo] "v"(slo),    \
-               [oh] "s"(overhead)                                                                               \
-             : "vcc", "scc", "memory", NAME##_CLOBBERS)
-                    if constexpr (UNIFORM) {
-                        if (pow2) {
-                            if constexpr (SMAX == 4)
-                                MMSIM_WALK(MMSIM_WALK_PU4, lc, l_last);
-                            else
-                                MMSIM_WALK(MMSIM_WALK_PU16, lc, l_last);
-                        } else {
-                            if constexpr (SMAX == 4)
-                                MMSIM_WALK(MMSIM_WALK_U4, lc, l_last);
-                            else
-                                MMSIM_WALK(MMSIM_WALK_U16, lc, l_last);
-                        }
-                    } else {
-                        const uint32_t lb = lds_addr(lrow);
-                        if (pow2) {
-                            if constexpr (SMAX == 4)
-                                MMSIM_WALK(MMSIM_WALK_PN4, lb, lb);
-                            else
-                                MMSIM_WALK(MMSIM_WALK_PN16, lb, lb);
-                        } else {
-                            if constexpr (SMAX == 4)
-                                MMSIM_WALK(MMSIM_WALK_N4, lb, lb);
-                            else
-                                MMSIM_WALK(MMSIM_WALK_N16, lb, lb);
-                        }
-                    }
-#undef MMSIM_WALK
-                    acc = accepted != 0;
-                } else {
-                    // ---- the same in plain C++ (other stage buckets, latency table in global memory):
-                    //      fetch, then the dependent chain (:605-608)
-                    double *gclk = reinterpret_cast<double *>(lds_raw + first_addr);
-                    double cv[SMAX];
-                    float lv[SMAX];
-                    walk_blocks<0, 1, SMAX>(
-                        [&](auto K) { return decltype(K)::value <= walk; },
-                        [&](auto K) {
-                            constexpr int k = decltype(K)::value;
-                            cv[k] = gclk[k * kWave];
-                            if (!UNIFORM) lv[k] = lrow[k];
-                        });
-                    double t = tstamp;
-                    walk_blocks<0, 1, SMAX>(
-                        [&](auto K) { return decltype(K)::value <= walk; },
-                        [&](auto K) {
-                            constexpr int k = decltype(K)::value;
-                            t = vmax(t, cv[k]) + (UNIFORM ? l_last : (double)lv[k]);
-                            cv[k] = t;
-                        });
-                    finish_time = t + overhead;  // :610
-                    const double latency = finish_time - tstamp;
-                    acc = walk >= 0 && latency <= slo;  // :613
-                    if (acc) {  // :614-619
-                        n_good += 1;
-                        lat_sum += latency;
-                    }
-                    const int commit = acc ? walk : -1;
-                    walk_blocks<0, 1, SMAX>(
-                        [&](auto K) { return decltype(K)::value <= commit; },
-                        [&](auto K) {
-                            constexpr int k = decltype(K)::value;
-                            gclk[k * kWave] = cv[k];
-                        });
-                }
-            }
-            ch_stale = __ballot(acc) != 0ull;
-            if (ch_stale) skip = 0;
-            if (want_group && has) {  // :611, :618
-                const uint32_t g = owner[(last_addr - clk_off) >> 3];  // (slot * 512 + lane * 8) / 8
-                // LDS adds that return nothing: the wavefront does not wait for them
-                __hip_atomic_fetch_add(&gcnt[g * kWave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-                __hip_atomic_fetch_add(&gcnt[(a.Gmax + g) * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_WAVEFRONT);
-            }
-            if (want_ops) {
-                asm volatile("" ::: "memory");  // keep this a wave-uniform branch, off the common path
-                int nvalid = 0;
-                static_while<0, RREG>([&](auto J) {
-                    constexpr int j = decltype(J)::value;
-                    nvalid += (j < n && (int32_t)pick_desc<j>(da, db) >= 0) ? 1 : 0;
-                    return true;
-                });
-                if (n > RREG) {
-                    const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
-                    for (int j = RREG; j < n; ++j) nvalid += (int32_t)row[(size_t)(j - RREG) * kWave] >= 0 ? 1 : 0;
-                }
-                if (has) fp_ops += 2 * (sm1 + 1) + nvalid + 3;
-            }
-            if (model_lds) {  // an LDS add that returns nothing
-                if (m >= 0)
-                    __hip_atomic_fetch_add(&mcnt[m * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-            } else if (want_model && m >= 0 && acc) {  // one owner per counter: a relaxed add that nobody waits for
-                __hip_atomic_fetch_add(&model_good[(size_t)m * kWave], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            if (want_req) {
-                fin_out[(blk + i) * kWave] = acc ? finish_time : tstamp;
-                good_out[(blk + i) * kWave] = acc ? 1 : 0;
-            }
-            };
-
+            // Bursts make most requests repeat the model of the one before: the block is cut into runs of
+            // equal model words, and descriptors are fetched once per run.
+            const int before = __builtin_amdgcn_ds_bpermute(((lane - 1) & 63) << 2, r.z);
+            const uint64_t starts = __ballot(lane < nblk && (lane == 0 || r.z != before)) | 1ull;
+            const uint64_t valid = nblk == kWave ? ~0ull : ((1ull << nblk) - 1ull);
             if constexpr (SKIP) {
-                for (int i = s0; i < s1;) {
-                    request(i);
-                    // Nobody accepted: until somebody does, a request of this model is rejected by every lane
-                    // (before any walk) if  fl(fl(fl(max(t, best) + l_last) + overhead) - t) > slo  in every
-                    // lane.  For t <= best in every lane the left side is fl(C - t) with
-                    // C = fl(fl(best + l_last) + overhead), and rounding is monotone, so the smallest C of
-                    // the wavefront decides for all lanes at once: lane j tests request j of the block, and
-                    // the requests found are not simulated (a rejected request changes nothing and, with
-                    // scores only, counts nowhere).
-                    if (a.skip_ahead && !ch_stale && !ch_looked && i + 1 < s1) {
-                        ch_looked = true;
-                        const bool chosen = (int32_t)ch_sel >= 0;
-                        const double cmin = wave_min(chosen ? (ch_best + ch_l_last) + overhead : __builtin_inf());
-                        const double bmin = wave_min(chosen ? ch_best : __builtin_inf());
-                        const double tj = __hiloint2double(r.y, r.x);
-                        const bool rejected = r.z == w && tj <= bmin && (cmin - tj) > (double)__int_as_float(r.w);
-                        skip |= __ballot(rejected);
-                    }
-                    const uint64_t todo = run & ~skip & (i >= 63 ? 0ull : (~0ull << (i + 1)));
-                    i = todo ? (int)__builtin_ctzll(todo) : s1;
-                }
-            } else {
-                for (int i = s0; i < s1; ++i) request(i);
+                skip = 0;
+                ch_looked = false;
             }
-            s0 = s1;
+
+            for (int s0 = 0; s0 < nblk;) {
+                const uint64_t later = starts & (s0 >= 63 ? 0ull : (~0ull << (s0 + 1)));
+                const int s1 = later ? (int)__builtin_ctzll(later) : nblk;  // the run is requests [s0, s1)
+                const uint4 da = nda, db = ndb;
+                {   // the run after this one: of this block, or the first of the next block
+                    int zn = -1;
+                    if (s1 < nblk)
+                        zn = __builtin_amdgcn_readlane(r.z, s1);
+                    else if (blk + kWave < r1)
+                        zn = __builtin_amdgcn_readlane(ahead.z, 0);
+                    fetch_run(zn < 0 ? -1 : (zn & 0xFFFFFF));
+                }
+                const int w = __builtin_amdgcn_readlane(r.z, s0);
+                const int m = w >= 0 ? (w & 0xFFFFFF) : -1;  // wave-uniform model id (or -1)
+                const int n = w >= 0 ? (w >> 24) : 0;        // replica bound of the tile; 0: nothing to simulate
+                const uint64_t run = (s1 >= 64 ? ~0ull : ((1ull << s1) - 1ull)) & (~0ull << s0) & valid;
+
+                auto request = [&](int i) {
+                    simulate(blk + i, m, n, da, db,
+                             __hiloint2double(__builtin_amdgcn_readlane(r.y, i), __builtin_amdgcn_readlane(r.x, i)),
+                             (double)__int_as_float(__builtin_amdgcn_readlane(r.w, i)));
+                };
+
+                if constexpr (SKIP) {
+                    for (int i = s0; i < s1;) {
+                        request(i);
+                        // Nobody accepted: until somebody does, a request of this model is rejected by every lane
+                        // (before any walk) if  fl(fl(fl(max(t, best) + l_last) + overhead) - t) > slo  in every
+                        // lane.  For t <= best in every lane the left side is fl(C - t) with
+                        // C = fl(fl(best + l_last) + overhead), and rounding is monotone, so the smallest C of
+                        // the wavefront decides for all lanes at once: lane j tests request j of the block, and
+                        // the requests found are not simulated (a rejected request changes nothing and, with
+                        // scores only, counts nowhere).
+                        if (a.skip_ahead && !ch_stale && !ch_looked && i + 1 < s1) {
+                            ch_looked = true;
+                            const bool chosen = (int32_t)ch_sel >= 0;
+                            const double cmin = wave_min(chosen ? (ch_best + ch_l_last) + overhead : __builtin_inf());
+                            const double bmin = wave_min(chosen ? ch_best : __builtin_inf());
+                            const double tj = __hiloint2double(r.y, r.x);
+                            const bool rejected = r.z == w && tj <= bmin && (cmin - tj) > (double)__int_as_float(r.w);
+                            skip |= __ballot(rejected);
+                        }
+                        const uint64_t todo = run & ~skip & (i >= 63 ? 0ull : (~0ull << (i + 1)));
+                        i = todo ? (int)__builtin_ctzll(todo) : s1;
+                    }
+                } else {
+                    for (int i = s0; i < s1; ++i) request(i);
+                }
+                s0 = s1;
+            }
+        }
+    } else {
+        int4 *stage4 = reinterpret_cast<int4 *>(mine);
+        for (int64_t blk = r0; blk < r1; blk += kWave) {
+            {   // park this block's requests; the model word also carries the tile's replica bound
+                int4 r = ahead;
+                const bool ok = blk + lane < r1 && r.z >= 0;
+                const int bound = (int)rmax_lds[ok ? r.z : 0];
+                r.z = ok ? (r.z | (bound << 24)) : -1;
+                stage4[lane] = r;
+            }
+            {
+                const int64_t nx = blk + kWave + lane;
+                ahead = reqs4[nx < R ? nx : R - 1];
+            }
+            const int nblk = (int)(r1 - blk < kWave ? r1 - blk : kWave);  // requests in this block
+
+            // Always 2 * kChunk loads per chunk, whatever the requests are, so that the wait counters let
+            // the fetch of the next chunk overlap the simulation of this one.
+            auto load_chunk = [&](Chunk &c, int cb) {
+                int4 r[kChunk];
+                static_while<0, kChunk>([&](auto U) {
+                    constexpr int u = decltype(U)::value;
+                    r[u] = stage4[cb + u];  // broadcast read; cb + u < 64
+                    return true;
+                });
+                static_while<0, kChunk>([&](auto U) {
+                    constexpr int u = decltype(U)::value;
+                    const int w = uniform(r[u].z);
+                    const bool ok = w >= 0;
+                    const int m = ok ? (w & 0xFFFFFF) : -1;
+                    c.m[u] = m;
+                    c.nrep[u] = ok ? (w >> 24) : 0;  // 0: nothing to simulate (unknown model or no replica in the tile)
+                    c.t[u] = __hiloint2double(r[u].y, r[u].x);
+                    c.slo[u] = __int_as_float(r[u].w);
+                    const uint4 *row = rep_tile + (size_t)(ok ? m : 0) * (2 * kWave);
+                    c.da[u] = row[0];
+                    c.db[u] = row[kWave];
+                    return true;
+                });
+            };
+
+            Chunk cur, nxt;
+            load_chunk(cur, 0);
+            for (int cb = 0; cb < nblk; cb += kChunk) {
+                const bool more = cb + kChunk < nblk;
+                load_chunk(nxt, more ? cb + kChunk : cb);
+                static_while<0, kChunk>([&](auto U) {
+                    constexpr int u = decltype(U)::value;
+                    if (cb + u >= nblk) return false;
+                    simulate(blk + cb + u, cur.m[u], cur.nrep[u], cur.da[u], cur.db[u], cur.t[u], (double)cur.slo[u]);
+                    return true;
+                });
+                cur = nxt;
+            }
         }
     }
 
@@ -574,9 +653,9 @@ asm volatile(NAME##_TEXT                                                        
     }
 }
 
-template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT>
-hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
-    auto kern = sim_mixed_kernel<SMAX, LATLDS, UNIFORM, POW2, OUT>;
+template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT, bool RUNS>
+hipError_t launch_kernel(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
+    auto kern = sim_mixed_kernel<SMAX, LATLDS, UNIFORM, POW2, OUT, RUNS>;
     if (lds_bytes > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -586,6 +665,12 @@ hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStrea
     const dim3 grid((args.xcd_map ? ((tile_groups + 7u) & ~7u) : tile_groups) * (unsigned)args.n_seeds);
     hipLaunchKernelGGL(kern, grid, dim3(wpb * kWave), lds_bytes, stream, args);
     return hipGetLastError();
+}
+
+template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT>
+hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
+    return args.runs ? launch_kernel<SMAX, LATLDS, UNIFORM, POW2, OUT, true>(args, wpb, lds_bytes, stream)
+                     : launch_kernel<SMAX, LATLDS, UNIFORM, POW2, OUT, false>(args, wpb, lds_bytes, stream);
 }
 
 // The specialisations that pay are compiled for the usual case (latency table in LDS); with the

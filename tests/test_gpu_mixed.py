@@ -292,22 +292,26 @@ def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placem
     assert np.mean(st.model_ids[1:] == st.model_ids[:-1]) > 0.8
     ref = oracle_batch(st, table, packed)
     dw = E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models)
-    for skip in ("1", "0"):
+    for runs, skip in (("1", "1"), ("1", "0"), ("0", "1")):   # loop over runs (with / without skipping), chunked loop
+        monkeypatch.setenv("MMSIM_RUNS", runs)
         monkeypatch.setenv("MMSIM_SKIP_AHEAD", skip)
         batch = E.Batch(eng, [dw], table, packed, 0)
         batch.run()
         batch.sync()
         out = batch.fetch()
         batch.close()
-        assert np.array_equal(out["n_good"][0], ref["n_good"]), f"n_good differs (skip {skip})"
-        assert np.array_equal(out["latency_sum"][0], ref["latency_sum"]), f"latency_sum differs (skip {skip})"
+        assert np.array_equal(out["n_good"][0], ref["n_good"]), f"n_good differs (runs {runs}, skip {skip})"
+        assert np.array_equal(out["latency_sum"][0], ref["latency_sum"]), f"latency_sum differs (runs {runs}, skip {skip})"
     dw.close()
 
 
-def test_scores_only_on_runs_of_one_model_with_odd_requests(eng):
+@pytest.mark.parametrize("loop", ["runs", "chunks"])
+@pytest.mark.parametrize("flags", [0, ALL])
+def test_runs_of_one_model_with_odd_requests(eng, monkeypatch, loop, flags):
     """Runs of equal models with tied arrival times, SLOs that change inside a run (also inf and NaN),
-    unknown models, streams that end inside a block of 64, several seeds: scores-only results equal the
-    oracle's for every placement of configuration 2."""
+    unknown models, streams that end inside a block of 64, several seeds: results equal the oracle's for
+    every placement of configuration 2, with either request loop, scores only and with every output."""
+    monkeypatch.setenv("MMSIM_RUNS", "1" if loop == "runs" else "0")
     cfg = make_config(2)
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
     packed = E.pack_placements(cfg.placements, table)
@@ -328,16 +332,15 @@ def test_scores_only_on_runs_of_one_model_with_odd_requests(eng):
         slos[rng.random(R) < 0.01] = np.nan
         streams.append((ts, models, slos.astype(np.float32)))
     dws = [E.DeviceWorkload(eng, t, m, s, M) for t, m, s in streams]
-    batch = E.Batch(eng, dws, table, packed, 0)
+    batch = E.Batch(eng, dws, table, packed, flags)
     batch.run()
     batch.sync()
     out = batch.fetch()
     batch.close()
     from mms_amd.synthetic import Stream
     for k, (t, m, s) in enumerate(streams):
-        ref = oracle_batch(Stream(t, m, s), table, packed)
-        assert np.array_equal(out["n_good"][k], ref["n_good"]), f"n_good differs, stream {k}"
-        assert np.array_equal(out["latency_sum"][k], ref["latency_sum"]), f"latency_sum differs, stream {k}"
+        ref = oracle_batch(Stream(t, m, s), table, packed, want_per_request=bool(flags))
+        assert_batch_matches(out, ref, k, packed[0], per_request=bool(flags), where=f"stream {k}, {loop}")
         assert 0 < ref["n_good"].sum() < len(t) * len(cfg.placements) or len(t) < 64
 
 
