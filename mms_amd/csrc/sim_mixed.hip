@@ -10,18 +10,14 @@
 // touches global memory:
 //
 //   * requests are fetched 64 at a time with one coalesced 1 KiB load per
-//     wavefront (one block ahead, into registers), parked in LDS and read
-//     back with broadcast LDS reads;
+//     wavefront, one block ahead, into registers (lane j holds request j);
 //   * the replicas of the request's model are 32-bit descriptors made for the
 //     lane that reads them (LDS address of the group's last-stage clock,
 //     stage count, index of its last-stage latency), eight per (tile, model,
 //     lane) in two 16-byte words rep32[tile][model][2][lane] (two coalesced
-//     1 KiB loads per request, listed in the order the reference scans them).
+//     1 KiB loads, listed in the order the reference scans them).
 //     Missing replicas point at a clock that is +inf forever, so the scan
-//     needs no validity test.  Descriptors are fetched one chunk of requests
-//     ahead into registers together with the request's arrival time and SLO;
-//     the load count per chunk is fixed so the wait counters let the
-//     prefetch overlap the current chunk;
+//     needs no validity test;
 //   * per-lane stage clocks live in LDS as clk[slot][lane] (8 bytes each);
 //     the slots of a lane are its groups' pipeline stages laid end to end.
 //     The bank an access hits depends on the lane only, so any per-lane
@@ -35,9 +31,27 @@
 // clock and last-stage latency of every listed replica, (2) the stage clocks
 // of the chosen group; single-stage placements need only the first.
 // Group choice (strictly smallest last-stage clock, first listed wins ties)
-// is a select chain; stage walk, SLO decision and commit are one
+// is a tournament of selects; stage walk, SLO decision and commit are one
 // hand-scheduled inline-asm block (walk_asm.inc), with a C++ version for the
 // shapes the block is not generated for.
+//
+// Two request loops (template argument RUNS, chosen by the host from how often
+// a stream's requests repeat the model of the one before):
+//   * chunks: the block is parked in LDS; four requests at a time are read
+//     back with broadcast reads and their descriptors fetched one chunk
+//     ahead (always eight loads per chunk, so the wait counters let the
+//     fetch overlap the current chunk);
+//   * runs (bursty streams): the block is cut into runs of equal models with
+//     one ballot; descriptors are fetched once per run, one run ahead, and
+//     the request simulated is read out of the lanes' registers with
+//     v_readlane.  Clocks change only when a request is accepted, so the
+//     chosen group is kept from request to request while no lane of the
+//     wavefront has accepted anything, and with scores as the only output the
+//     requests that every lane must then reject are found for the whole block
+//     at once and not simulated at all (see the loop).
+// One wavefront per SIMD issues at most one instruction every four cycles,
+// whatever its kind, so the loops are written for few instructions and few
+// per-lane branches.
 //
 // A lane whose request cannot meet its SLO even if it only had to wait for
 // the chosen group's last stage skips the walk: with t >= arrival at every
@@ -282,7 +296,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     bool ch_stale = true;     // wave-uniform: some lane accepted a request since
     double ch_best = __builtin_inf(), ch_l_last = 0.0;
     uint32_t ch_sel = kEmpty;
-    constexpr bool SKIP = RUNS && OUT == 0;
+    constexpr bool SKIP = RUNS && OUT <= 1;  // per-request outputs and operation counts need every request
     bool ch_looked = false;   // wave-uniform: the block has been searched for requests that the current choice rejects
     uint64_t skip = 0;        // wave-uniform: requests of the block that every lane rejects while nobody accepts
 
@@ -561,8 +575,9 @@ asm volatile(NAME##_TEXT                                                        
                         // lane.  For t <= best in every lane the left side is fl(C - t) with
                         // C = fl(fl(best + l_last) + overhead), and rounding is monotone, so the smallest C of
                         // the wavefront decides for all lanes at once: lane j tests request j of the block, and
-                        // the requests found are not simulated (a rejected request changes nothing and, with
-                        // scores only, counts nowhere).
+                        // the requests found are not simulated: a rejected request changes nothing and counts
+                        // only as a request of the group its lane would have chosen (:611), which is the group
+                        // kept from the request before.
                         if (a.skip_ahead && !ch_stale && !ch_looked && i + 1 < s1) {
                             ch_looked = true;
                             const bool chosen = (int32_t)ch_sel >= 0;
@@ -573,7 +588,16 @@ asm volatile(NAME##_TEXT                                                        
                             skip |= __ballot(rejected);
                         }
                         const uint64_t todo = run & ~skip & (i >= 63 ? 0ull : (~0ull << (i + 1)));
-                        i = todo ? (int)__builtin_ctzll(todo) : s1;
+                        const int next = todo ? (int)__builtin_ctzll(todo) : s1;
+                        if constexpr (OUT == 1) {
+                            const int passed = next - (i + 1);  // requests of the run that are not simulated
+                            if (want_group && passed > 0 && (int32_t)ch_sel >= 0) {
+                                const uint32_t g = owner[(rep_addr(ch_sel) - clk_off) >> 3];
+                                __hip_atomic_fetch_add(&gcnt[g * kWave], (uint32_t)passed, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_WAVEFRONT);
+                            }
+                        }
+                        i = next;
                     }
                 } else {
                     for (int i = s0; i < s1; ++i) request(i);

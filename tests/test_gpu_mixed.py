@@ -302,11 +302,19 @@ def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placem
         batch.close()
         assert np.array_equal(out["n_good"][0], ref["n_good"]), f"n_good differs (runs {runs}, skip {skip})"
         assert np.array_equal(out["latency_sum"][0], ref["latency_sum"]), f"latency_sum differs (runs {runs}, skip {skip})"
+    # per-model and per-group counts: requests that are not simulated still count for the group they would have chosen
+    monkeypatch.setenv("MMSIM_RUNS", "1")
+    batch = E.Batch(eng, [dw], table, packed, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
+    batch.run()
+    batch.sync()
+    out = batch.fetch()
+    batch.close()
+    assert_batch_matches(out, ref, 0, packed[0], where="counts, loop over runs")
     dw.close()
 
 
 @pytest.mark.parametrize("loop", ["runs", "chunks"])
-@pytest.mark.parametrize("flags", [0, ALL])
+@pytest.mark.parametrize("flags", [0, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS, ALL])
 def test_runs_of_one_model_with_odd_requests(eng, monkeypatch, loop, flags):
     """Runs of equal models with tied arrival times, SLOs that change inside a run (also inf and NaN),
     unknown models, streams that end inside a block of 64, several seeds: results equal the oracle's for
@@ -339,8 +347,9 @@ def test_runs_of_one_model_with_odd_requests(eng, monkeypatch, loop, flags):
     batch.close()
     from mms_amd.synthetic import Stream
     for k, (t, m, s) in enumerate(streams):
-        ref = oracle_batch(Stream(t, m, s), table, packed, want_per_request=bool(flags))
-        assert_batch_matches(out, ref, k, packed[0], per_request=bool(flags), where=f"stream {k}, {loop}")
+        traces = bool(flags & _lib.WANT_PER_REQUEST)
+        ref = oracle_batch(Stream(t, m, s), table, packed, want_per_request=traces)
+        assert_batch_matches(out, ref, k, packed[0], per_request=traces, where=f"stream {k}, {loop}")
         assert 0 < ref["n_good"].sum() < len(t) * len(cfg.placements) or len(t) < 64
 
 
