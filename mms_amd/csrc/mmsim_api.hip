@@ -132,6 +132,9 @@ struct mmsim_batch {
     DevBuf<int32_t> n_good;
     DevBuf<double> lat_sum;
     DevBuf<int32_t> model_good, group_req, group_good;
+    DevBuf<unsigned long long> slot_cnt;      // per-group counts by last clock slot [waves][nslots][64] (group_global)
+    std::vector<int16_t> group_last_slot;     // [B][Gmax] last clock slot of each group, -1: no such group (group_global)
+    int32_t group_global = 0, slot_rows = 0;
     DevBuf<double> finish;
     DevBuf<uint8_t> good;
     DevBuf<int64_t> fp_ops;
@@ -315,9 +318,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     // plain simulator, per wavefront: request block | replica bounds | clocks (one extra row that stays +inf)
     // | slot owners | group counters | model counters; the latency table is shared by the workgroup
     size_t model_lds_bytes = 0;  // per-model counters [M][64] in LDS (decided below)
+    bool group_in_lds = (flags & MMSIM_WANT_GROUP_COUNTS) != 0;  // slot owners and group counters in LDS (decided below)
     auto mixed_wave_bytes = [&](int ns) {
         return ((size_t)mixed_clock_offset(rmax_lds_bytes) + (size_t)(ns + 1) * kSlotBytes +
-                ((flags & MMSIM_WANT_GROUP_COUNTS)
+                (group_in_lds
                      ? (((size_t)ns * kWave + 15) & ~(size_t)15) + (size_t)2 * Gmax * kWave * sizeof(uint32_t)
                      : 0) + model_lds_bytes + 15) & ~(size_t)15;
     };
@@ -337,6 +341,19 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (lat_bytes + wave_bytes + lds_tail > (size_t)ctx->max_lds) {
             lds_tail = 0;
             pow2_depths = false;
+        }
+        // Per-group counters: slot owners and counters in LDS can cost a CU a wavefront (configuration 4: three
+        // instead of four, i.e. three rounds of wavefronts instead of two).  The counts-only kernel can keep them in
+        // registers per lane instead and add them to global rows when the lane's group changes; that is used when
+        // it gives a CU more wavefronts.  MMSIM_GROUP_COUNTS_LDS=0/1 forces the choice (tuning knob).
+        if (group_in_lds && !(flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT))) {
+            const size_t room = (size_t)ctx->max_lds - lat_bytes - lds_tail;
+            const size_t with = std::min<size_t>(wpb_cap, room / wave_bytes);
+            group_in_lds = false;
+            const size_t without = std::min<size_t>(wpb_cap, room / mixed_wave_bytes(nslots));
+            group_in_lds = without <= with;
+            if (const char *env = std::getenv("MMSIM_GROUP_COUNTS_LDS")) group_in_lds = std::atoi(env) != 0;
+            wave_bytes = mixed_wave_bytes(nslots);
         }
         // Per-model counters: one relaxed add to a global row per accepted (lane, request) costs a small
         // batch (one wavefront per CU, nothing to hide behind) about 300 cycles per request, because later
@@ -761,6 +778,16 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         HIP_TRY(b->group_req.alloc(lanes_padded * Gmax));
         HIP_TRY(b->group_good.alloc(lanes_padded * Gmax));
     }
+    if (!batching && (flags & MMSIM_WANT_GROUP_COUNTS) && !group_in_lds) {
+        b->group_global = 1;
+        b->slot_rows = nslots;
+        HIP_TRY(b->slot_cnt.alloc(lanes_padded * (size_t)nslots));
+        b->group_last_slot.assign((size_t)B * Gmax, -1);
+        for (int32_t p = 0; p < B; ++p)
+            for (int32_t g = 0; g < rl.num_groups[p]; ++g)
+                b->group_last_slot[(size_t)p * Gmax + g] =
+                    (int16_t)(slot0[(size_t)p * Gmax + g] + t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]] - 1);
+    }
     if (flags & MMSIM_WANT_PER_REQUEST) {
         HIP_TRY(b->finish.alloc(lanes_padded * (size_t)b->Rmax));
         HIP_TRY(b->good.alloc(lanes_padded * (size_t)b->Rmax));
@@ -825,6 +852,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.lat_sum = b->lat_sum.p;
     a.model_good = b->model_good.p;
     a.model_lds = model_lds_bytes ? 1 : 0;
+    a.group_global = b->group_global;
+    a.slot_cnt = b->slot_cnt.p;
     a.xcd_map = 1;
     {   // bursty streams (most requests repeat the model of the one before) get the loop over runs
         int64_t rep = 0, tot = 0;
@@ -1041,6 +1070,9 @@ int mmsim_batch_run(mmsim_batch *b) {
     HIP_TRY(hipSetDevice(ctx->device));
     if (b->flags & MMSIM_WANT_MODEL_COUNTS)
         HIP_TRY(hipMemsetAsync(b->model_good.p, 0, b->model_good.bytes(), ctx->stream));
+    if (b->group_global) {
+        HIP_TRY(hipMemsetAsync(b->slot_cnt.p, 0, b->slot_cnt.bytes(), ctx->stream));
+    }
     if ((b->flags & MMSIM_BATCHING) && (b->flags & MMSIM_WANT_GROUP_COUNTS)) {
         HIP_TRY(hipMemsetAsync(b->group_req.p, 0, b->group_req.bytes(), ctx->stream));
         HIP_TRY(hipMemsetAsync(b->group_good.p, 0, b->group_good.bytes(), ctx->stream));
@@ -1157,7 +1189,21 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
                     out->model_num_requests[((size_t)s * B + p) * M + m] =
                         (b->hosted.empty() || b->hosted[(size_t)p * M + m]) ? b->wl[s]->model_num_requests[m] : 0;
     }
-    if (wg) {
+    if (wg && b->group_global) {  // counted per last clock slot of the group: map slots back to groups
+        std::vector<unsigned long long> h(b->slot_cnt.n);
+        HIP_TRY(hipMemcpy(h.data(), b->slot_cnt.p, b->slot_cnt.bytes(), hipMemcpyDeviceToHost));
+        const size_t rows = (size_t)b->slot_rows;
+        for (int s = 0; s < b->n_seeds; ++s)
+            for (int32_t p = 0; p < B; ++p) {
+                const size_t wave = (size_t)s * tiles + b->pos[p] / kWave;
+                for (int32_t g = 0; g < Gmax; ++g) {
+                    const int slot = b->group_last_slot[(size_t)p * Gmax + g];
+                    const unsigned long long v = slot < 0 ? 0ull : h[(wave * rows + slot) * kWave + b->pos[p] % kWave];
+                    out->group_num_requests[((size_t)s * B + p) * Gmax + g] = (int32_t)(v & 0xFFFFFFFFull);
+                    out->group_num_good[((size_t)s * B + p) * Gmax + g] = (int32_t)(v >> 32);
+                }
+            }
+    } else if (wg) {
         int rc = unpack_i32(b->group_req, Gmax, out->group_num_requests);
         if (rc) return rc;
         rc = unpack_i32(b->group_good, Gmax, out->group_num_good);

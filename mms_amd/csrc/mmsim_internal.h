@@ -120,6 +120,10 @@ struct MixedArgs {
     int32_t *error;              // set to 1 if the kernel finds its LDS layout assumption broken
     int32_t model_lds;           // 1: per-model counters [M][64] live in LDS behind the group counters (small batches,
                                  // where LDS is not what limits the wavefronts per CU); 0: relaxed adds to model_good
+    int32_t group_global;        // 1: per-group counts are kept per lane in registers and added to slot_cnt when
+                                 // the lane's group changes (no group counters or slot owners in LDS); 0: counters in LDS
+    unsigned long long *slot_cnt;  // [waves][slot_rows][64] requests (low half) and accepted requests (high half) of the group
+                                 // whose last clock slot this is (group_global; zeroed by the host before the first segment)
     int32_t runs;                // 1: the request loop walks runs of equal models (streams whose requests mostly repeat the
                                  // model of the one before); 0: fixed chunks of four requests
     int32_t skip_ahead;          // 1: requests that every lane must reject are found a block at a time and not simulated (scores only)

@@ -234,11 +234,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     uint8_t *rmax_lds = mine + kStageBytes;
     const uint32_t clk_off = (uint32_t)(a.lat_lds_bytes + wv * a.wave_lds_bytes) + mixed_clock_offset(a.rmax_lds_bytes);
     double *clk = reinterpret_cast<double *>(lds_raw + clk_off) + lane;
-    const int own_bytes = want_group ? ((a.nslots * kWave + 15) & ~15) : 0;
+    const bool group_regs = want_group && a.group_global != 0;  // counts per lane in registers, flushed to global rows
+    const bool group_lds = want_group && !group_regs;
+    const int own_bytes = group_lds ? ((a.nslots * kWave + 15) & ~15) : 0;
     uint8_t *owner = lds_raw + clk_off + (a.nslots + 1) * kSlotBytes;  // owner[slot * 64 + lane]
     uint32_t *gcnt = reinterpret_cast<uint32_t *>(owner + own_bytes) + lane;
     const bool model_lds = want_model && a.model_lds != 0;
-    uint32_t *mcnt = gcnt + (want_group ? 2 * a.Gmax * kWave : 0);  // [M][64] accepted requests per model
+    uint32_t *mcnt = gcnt + (group_lds ? 2 * a.Gmax * kWave : 0);  // [M][64] accepted requests per model
 
     for (int i = (int)threadIdx.x; i < lat_floats; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
     if (live)
@@ -271,7 +273,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
     }
     clk[a.nslots * kWave] = __builtin_inf();
-    if (want_group) {
+    if (group_lds) {
         for (int s = 0; s < a.nslots; ++s) owner[s * kWave + lane] = a.slot_group[((size_t)tile * a.slot_rows + s) * kWave + lane];
         for (int g = 0; g < a.Gmax; ++g) {
             gcnt[g * kWave] = resume ? (uint32_t)greq[g * kWave] : 0u;
@@ -299,6 +301,17 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     constexpr bool SKIP = RUNS && OUT <= 1;  // per-request outputs and operation counts need every request
     bool ch_looked = false;   // wave-uniform: the block has been searched for requests that the current choice rejects
     uint64_t skip = 0;        // wave-uniform: requests of the block that every lane rejects while nobody accepts
+
+    // Per-group counts without LDS (group_regs): a lane's group changes about once per run of equal models, so the
+    // lane counts in registers and adds them to the global row of the group's last clock slot only when its group
+    // changes (relaxed adds that nobody waits for; every counter has one owner).
+    uint32_t pg_addr = 0xFFFFFFFFu, pg_req = 0, pg_good = 0;  // LDS address of the group's last-stage clock, or none
+    unsigned long long *slot_cnt = a.slot_cnt + (size_t)wave * a.slot_rows * kWave;
+    auto flush_group = [&]() {
+        if (pg_addr != 0xFFFFFFFFu && pg_req != 0)  // one 64-bit add: requests in the low half, accepted ones in the high half
+            __hip_atomic_fetch_add(&slot_cnt[(pg_addr - clk_off) >> 3], ((unsigned long long)pg_good << 32) | pg_req,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
 
     // One request for the whole wavefront: `at` is its place in the stream, m / n the model and the tile's
     // replica bound for it (wave-uniform), da / db this lane's descriptors of the model's replicas.
@@ -471,7 +484,17 @@ asm volatile(NAME##_TEXT                                                        
             ch_stale = __ballot(acc) != 0ull;
             if (ch_stale) skip = 0;
         }
-        if (want_group && has) {  // :611, :618
+        if (group_regs) {  // :611, :618
+            const uint32_t now = has ? last_addr : 0xFFFFFFFFu;
+            if (now != pg_addr) {
+                flush_group();
+                pg_addr = now;
+                pg_req = 0;
+                pg_good = 0;
+            }
+            pg_req += has ? 1u : 0u;
+            pg_good += acc ? 1u : 0u;
+        } else if (want_group && has) {  // :611, :618
             const uint32_t g = owner[(last_addr - clk_off) >> 3];  // (slot * 512 + lane * 8) / 8
             // LDS adds that return nothing: the wavefront does not wait for them
             __hip_atomic_fetch_add(&gcnt[g * kWave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
@@ -591,7 +614,9 @@ asm volatile(NAME##_TEXT                                                        
                         const int next = todo ? (int)__builtin_ctzll(todo) : s1;
                         if constexpr (OUT == 1) {
                             const int passed = next - (i + 1);  // requests of the run that are not simulated
-                            if (want_group && passed > 0 && (int32_t)ch_sel >= 0) {
+                            if (group_regs) {  // the lane's pending group is the one kept from the request before
+                                if ((int32_t)ch_sel >= 0) pg_req += (uint32_t)passed;
+                            } else if (want_group && passed > 0 && (int32_t)ch_sel >= 0) {
                                 const uint32_t g = owner[(rep_addr(ch_sel) - clk_off) >> 3];
                                 __hip_atomic_fetch_add(&gcnt[g * kWave], (uint32_t)passed, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_WAVEFRONT);
@@ -669,7 +694,8 @@ asm volatile(NAME##_TEXT                                                        
         for (int s = 0; s < a.nslots; ++s) saved[(size_t)s * kWave] = clk[s * kWave];
     if (model_lds)
         for (int m = 0; m < a.M; ++m) model_good[(size_t)m * kWave] = (int32_t)mcnt[m * kWave];
-    if (want_group) {
+    if (group_regs) flush_group();
+    if (group_lds) {
         for (int g = 0; g < a.Gmax; ++g) {
             greq[g * kWave] = (int32_t)gcnt[g * kWave];
             ggood[g * kWave] = (int32_t)gcnt[(a.Gmax + g) * kWave];

@@ -207,7 +207,10 @@ def test_stage_walk_variants(eng, depths, uniform):
     assert 0.05 * R * 130 < ref["n_good"].sum() < 0.98 * R * 130    # both accepts and rejects are exercised
 
 
-@pytest.mark.parametrize("flags", [0, ALL])
+COUNTS_IN_REGISTERS = -1    # per-model and per-group counts, the latter in registers with adds to global rows
+
+
+@pytest.mark.parametrize("flags", [0, COUNTS_IN_REGISTERS, ALL])
 @pytest.mark.parametrize("segments", [1, 5])
 def test_tile_classes_and_stream_segments(eng, monkeypatch, flags, segments):
     """Large batches are split into classes of tiles by clock-slot count (each launched with its own
@@ -220,6 +223,10 @@ def test_tile_classes_and_stream_segments(eng, monkeypatch, flags, segments):
     monkeypatch.setenv("MMSIM_WAVES_PER_CU", "8")
     monkeypatch.setenv("MMSIM_TILE_CLASSES", "1")
     monkeypatch.setenv("MMSIM_SEGMENTS", str(segments))
+    if flags == COUNTS_IN_REGISTERS:
+        flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
+        monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", "0")
+    traces = bool(flags & _lib.WANT_PER_REQUEST)
     rng = np.random.default_rng(77)
     M, R = 24, 3001
     pcs = [ParallelConfig(1, 1, d) for d in (1, 2, 4, 8)]
@@ -252,9 +259,9 @@ def test_tile_classes_and_stream_segments(eng, monkeypatch, flags, segments):
     out = batch.fetch()
     batch.close()
     for s, st in enumerate(streams):
-        ref = oracle_batch(st, table, packed, want_per_request=bool(flags))
-        assert_batch_matches(out, ref, s, packed[0], per_request=bool(flags), where=f"seed {s}")
-        if flags:
+        ref = oracle_batch(st, table, packed, want_per_request=traces)
+        assert_batch_matches(out, ref, s, packed[0], per_request=traces, where=f"seed {s}")
+        if traces:
             assert out["fp_ops"][s].sum() == ref["fp_ops"]
 
 
@@ -303,23 +310,30 @@ def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placem
         assert np.array_equal(out["n_good"][0], ref["n_good"]), f"n_good differs (runs {runs}, skip {skip})"
         assert np.array_equal(out["latency_sum"][0], ref["latency_sum"]), f"latency_sum differs (runs {runs}, skip {skip})"
     # per-model and per-group counts: requests that are not simulated still count for the group they would have chosen
-    monkeypatch.setenv("MMSIM_RUNS", "1")
-    batch = E.Batch(eng, [dw], table, packed, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
-    batch.run()
-    batch.sync()
-    out = batch.fetch()
-    batch.close()
-    assert_batch_matches(out, ref, 0, packed[0], where="counts, loop over runs")
+    # (group counters in LDS, or in registers with adds to global rows when a lane's group changes)
+    for runs, lds in (("1", "1"), ("1", "0"), ("0", "0")):
+        monkeypatch.setenv("MMSIM_RUNS", runs)
+        monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", lds)
+        batch = E.Batch(eng, [dw], table, packed, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
+        for _ in range(2):      # a second run starts from zeroed counters again
+            batch.run()
+            batch.sync()
+        out = batch.fetch()
+        batch.close()
+        assert_batch_matches(out, ref, 0, packed[0], where=f"counts, runs {runs}, group counters in LDS {lds}")
     dw.close()
 
 
 @pytest.mark.parametrize("loop", ["runs", "chunks"])
-@pytest.mark.parametrize("flags", [0, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS, ALL])
+@pytest.mark.parametrize("flags", [0, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS, _lib.WANT_GROUP_COUNTS + 1000, ALL])
 def test_runs_of_one_model_with_odd_requests(eng, monkeypatch, loop, flags):
     """Runs of equal models with tied arrival times, SLOs that change inside a run (also inf and NaN),
     unknown models, streams that end inside a block of 64, several seeds: results equal the oracle's for
     every placement of configuration 2, with either request loop, scores only and with every output."""
     monkeypatch.setenv("MMSIM_RUNS", "1" if loop == "runs" else "0")
+    if flags >= 1000:       # per-group counts alone, kept in registers and added to global rows
+        flags -= 1000
+        monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", "0")
     cfg = make_config(2)
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
     packed = E.pack_placements(cfg.placements, table)
