@@ -156,7 +156,8 @@ typedef struct {
                                                performs (controller.py:590-613) */
 } mmsim_result;
 
-/* Packs the placements, uploads them and allocates device result buffers. */
+/* Packs the placements, uploads them and allocates device result buffers.  The
+ * batch copies what it needs of the workloads: they may be destroyed before it. */
 int mmsim_batch_create(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
                        const mmsim_tables *tables, const mmsim_placements *placements,
                        uint32_t flags, mmsim_batch **out);
@@ -168,6 +169,25 @@ int mmsim_batch_sync(mmsim_batch *batch, float *kernel_ms);
 /* Copies results of the last completed run into caller memory. */
 int mmsim_batch_fetch(mmsim_batch *batch, mmsim_result *out);
 void mmsim_batch_destroy(mmsim_batch *batch);
+
+/*
+ * mmsim_eval_batch without any device allocation.  It has no counterpart in
+ * the reference; it is for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight search or serving loops, harnesses that
+ * forbid hipMalloc.  Same arguments, results and error codes as
+ * mmsim_eval_batch, bit for bit, but every device table and result buffer of
+ * the batch lives in a static device array of MMSIM_STATIC_SCRATCH_BYTES that
+ * the library holds on each GPU it runs on until the process ends: no
+ * hipMalloc, no hipFree.  A batch that needs more (many placements x models,
+ * several long streams, per-request outputs) is refused with MMSIM_E_NOMEM
+ * and a message that names the limit.  All calls on one GPU share that GPU's
+ * array: calls that overlap on one GPU race, from whichever contexts or
+ * threads they come.  The workloads are inputs and stay the caller's.
+ */
+#define MMSIM_STATIC_SCRATCH_BYTES (32u << 20)
+int mmsim_eval_batch_static(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                            const mmsim_tables *tables, const mmsim_placements *placements,
+                            uint32_t flags, mmsim_result *out);
 
 typedef struct {
     int32_t lanes, waves, n_seeds, B;

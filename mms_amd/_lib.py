@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("MMSIM_LIBRARY") or os.path.join(_HERE, "libmmsim.so")
 
 MMSIM_OK = 0
 E_INVALID, E_UNSUPPORTED, E_HIP, E_NOMEM, E_OVERFLOW = -1, -2, -3, -4, -5
+STATIC_SCRATCH_BYTES = 32 << 20
 BATCHING, WANT_MODEL_COUNTS, WANT_GROUP_COUNTS, WANT_PER_REQUEST, WANT_OP_COUNT = 1, 2, 4, 8, 16
 
 _p_i32 = C.POINTER(C.c_int32)
@@ -80,6 +81,8 @@ SIGNATURES = {
     "mmsim_batch_get_info": (C.c_int, [C.c_void_p, C.POINTER(BatchInfo)]),
     "mmsim_eval_batch": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
                                     C.POINTER(Placements), C.c_uint32, C.POINTER(Result)]),
+    "mmsim_eval_batch_static": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
+                                           C.POINTER(Placements), C.c_uint32, C.POINTER(Result)]),
     "mmsim_simulate_requests_mixed": (C.c_int, [
         C.c_void_p, _p_f64, _p_u8, _p_f64, _p_i32, _p_f32, _p_i32, _p_i32, _p_f32, C.c_int64,
         C.c_int32, C.c_int32, C.c_int32, C.c_double, _p_i32, _p_i32, _p_i32, _p_i32]),

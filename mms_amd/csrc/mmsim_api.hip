@@ -14,6 +14,7 @@
 #include <functional>
 #include <limits>
 #include <memory>
+#include <mutex>
 #include <new>
 
 #include "mmsim_internal.h"
@@ -40,23 +41,47 @@ int hip_fail(hipError_t e, const char *what) {
         if (e__ != hipSuccess) return hip_fail(e__, #expr); \
     } while (0)
 
+// Device memory for a batch comes either from hipMalloc or, while g_arena is set (mmsim_eval_batch_static), from
+// a bump allocator over the library's static device scratch: such buffers are never freed one by one.
+struct Arena {
+    unsigned char *base = nullptr;
+    size_t cap = 0, used = 0;
+    bool overflow = false;
+};
+thread_local Arena *g_arena = nullptr;
+
 template <typename T>
 struct DevBuf {
     T *p = nullptr;
     size_t n = 0;
+    bool owned = true;
     DevBuf() = default;
     DevBuf(const DevBuf &) = delete;
     DevBuf &operator=(const DevBuf &) = delete;
     ~DevBuf() { release(); }
     void release() {
-        if (p) (void)hipFree(p);
+        if (p && owned) (void)hipFree(p);
         p = nullptr;
         n = 0;
+        owned = true;
     }
     hipError_t alloc(size_t count) {
         release();
         n = count;
-        return hipMalloc(reinterpret_cast<void **>(&p), std::max<size_t>(count, 1) * sizeof(T));
+        const size_t bytes = std::max<size_t>(count, 1) * sizeof(T);
+        if (Arena *ar = g_arena) {
+            const size_t rounded = (bytes + 255) & ~(size_t)255;
+            if (rounded > ar->cap - ar->used) {
+                ar->overflow = true;
+                n = 0;
+                return hipErrorOutOfMemory;
+            }
+            p = reinterpret_cast<T *>(ar->base + ar->used);
+            ar->used += rounded;
+            owned = false;
+            return hipSuccess;
+        }
+        return hipMalloc(reinterpret_cast<void **>(&p), bytes);
     }
     size_t bytes() const { return n * sizeof(T); }
 };
@@ -65,6 +90,15 @@ struct DevBuf {
 
 constexpr int kSideStreams = 4;
 
+// Device scratch of mmsim_eval_batch_static: every device table and result buffer of one batch is carved out
+// of this array, so that entry point never allocates.  Each GPU the library runs on holds its own copy at its
+// own address until the process ends; host code only ever uses the address hipGetSymbolAddress returned for
+// the current device (kept in the context), never the array's name.
+static __device__ __align__(256) unsigned char scratch[MMSIM_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static unsigned char *g_scratch_ptr[kMaxDevices] = {};  // per device, filled by the first context made on it
+
 struct mmsim_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -72,6 +106,8 @@ struct mmsim_ctx {
     int max_lds = 0;
     hipStream_t side[kSideStreams] = {};  // tile classes of one batch run side by side on these
     hipEvent_t ev_fork = nullptr, ev_join[kSideStreams] = {};
+    unsigned char *scratch = nullptr;     // this device's copy of the static scratch (mmsim_eval_batch_static)
+    hipEvent_t ev_static[2] = {};         // timing events of batches that live in the static scratch
 };
 
 struct mmsim_workload {
@@ -107,7 +143,8 @@ struct mmsim_batch {
     int32_t smax_bucket = 0, rmax_all = 0, nslots = 0, waves_per_block = 1;
     size_t lds_bytes = 0;
     int64_t Rmax = 0, Rtotal = 0;
-    std::vector<const mmsim_workload *> wl;
+    std::vector<int64_t> wl_R;                           // [n_seeds] stream lengths
+    std::vector<std::vector<int32_t>> wl_model_requests;  // [n_seeds][M] requests per model of each stream
     std::vector<int32_t> pos;  // pos[placement] = tile * 64 + lane it is simulated on
     // Plain simulator: tiles are grouped into classes by how many clock slots they need; a class is
     // launched with its own LDS size and as many wavefronts per workgroup as then fit a CU.
@@ -149,11 +186,12 @@ struct mmsim_batch {
 
     MixedArgs args{};
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    bool own_events = true;  // false: the context's events (batch in the static scratch)
     bool ran = false;
 
     ~mmsim_batch() {
-        if (ev_start) (void)hipEventDestroy(ev_start);
-        if (ev_stop) (void)hipEventDestroy(ev_stop);
+        if (own_events && ev_start) (void)hipEventDestroy(ev_start);
+        if (own_events && ev_stop) (void)hipEventDestroy(ev_stop);
     }
 };
 
@@ -243,7 +281,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     b->B = B;
     b->M = M;
     b->Gmax = Gmax;
-    b->wl.assign(wls, wls + n_seeds);
+    for (int s = 0; s < n_seeds; ++s) {  // copied: the batch does not depend on the workloads outliving it
+        b->wl_R.push_back(wls[s]->R);
+        b->wl_model_requests.push_back(wls[s]->model_num_requests);
+    }
 
     // ---- per placement: slot layout; per (placement, model): replica count
     int smax = 1, rmax_all = 1, nslots = 1;
@@ -793,8 +834,14 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         HIP_TRY(b->good.alloc(lanes_padded * (size_t)b->Rmax));
     }
     if (flags & MMSIM_WANT_OP_COUNT) HIP_TRY(b->fp_ops.alloc(lanes_padded));
-    HIP_TRY(hipEventCreate(&b->ev_start));
-    HIP_TRY(hipEventCreate(&b->ev_stop));
+    if (g_arena) {
+        b->own_events = false;
+        b->ev_start = ctx->ev_static[0];
+        b->ev_stop = ctx->ev_static[1];
+    } else {
+        HIP_TRY(hipEventCreate(&b->ev_start));
+        HIP_TRY(hipEventCreate(&b->ev_stop));
+    }
     HIP_TRY(hipStreamSynchronize(st));  // host staging vectors go out of scope below
 
     // ---- segments.  When the workgroups of a run do not all fit on the chip at once, the streams are
@@ -949,6 +996,20 @@ int mmsim_ctx_create(int device, mmsim_ctx **out) {
         HIP_TRY(hipEventCreateWithFlags(&c->ev_join[i], hipEventDisableTiming));
     }
     HIP_TRY(hipEventCreateWithFlags(&c->ev_fork, hipEventDisableTiming));
+    HIP_TRY(hipEventCreate(&c->ev_static[0]));
+    HIP_TRY(hipEventCreate(&c->ev_static[1]));
+    {   // address of this device's copy of the static scratch: once per device, with that device current
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (device < kMaxDevices && g_scratch_ptr[device]) {
+            c->scratch = g_scratch_ptr[device];
+        } else {
+            void *sp = nullptr;
+            HIP_TRY(hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)));
+            if (!sp) return fail(MMSIM_E_HIP, "ctx_create: the static scratch has no device address");
+            c->scratch = static_cast<unsigned char *>(sp);
+            if (device < kMaxDevices) g_scratch_ptr[device] = c->scratch;
+        }
+    }
     *out = c.release();
     return MMSIM_OK;
 }
@@ -968,6 +1029,8 @@ void mmsim_ctx_destroy(mmsim_ctx *ctx) {
         if (ctx->ev_join[i]) (void)hipEventDestroy(ctx->ev_join[i]);
     }
     if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
+    for (hipEvent_t e : ctx->ev_static)
+        if (e) (void)hipEventDestroy(e);
     delete ctx;
 }
 
@@ -1187,7 +1250,7 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
             for (int32_t p = 0; p < B; ++p)
                 for (int32_t m = 0; m < M; ++m)  // the batching loop only counts requests of hosted models (:754-757, :773)
                     out->model_num_requests[((size_t)s * B + p) * M + m] =
-                        (b->hosted.empty() || b->hosted[(size_t)p * M + m]) ? b->wl[s]->model_num_requests[m] : 0;
+                        (b->hosted.empty() || b->hosted[(size_t)p * M + m]) ? b->wl_model_requests[s][m] : 0;
     }
     if (wg && b->group_global) {  // counted per last clock slot of the group: map slots back to groups
         std::vector<unsigned long long> h(b->slot_cnt.n);
@@ -1220,7 +1283,7 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
                 const size_t wave = (size_t)s * tiles + tile;
                 HIP_TRY(hipMemcpy(hf.data(), b->finish.p + wave * Rm * kWave, sizeof(double) * Rm * kWave, hipMemcpyDeviceToHost));
                 HIP_TRY(hipMemcpy(hg.data(), b->good.p + wave * Rm * kWave, Rm * kWave, hipMemcpyDeviceToHost));
-                const size_t Rs = (size_t)b->wl[s]->R;
+                const size_t Rs = (size_t)b->wl_R[s];
                 for (int l = 0; l < kWave; ++l) {
                     const int32_t p = owner[(size_t)tile * kWave + l];
                     if (p < 0) continue;
@@ -1279,6 +1342,37 @@ int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
     if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
     if (rc == MMSIM_OK) rc = mmsim_batch_fetch(b, out);
     mmsim_batch_destroy(b);
+    return rc;
+}
+
+int mmsim_eval_batch_static(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                            const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
+                            mmsim_result *out) {
+    if (!ctx || !out) return fail(MMSIM_E_INVALID, "eval_batch_static: null pointer");
+    if (!ctx->scratch) return fail(MMSIM_E_HIP, "eval_batch_static: the context has no static scratch");
+    int rc = check_tables(tables);
+    if (rc) return rc;
+    RepLists rl;
+    rc = lists_from_placements(placements, tables->M, tables->C, &rl);
+    if (rc) return rc;
+    // Every device buffer of the batch is carved out of the device's static scratch (nothing is allocated or
+    // freed on the device); the scratch keeps the last call's contents, and what must start at zero is
+    // cleared by build_batch / mmsim_batch_run as for any batch.
+    Arena arena;
+    arena.base = ctx->scratch;
+    arena.cap = MMSIM_STATIC_SCRATCH_BYTES;
+    mmsim_batch *b = nullptr;
+    g_arena = &arena;
+    rc = build_batch(ctx, workloads, n_seeds, tables, rl, flags, &b);
+    g_arena = nullptr;
+    if (rc != MMSIM_OK && arena.overflow)
+        return fail(MMSIM_E_NOMEM, "eval_batch_static: the batch (placements x models x seeds, streams, requested outputs) "
+                                   "needs more device scratch than the static " +
+                                       std::to_string((size_t)MMSIM_STATIC_SCRATCH_BYTES) + " bytes; use mmsim_eval_batch");
+    if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
+    if (rc == MMSIM_OK) rc = mmsim_batch_fetch(b, out);
+    mmsim_batch_destroy(b);  // frees nothing on the device: the buffers belong to the scratch
     return rc;
 }
 

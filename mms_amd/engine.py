@@ -155,6 +155,82 @@ def pack_placements(sols: Sequence, table: LatencyTable):
     return num_groups, group_cfg, gm_off, gm_idx
 
 
+def _result_arrays(flags, n_seeds, B, M, Gmax, Rmax):
+    """Caller-owned result arrays for L = n_seeds * B simulations and the mmsim_result that points at them."""
+    L = B * n_seeds
+    out = {"n_good": np.zeros(L, np.int64), "latency_sum": np.zeros(L, np.float64),
+           "status": np.zeros(L, np.int32)}
+    r = _lib.Result()
+    r.n_good = _lib.ptr(out["n_good"], C.c_int64)
+    r.latency_sum = _lib.ptr(out["latency_sum"], C.c_double)
+    r.status = _lib.ptr(out["status"], C.c_int32)
+    if flags & _lib.WANT_MODEL_COUNTS:
+        out["model_num_requests"] = np.zeros((L, M), np.int32)
+        out["model_num_good"] = np.zeros((L, M), np.int32)
+        r.model_num_requests = _lib.ptr(out["model_num_requests"], C.c_int32)
+        r.model_num_good = _lib.ptr(out["model_num_good"], C.c_int32)
+    if flags & _lib.WANT_GROUP_COUNTS:
+        out["group_num_requests"] = np.zeros((L, Gmax), np.int32)
+        out["group_num_good"] = np.zeros((L, Gmax), np.int32)
+        r.group_num_requests = _lib.ptr(out["group_num_requests"], C.c_int32)
+        r.group_num_good = _lib.ptr(out["group_num_good"], C.c_int32)
+    if flags & _lib.WANT_PER_REQUEST:
+        out["finish"] = np.zeros((L, Rmax), np.float64)
+        out["good"] = np.zeros((L, Rmax), np.uint8)
+        r.finish = _lib.ptr(out["finish"], C.c_double)
+        r.good = _lib.ptr(out["good"], C.c_uint8)
+    if flags & _lib.WANT_OP_COUNT:
+        out["fp_ops"] = np.zeros(L, np.int64)
+        r.fp_ops = _lib.ptr(out["fp_ops"], C.c_int64)
+    return out, r
+
+
+def _shape_results(out, n_seeds, B):
+    L = n_seeds * B
+    if "good" in out:
+        out["good"] = out["good"].astype(bool)
+    for k in list(out):
+        if out[k].ndim >= 1 and out[k].shape[0] == L:
+            out[k] = out[k].reshape((n_seeds, B) + out[k].shape[1:])
+    return out
+
+
+def _abi_inputs(workloads, table, packed, fixed_overhead):
+    """The mmsim_tables / mmsim_placements / workload-handle arguments of the batch entry points.
+    Returns (tables, placements, handles, keep): `keep` holds the arrays the structs point into."""
+    num_groups, group_cfg, gm_off, gm_idx = packed
+    lat, pp = table.arrays()
+    bss = _lib.carray(table.batch_sizes, np.int32)
+    B, Gmax = group_cfg.shape
+    t = _lib.Tables(lat.shape[0], lat.shape[1], lat.shape[2], lat.shape[3],
+                    _lib.ptr(lat, C.c_float), _lib.ptr(pp, C.c_int32), _lib.ptr(bss, C.c_int32),
+                    float(fixed_overhead))
+    num_groups = _lib.carray(num_groups, np.int32)
+    group_cfg = _lib.carray(group_cfg, np.int32)
+    gm_off = _lib.carray(gm_off, np.int64)
+    gm_idx = _lib.carray(gm_idx, np.int32)
+    p = _lib.Placements(B, Gmax, _lib.ptr(num_groups, C.c_int32),
+                        _lib.ptr(group_cfg, C.c_int32), _lib.ptr(gm_off, C.c_int64),
+                        _lib.ptr(gm_idx, C.c_int32))
+    wl = (C.c_void_p * len(workloads))(*[w._h for w in workloads])
+    return t, p, wl, (lat, pp, bss, num_groups, group_cfg, gm_off, gm_idx)
+
+
+def eval_batch(engine: "Engine", workloads, table: "LatencyTable", packed, flags: int = 0,
+               fixed_overhead: float = FIXED_OVERHEAD, static: bool = False):
+    """One call of ``mmsim_eval_batch`` (create + run + sync + fetch + destroy inside the library), or of
+    ``mmsim_eval_batch_static`` -- the same without any device allocation, for batches that fit the
+    library's static device scratch.  Result arrays are [n_seeds][B][...]."""
+    workloads = list(workloads)
+    t, p, wl, keep = _abi_inputs(workloads, table, packed, fixed_overhead)
+    n_seeds, B, Gmax = len(workloads), p.B, p.Gmax
+    out, r = _result_arrays(flags, n_seeds, B, t.M, Gmax, max(w.R for w in workloads))
+    fn = engine.lib.mmsim_eval_batch_static if static else engine.lib.mmsim_eval_batch
+    _lib.check(fn(engine._h, wl, n_seeds, C.byref(t), C.byref(p), int(flags), C.byref(r)))
+    del keep
+    return _shape_results(out, n_seeds, B)
+
+
 class Batch:
     """Device-resident batch of placements x seeds; run() may be repeated."""
 
@@ -163,24 +239,10 @@ class Batch:
         self.engine = engine
         self.workloads = list(workloads)
         self.flags = int(flags)
-        num_groups, group_cfg, gm_off, gm_idx = packed
-        lat, pp = table.arrays()
-        bss = _lib.carray(table.batch_sizes, np.int32)
-        self.B, self.Gmax = group_cfg.shape
-        self.M = lat.shape[0]
+        t, p, wl, keep = _abi_inputs(self.workloads, table, packed, fixed_overhead)
+        self.B, self.Gmax, self.M = p.B, p.Gmax, t.M
         self.n_seeds = len(self.workloads)
         self.Rmax = max(w.R for w in self.workloads)
-        t = _lib.Tables(lat.shape[0], lat.shape[1], lat.shape[2], lat.shape[3],
-                        _lib.ptr(lat, C.c_float), _lib.ptr(pp, C.c_int32), _lib.ptr(bss, C.c_int32),
-                        float(fixed_overhead))
-        num_groups = _lib.carray(num_groups, np.int32)
-        group_cfg = _lib.carray(group_cfg, np.int32)
-        gm_off = _lib.carray(gm_off, np.int64)
-        gm_idx = _lib.carray(gm_idx, np.int32)
-        p = _lib.Placements(self.B, self.Gmax, _lib.ptr(num_groups, C.c_int32),
-                            _lib.ptr(group_cfg, C.c_int32), _lib.ptr(gm_off, C.c_int64),
-                            _lib.ptr(gm_idx, C.c_int32))
-        wl = (C.c_void_p * self.n_seeds)(*[w._h for w in self.workloads])
         self._h = C.c_void_p()
         _lib.check(engine.lib.mmsim_batch_create(engine._h, wl, self.n_seeds, C.byref(t), C.byref(p),
                                                  self.flags, C.byref(self._h)))
@@ -200,38 +262,9 @@ class Batch:
         return {f[0]: getattr(bi, f[0]) for f in bi._fields_}
 
     def fetch(self):
-        L = self.B * self.n_seeds
-        out = {"n_good": np.zeros(L, np.int64), "latency_sum": np.zeros(L, np.float64),
-               "status": np.zeros(L, np.int32)}
-        r = _lib.Result()
-        r.n_good = _lib.ptr(out["n_good"], C.c_int64)
-        r.latency_sum = _lib.ptr(out["latency_sum"], C.c_double)
-        r.status = _lib.ptr(out["status"], C.c_int32)
-        if self.flags & _lib.WANT_MODEL_COUNTS:
-            out["model_num_requests"] = np.zeros((L, self.M), np.int32)
-            out["model_num_good"] = np.zeros((L, self.M), np.int32)
-            r.model_num_requests = _lib.ptr(out["model_num_requests"], C.c_int32)
-            r.model_num_good = _lib.ptr(out["model_num_good"], C.c_int32)
-        if self.flags & _lib.WANT_GROUP_COUNTS:
-            out["group_num_requests"] = np.zeros((L, self.Gmax), np.int32)
-            out["group_num_good"] = np.zeros((L, self.Gmax), np.int32)
-            r.group_num_requests = _lib.ptr(out["group_num_requests"], C.c_int32)
-            r.group_num_good = _lib.ptr(out["group_num_good"], C.c_int32)
-        if self.flags & _lib.WANT_PER_REQUEST:
-            out["finish"] = np.zeros((L, self.Rmax), np.float64)
-            out["good"] = np.zeros((L, self.Rmax), np.uint8)
-            r.finish = _lib.ptr(out["finish"], C.c_double)
-            r.good = _lib.ptr(out["good"], C.c_uint8)
-        if self.flags & _lib.WANT_OP_COUNT:
-            out["fp_ops"] = np.zeros(L, np.int64)
-            r.fp_ops = _lib.ptr(out["fp_ops"], C.c_int64)
+        out, r = _result_arrays(self.flags, self.n_seeds, self.B, self.M, self.Gmax, self.Rmax)
         _lib.check(self.engine.lib.mmsim_batch_fetch(self._h, C.byref(r)))
-        if "good" in out:
-            out["good"] = out["good"].astype(bool)
-        for k in list(out):
-            if out[k].ndim >= 1 and out[k].shape[0] == L:
-                out[k] = out[k].reshape((self.n_seeds, self.B) + out[k].shape[1:])
-        return out
+        return _shape_results(out, self.n_seeds, self.B)
 
     def close(self):
         if self._h:
