@@ -195,10 +195,11 @@ typedef struct {
     int64_t requests_total;   /* sum of stream lengths over seeds                     */
     int64_t table_bytes;      /* device bytes of the packed placement tables          */
     int64_t stream_bytes;     /* device bytes of the request streams                  */
-    int32_t tile_classes;     /* groups of wavefronts launched with their own LDS size */
-    int32_t segments;         /* launches per class a stream is cut into              */
-    int32_t launches;         /* kernel launches of one mmsim_batch_run               */
-    int32_t reserved;
+    int32_t workgroups;       /* scheduled launch (bursty streams): workgroups, each owning a set of
+                                 (64 placements, stream) items; 0 for the other launches            */
+    int32_t segments;         /* pieces a stream is cut into so that a workgroup's items take turns  */
+    int32_t launches;         /* kernel launches of one mmsim_batch_run                             */
+    int32_t waves_per_group;  /* wavefronts of a workgroup that simulate side by side               */
 } mmsim_batch_info;
 int mmsim_batch_get_info(const mmsim_batch *batch, mmsim_batch_info *out);
 

@@ -88,8 +88,6 @@ struct DevBuf {
 
 }  // namespace
 
-constexpr int kSideStreams = 4;
-
 // Device scratch of mmsim_eval_batch_static: every device table and result buffer of one batch is carved out
 // of this array, so that entry point never allocates.  Each GPU the library runs on holds its own copy at its
 // own address until the process ends; host code only ever uses the address hipGetSymbolAddress returned for
@@ -104,8 +102,6 @@ struct mmsim_ctx {
     hipStream_t stream = nullptr;
     hipDeviceProp_t prop{};
     int max_lds = 0;
-    hipStream_t side[kSideStreams] = {};  // tile classes of one batch run side by side on these
-    hipEvent_t ev_fork = nullptr, ev_join[kSideStreams] = {};
     unsigned char *scratch = nullptr;     // this device's copy of the static scratch (mmsim_eval_batch_static)
     hipEvent_t ev_static[2] = {};         // timing events of batches that live in the static scratch
 };
@@ -146,16 +142,12 @@ struct mmsim_batch {
     std::vector<int64_t> wl_R;                           // [n_seeds] stream lengths
     std::vector<std::vector<int32_t>> wl_model_requests;  // [n_seeds][M] requests per model of each stream
     std::vector<int32_t> pos;  // pos[placement] = tile * 64 + lane it is simulated on
-    // Plain simulator: tiles are grouped into classes by how many clock slots they need; a class is
-    // launched with its own LDS size and as many wavefronts per workgroup as then fit a CU.
-    struct TileClass {
-        int32_t tile0 = 0, tile1 = 0, nslots = 0, wpb = 1;
-        size_t wave_bytes = 0, lds_bytes = 0;
-    };
-    std::vector<TileClass> classes;
-    int32_t nseg = 1;          // streams are simulated in nseg launches per class, state kept in `state`
+    size_t wave_bytes = 0;     // LDS bytes of one wavefront's region (chunked loop, batching simulator)
+    // Plain simulator, loop over runs: one launch of `sched_groups` workgroups, each owning a set of (tile, stream)
+    // items that its wavefronts simulate segment by segment (clocks parked in `state` between segments).
+    int32_t sched_groups = 0, sched_waves = 0, seg_requests = 0, max_nseg = 1;
+    DevBuf<int32_t> plan;      // wg_off | item_tile | item_seed | item_nslots | item_bytes | item_nseg | part_off | part_bytes
     DevBuf<double> state;
-    int32_t launches = 0;      // kernel launches of one run
 
     DevBuf<Req> streams;
     DevBuf<int64_t> stream_off;
@@ -338,9 +330,21 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 lat[(size_t)m * lat_row + lat_off[c] + k] = v;
             }
 
+    // ---- which request loop: bursty streams (most requests repeat the model of the one before) get the loop over runs
+    bool runs = false;
+    if (!batching) {
+        int64_t rep = 0, tot = 0;
+        for (int s = 0; s < n_seeds; ++s) {
+            rep += wls[s]->repeats;
+            tot += wls[s]->R;
+        }
+        runs = 5 * rep > 4 * tot;  // four in five (measured: at three in four the chunked loop is still ahead)
+        if (const char *env = std::getenv("MMSIM_RUNS")) runs = std::atoi(env) != 0;  // tuning knob
+    }
+
     // ---- LDS budget
     const int32_t rmax_lds_bytes = (M + 15) & ~15;
-    size_t wave_bytes = 0, lat_bytes = 0, lds_tail = 0;
+    size_t wave_bytes = 0, lat_bytes = 0, lds_tail = 0, sched_bytes = 0;
     int lat_in_lds = 1;
     int wpb = 0;
     int heap_cap = 0, heap_min = 0, heap_pref = 0;  // batching simulator: event slots per lane (chosen, least, preferred)
@@ -361,7 +365,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     size_t model_lds_bytes = 0;  // per-model counters [M][64] in LDS (decided below)
     bool group_in_lds = (flags & MMSIM_WANT_GROUP_COUNTS) != 0;  // slot owners and group counters in LDS (decided below)
     auto mixed_wave_bytes = [&](int ns) {
-        return ((size_t)mixed_clock_offset(rmax_lds_bytes) + (size_t)(ns + 1) * kSlotBytes +
+        return ((size_t)mixed_clock_offset(rmax_lds_bytes, runs) + (size_t)(ns + 1) * kSlotBytes +
                 (group_in_lds
                      ? (((size_t)ns * kWave + 15) & ~(size_t)15) + (size_t)2 * Gmax * kWave * sizeof(uint32_t)
                      : 0) + model_lds_bytes + 15) & ~(size_t)15;
@@ -369,17 +373,18 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     if (!batching) {
         wave_bytes = mixed_wave_bytes(nslots);  // of the largest placement
         lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
-        if (lat_bytes + wave_bytes > (size_t)ctx->max_lds) {
+        sched_bytes = runs ? (size_t)kSchedLdsBytes : 0;
+        if (lat_bytes + sched_bytes + wave_bytes > (size_t)ctx->max_lds) {
             lat_in_lds = 0;
             lat_bytes = 0;
         }
-        if (wave_bytes > (size_t)ctx->max_lds) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
+        if (sched_bytes + wave_bytes > (size_t)ctx->max_lds) return fail(MMSIM_E_UNSUPPORTED, "per-wavefront state does not fit in LDS (too many stages/groups/models)");
         if ((size_t)ctx->max_lds > (size_t)kRepAddrMask) return fail(MMSIM_E_UNSUPPORTED, "LDS is larger than the descriptor's address field");
         // The walk for power-of-two depths lets every walking lane read as many clock rows as the deepest
         // one (up to 15 past its own group); the rows after the last wavefront's clocks must exist.  If that
         // tail does not fit beside even one wavefront, the general walk is used.
         lds_tail = pow2_depths ? (size_t)(b->smax_bucket - 1) * kSlotBytes : 0;
-        if (lat_bytes + wave_bytes + lds_tail > (size_t)ctx->max_lds) {
+        if (lat_bytes + sched_bytes + wave_bytes + lds_tail > (size_t)ctx->max_lds) {
             lds_tail = 0;
             pow2_depths = false;
         }
@@ -388,7 +393,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         // registers per lane instead and add them to global rows when the lane's group changes; that is used when
         // it gives a CU more wavefronts.  MMSIM_GROUP_COUNTS_LDS=0/1 forces the choice (tuning knob).
         if (group_in_lds && !(flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT))) {
-            const size_t room = (size_t)ctx->max_lds - lat_bytes - lds_tail;
+            const size_t room = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail;
             const size_t with = std::min<size_t>(wpb_cap, room / wave_bytes);
             group_in_lds = false;
             const size_t without = std::min<size_t>(wpb_cap, room / mixed_wave_bytes(nslots));
@@ -401,7 +406,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         // loads wait behind it; counters in LDS do not.  They take M * 256 bytes per wavefront, so they are
         // used when that does not lower the wavefronts a CU gets.
         if (flags & MMSIM_WANT_MODEL_COUNTS) {
-            const size_t room = (size_t)ctx->max_lds - lat_bytes - lds_tail, extra = (size_t)M * kWave * sizeof(uint32_t);
+            const size_t room = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail, extra = (size_t)M * kWave * sizeof(uint32_t);
             const size_t used_now = std::min<size_t>(wpb_cap, room / wave_bytes);
             if (wave_bytes + extra <= room && std::min<size_t>(wpb_cap, room / (wave_bytes + extra)) >= used_now) {
                 model_lds_bytes = extra;
@@ -457,6 +462,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         wpb = (int)std::min<size_t>(kMaxWavesPerBlockBatching, (size_t)ctx->max_lds / wave_bytes);
     }
 
+    std::vector<int32_t> tile_nslots;  // most clock slots of a placement of each tile
     // ---- lane assignment.  A wavefront walks as many pipeline stages as its deepest
     //      lane needs, so placements are ordered by depth before they are cut into
     //      tiles of 64: first by their deepest group, then by the expected depth of a
@@ -481,68 +487,137 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 expected[p] += weight[m] * depth_of[m];
             }
         }
-        // Plain simulator: a placement's clock slots decide how many wavefronts like it fit a CU.
-        // Placements are grouped by that number ("class"), most wavefronts first; a class too small
-        // to fill one tile joins the next one.
-        // By default every placement is treated like the largest one (one class); with
-        // MMSIM_TILE_CLASSES=1 the classes are formed (measured no faster on the mixes tried: the
-        // classes' launches do not pack the chip evenly enough to pay for the smaller ones' gain).
-        const char *tc_env = std::getenv("MMSIM_TILE_CLASSES");
-        const bool by_class = tc_env && std::atoi(tc_env) != 0;
-        std::vector<int32_t> fit(B, 1);
-        if (!batching)
-            for (int32_t p = 0; p < B; ++p) {
-                int32_t f = (int32_t)std::max<size_t>(1, std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes - lds_tail) / mixed_wave_bytes(by_class ? slots_of[p] : nslots)));
-                if (f > 4) f = f == 8 ? 8 : 4;  // beyond one per SIMD only the same number on every SIMD pays
-                fit[p] = f;
-            }
+        // Deepest first: their wavefronts take longest.  The loop over runs sizes a wavefront's LDS region by the
+        // clock slots of its own tile, so there placements with similar slot counts share a tile
+        // (MMSIM_TILE_ORDER=0: by expected depth only, tuning knob).
+        bool by_slots = runs;
+        if (const char *env = std::getenv("MMSIM_TILE_ORDER")) by_slots = runs && std::atoi(env) != 0;
         std::vector<int32_t> order(B);
         for (int32_t p = 0; p < B; ++p) order[p] = p;
         std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
-            if (fit[x] != fit[y]) return fit[x] > fit[y];
-            // deepest first: their wavefronts take longest, so they are launched first and the short ones
-            // fill the CUs as they free up
             if (deepest[x] != deepest[y]) return deepest[x] > deepest[y];
+            if (by_slots && slots_of[x] != slots_of[y]) return slots_of[x] > slots_of[y];
             return expected[x] > expected[y];
         });
+        const int32_t tl = batching ? blanes : kWave;  // placements per tile
         b->pos.assign(B, 0);
-        int32_t tile_at = 0;
-        for (int32_t i = 0; i < B;) {
-            int32_t j = i, f = fit[order[i]];
-            while (j < B && (fit[order[j]] == f || j - i < kWave)) {  // less than a tile: take in the next class
-                f = std::min(f, fit[order[j]]);
-                ++j;
-            }
-            while (j < B && fit[order[j]] >= f) ++j;
-            mmsim_batch::TileClass c;
-            c.tile0 = tile_at;
-            const int32_t tl = batching ? blanes : kWave;  // placements per tile
-            c.tile1 = tile_at + (j - i + tl - 1) / tl;
-            for (int32_t k = i; k < j; ++k) {
-                c.nslots = std::max(c.nslots, slots_of[order[k]]);
-                b->pos[order[k]] = (c.tile0 + (k - i) / tl) * kWave + (k - i) % tl;
-            }
-            if (batching) {
-                c.nslots = nslots;
-                c.wpb = std::min(wpb, c.tile1 - c.tile0);
-                c.wave_bytes = wave_bytes;
-                c.lds_bytes = (size_t)c.wpb * wave_bytes;
-            } else {
-                c.wave_bytes = mixed_wave_bytes(c.nslots);
-                c.wpb = (int32_t)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes - lds_tail) / c.wave_bytes);
-                if (c.wpb > 4) c.wpb = c.wpb == 8 ? 8 : 4;
-                c.wpb = std::min(c.wpb, c.tile1 - c.tile0);
-                c.lds_bytes = lat_bytes + (size_t)c.wpb * c.wave_bytes + lds_tail;
-            }
-            b->classes.push_back(c);
-            tile_at = c.tile1;
-            i = j;
-        }
-        b->tiles = tile_at;
+        b->tiles = (B + tl - 1) / tl;
         b->waves = b->tiles * n_seeds;
-        b->lds_bytes = 0;
-        for (const auto &c : b->classes) b->lds_bytes = std::max(b->lds_bytes, c.lds_bytes);
-        b->waves_per_block = b->classes.front().wpb;
+        tile_nslots.assign(b->tiles, 1);
+        for (int32_t k = 0; k < B; ++k) {
+            b->pos[order[k]] = (k / tl) * kWave + k % tl;
+            tile_nslots[k / tl] = std::max(tile_nslots[k / tl], slots_of[order[k]]);
+        }
+        if (batching) {
+            b->waves_per_block = std::min(wpb, b->tiles);
+            b->wave_bytes = wave_bytes;
+            b->lds_bytes = (size_t)b->waves_per_block * wave_bytes;
+        } else if (!runs) {
+            // chunked loop: every wavefront gets the region of the largest placement; as many wavefronts per
+            // workgroup as fit (beyond one per SIMD only the same number on every SIMD pays)
+            int w = (int)std::min<size_t>(wpb_cap, ((size_t)ctx->max_lds - lat_bytes - lds_tail) / wave_bytes);
+            if (w > 4) w = w == 8 ? 8 : 4;
+            b->waves_per_block = std::max(1, std::min(w, b->tiles));
+            b->wave_bytes = wave_bytes;
+            b->lds_bytes = lat_bytes + (size_t)b->waves_per_block * wave_bytes + lds_tail;
+        }
+    }
+
+    // ---- loop over runs: the schedule.  An item is one (tile, stream) pair; it needs an LDS region as large as its
+    //      tile's clock slots ask for.  Items are dealt to at most one workgroup per CU, tiles staying on one XCD (a
+    //      workgroup goes to XCD blockIdx % 8; the tile's descriptor rows then live in one L2), largest first in
+    //      snake order so that every workgroup gets a similar mix.  A workgroup's LDS is cut into regions sized for
+    //      its largest items, one wavefront per region, as many as fit (up to 8: two per SIMD); its wavefronts then
+    //      take the items in turns, a segment of the stream at a time, always the item that is furthest behind, so
+    //      that all items of a workgroup finish together however many regions there are.
+    std::vector<int32_t> plan;
+    if (!batching && runs) {
+        const size_t cap = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail;
+        struct Item { int32_t tile, seed, bytes; };
+        const int64_t n_items = (int64_t)b->tiles * n_seeds;
+        const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
+        int64_t groups = std::min<int64_t>(cus, n_items);
+        if (const char *env = std::getenv("MMSIM_SCHED_GROUPS")) groups = std::max<int64_t>(1, std::min<int64_t>(n_items, std::atoi(env)));  // tuning knob
+        if (n_items > groups * kMaxGroupItems) return fail(MMSIM_E_UNSUPPORTED, "too many (tile, stream) pairs for one launch; split the batch");
+        std::vector<int32_t> tile_bytes(b->tiles);
+        for (int32_t t2 = 0; t2 < b->tiles; ++t2) tile_bytes[t2] = (int32_t)mixed_wave_bytes(tile_nslots[t2]);
+        std::vector<int32_t> torder(b->tiles);
+        for (int32_t t2 = 0; t2 < b->tiles; ++t2) torder[t2] = t2;
+        std::stable_sort(torder.begin(), torder.end(), [&](int32_t x, int32_t y) { return tile_bytes[x] > tile_bytes[y]; });
+        const int nx = groups >= 8 ? 8 : 1;  // XCDs that get workgroups of their own
+        std::vector<std::vector<Item>> per_xcd(nx);
+        for (int32_t i = 0; i < b->tiles; ++i) {
+            const int r = i % (2 * nx), x = r < nx ? r : 2 * nx - 1 - r;
+            for (int s2 = 0; s2 < n_seeds; ++s2) per_xcd[x].push_back(Item{torder[i], s2, tile_bytes[torder[i]]});
+        }
+        std::vector<std::vector<Item>> per_group((size_t)groups);
+        for (int x = 0; x < nx; ++x) {
+            std::vector<int64_t> mine;  // this XCD's workgroups
+            for (int64_t w = x; w < groups; w += nx) mine.push_back(w);
+            std::stable_sort(per_xcd[x].begin(), per_xcd[x].end(), [](const Item &u, const Item &v) { return u.bytes > v.bytes; });
+            const int64_t gx = (int64_t)mine.size();
+            for (size_t i = 0; i < per_xcd[x].size(); ++i) {
+                const int64_t r = (int64_t)(i % (size_t)(2 * gx)), at = r < gx ? r : 2 * gx - 1 - r;
+                per_group[(size_t)mine[(size_t)at]].push_back(per_xcd[x][i]);
+            }
+        }
+        int max_regions = kMaxWavesPerBlock;
+        if (const char *env = std::getenv("MMSIM_WAVES_PER_CU")) max_regions = std::max(1, std::min(kMaxWavesPerBlock, std::atoi(env)));
+        int64_t seg_requests = 16384;
+        if (const char *env = std::getenv("MMSIM_SEGMENT_REQUESTS")) seg_requests = std::max<int64_t>(kWave, std::atoll(env) & ~(int64_t)(kWave - 1));  // tuning knob
+        std::vector<int32_t> wg_off(groups + 1, 0), part_off((size_t)groups * kMaxWavesPerBlock, -1), part_bytes((size_t)groups * kMaxWavesPerBlock, 0);
+        bool shared = false;  // some workgroup has more items than regions: streams are cut into segments
+        size_t lds_used = 0;
+        int waves_max = 1;
+        for (int64_t w = 0; w < groups; ++w) {
+            const auto &its = per_group[(size_t)w];  // largest first
+            if ((int64_t)its.size() > kMaxGroupItems) return fail(MMSIM_E_UNSUPPORTED, "too many (tile, stream) pairs for one workgroup; split the batch");
+            wg_off[w + 1] = wg_off[w] + (int32_t)its.size();
+            size_t used = 0;
+            int regions = 0;
+            for (size_t i = 0; i < its.size() && regions < max_regions; ++i)
+                if (used + (size_t)its[i].bytes <= cap) {  // an item too large for what is left: smaller ones may still fit
+                    part_off[(size_t)w * kMaxWavesPerBlock + regions] = (int32_t)used;
+                    part_bytes[(size_t)w * kMaxWavesPerBlock + regions] = its[i].bytes;
+                    used += (size_t)its[i].bytes;
+                    ++regions;
+                }
+            if ((int)its.size() > regions) shared = true;
+            lds_used = std::max(lds_used, used);
+            waves_max = std::max(waves_max, regions);
+        }
+        int64_t rmin = b->wl_R.empty() ? 0 : b->wl_R[0];
+        for (int s2 = 0; s2 < n_seeds; ++s2) rmin = std::min(rmin, b->wl_R[(size_t)s2]);
+        if (!shared) seg_requests = 0x7FFFFFC0;  // every item has a wavefront of its own: one segment
+        int32_t max_nseg = 1;
+        const size_t total = (size_t)wg_off[groups];
+        plan.assign((size_t)(groups + 1) + 5 * total + 2 * (size_t)groups * kMaxWavesPerBlock, 0);
+        int32_t *p_off = plan.data(), *p_tile = p_off + groups + 1, *p_seed = p_tile + total, *p_ns = p_seed + total,
+                *p_bytes = p_ns + total, *p_nseg = p_bytes + total, *p_poff = p_nseg + total, *p_pbytes = p_poff + (size_t)groups * kMaxWavesPerBlock;
+        std::copy(wg_off.begin(), wg_off.end(), p_off);
+        for (int64_t w = 0; w < groups; ++w)
+            for (size_t i = 0; i < per_group[(size_t)w].size(); ++i) {
+                const Item &it = per_group[(size_t)w][i];
+                const size_t at = (size_t)wg_off[w] + i;
+                const int64_t Rs = b->wl_R[(size_t)it.seed];
+                const int64_t ns = std::max<int64_t>(1, (Rs + seg_requests - 1) / seg_requests);
+                if (ns > 60000) return fail(MMSIM_E_INVALID, "MMSIM_SEGMENT_REQUESTS is too small for these streams");
+                p_tile[at] = it.tile;
+                p_seed[at] = it.seed;
+                p_ns[at] = tile_nslots[it.tile];
+                p_bytes[at] = it.bytes;
+                p_nseg[at] = (int32_t)ns;
+                max_nseg = std::max(max_nseg, (int32_t)ns);
+            }
+        std::copy(part_off.begin(), part_off.end(), p_poff);
+        std::copy(part_bytes.begin(), part_bytes.end(), p_pbytes);
+        b->sched_groups = (int32_t)groups;
+        b->sched_waves = waves_max;
+        b->seg_requests = (int32_t)seg_requests;
+        b->max_nseg = max_nseg;
+        b->waves_per_block = waves_max;
+        b->wave_bytes = 0;
+        b->lds_bytes = lat_bytes + sched_bytes + lds_used + lds_tail;
     }
 
     // ---- per lane group descriptors [tiles][Gmax+1][64]; row Gmax stays empty
@@ -573,16 +648,13 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
     // LDS byte address of clock slot `slot` of the lane that simulates position `ps` (plain simulator);
     // slot < 0 names the lane's +inf clock.
-    std::vector<uint32_t> tile_clock0(b->tiles, 0);  // address of slot 0, lane 0 of each tile
-    std::vector<int32_t> tile_inf_slot(b->tiles, 0);
-    for (const auto &c : b->classes)
-        for (int32_t tile = c.tile0; tile < c.tile1; ++tile) {
-            tile_clock0[tile] = (uint32_t)(lat_bytes + (size_t)((tile - c.tile0) % c.wpb) * c.wave_bytes + mixed_clock_offset(rmax_lds_bytes));
-            tile_inf_slot[tile] = c.nslots;
-        }
+    // The loop over runs takes addresses relative to the wavefront's clock rows (its LDS region moves from turn to
+    // turn) and sizes the rows by the tile; the chunked loop takes LDS addresses, every region as large as the largest.
     auto clock_addr = [&](int ps, int slot) {
         const int tile = ps / kWave, lane = ps % kWave;
-        return tile_clock0[tile] + (uint32_t)(slot < 0 ? tile_inf_slot[tile] : slot) * kSlotBytes + (uint32_t)lane * (uint32_t)sizeof(double);
+        const uint32_t base = runs ? 0u : (uint32_t)(lat_bytes + (size_t)(tile % b->waves_per_block) * b->wave_bytes + mixed_clock_offset(rmax_lds_bytes, false));
+        const int inf_slot = runs ? tile_nslots[tile] : nslots;
+        return base + (uint32_t)(slot < 0 ? inf_slot : slot) * kSlotBytes + (uint32_t)lane * (uint32_t)sizeof(double);
     };
     if (!batching) {  // missing replicas: the +inf clock and the +inf latency, flagged empty
         const uint32_t inf_lat = (uint32_t)lat_off[C] << 18;
@@ -702,7 +774,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         const size_t lat_b = (lat_nb.size() * sizeof(float) + 15) & ~(size_t)15;
         const size_t g2m_b = ((size_t)(Gmax + 1) * blanes * 2 + (size_t)members_max * blanes * 2 + 15) & ~(size_t)15;
         const size_t cap = (size_t)ctx->max_lds;
-        const int tiles_here = std::max(1, b->classes.front().tile1 - b->classes.front().tile0);
+        const int tiles_here = std::max(1, b->tiles);
         // Fewer event slots (down to G+8) are accepted when that puts more wavefronts on a CU.
         const int wpb_max = kMaxWavesPerBlockBatching;
         const int heap_try_min = std::min(heap_cap, std::max(heap_min, (Gmax + 8 + 7) & ~7));
@@ -732,12 +804,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         wave_bytes = batching_bytes_for(blanes, heap_cap);
         wpb = std::max(1, best_w);
         if (batching_g2m_lds) wave_bytes += g2m_b;
-        mmsim_batch::TileClass &c = b->classes.front();
-        c.wpb = std::min(wpb, c.tile1 - c.tile0);
-        c.wave_bytes = wave_bytes;
-        c.lds_bytes = batching_lat_lds + (size_t)c.wpb * wave_bytes;
-        b->lds_bytes = c.lds_bytes;
-        b->waves_per_block = c.wpb;
+        b->waves_per_block = std::min(wpb, b->tiles);
+        b->wave_bytes = wave_bytes;
+        b->lds_bytes = batching_lat_lds + (size_t)b->waves_per_block * wave_bytes;
     }
 
     // ---- request streams back to back
@@ -775,8 +844,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         HIP_TRY(b->slot_group.alloc(slot_group.size()));
         HIP_TRY(hipMemcpyAsync(b->slot_group.p, slot_group.data(), slot_group.size(), hipMemcpyHostToDevice, st));
     }
-    HIP_TRY(b->kerr.alloc(1));
-    HIP_TRY(hipMemsetAsync(b->kerr.p, 0, sizeof(int32_t), st));
+    HIP_TRY(b->kerr.alloc(32));
+    HIP_TRY(hipMemsetAsync(b->kerr.p, 0, 32 * sizeof(int32_t), st));
     HIP_TRY(b->rmax.alloc(rmax.size()));
     HIP_TRY(hipMemcpyAsync(b->rmax.p, rmax.data(), rmax.size(), hipMemcpyHostToDevice, st));
     HIP_TRY(b->lat.alloc(lat.size()));
@@ -844,32 +913,33 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
     HIP_TRY(hipStreamSynchronize(st));  // host staging vectors go out of scope below
 
-    // ---- segments.  When the workgroups of a run do not all fit on the chip at once, the streams are
-    //      simulated in nseg launches per class (clocks parked in `state` in between), so that classes
-    //      with different workgroup sizes keep every CU busy instead of leaving a ragged last round.
-    //      MMSIM_SEGMENTS overrides the choice (tuning knob).
-    if (!batching) {
-        int64_t blocks = 0, rmin = b->Rmax;
-        for (const auto &c : b->classes) blocks += (int64_t)((c.tile1 - c.tile0 + c.wpb - 1) / c.wpb) * n_seeds;
-        for (int s = 0; s < n_seeds; ++s) rmin = std::min<int64_t>(rmin, wls[s]->R);
-        const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
-        int64_t nseg = 1;
-        if (blocks > cus && b->classes.size() > 1) nseg = std::min<int64_t>(32, (16 * cus + blocks - 1) / blocks);
-        nseg = std::min<int64_t>(nseg, rmin / 4096);  // a segment is at least 4096 requests
-        if (const char *env = std::getenv("MMSIM_SEGMENTS")) nseg = std::min<int64_t>(std::atoi(env), rmin / kWave);
-        nseg = std::max<int64_t>(1, nseg);
-        b->nseg = (int32_t)nseg;
-        if (b->nseg > 1) HIP_TRY(b->state.alloc((size_t)b->waves * nslots * kWave));
+    // ---- loop over runs: the schedule's tables, and room to park clocks between segments
+    if (!plan.empty()) {
+        HIP_TRY(b->plan.alloc(plan.size()));
+        HIP_TRY(hipMemcpy(b->plan.p, plan.data(), sizeof(int32_t) * plan.size(), hipMemcpyHostToDevice));
+        if (b->max_nseg > 1) HIP_TRY(b->state.alloc((size_t)b->waves * nslots * kWave));
     }
 
     MixedArgs &a = b->args;
     a.state = b->state.p;
     a.state_rows = nslots;
     a.slot_rows = nslots;
-    a.seg = 0;
-    a.nseg = b->nseg;
-    a.tile0 = 0;
-    a.tile1 = b->tiles;
+    if (!plan.empty()) {
+        const size_t groups = (size_t)b->sched_groups, total = (size_t)plan[groups];
+        a.wg_off = b->plan.p;
+        a.item_tile = a.wg_off + groups + 1;
+        a.item_seed = a.item_tile + total;
+        a.item_nslots = a.item_seed + total;
+        a.item_bytes = a.item_nslots + total;
+        a.item_nseg = a.item_bytes + total;
+        a.part_off = a.item_nseg + total;
+        a.part_bytes = a.part_off + groups * kMaxWavesPerBlock;
+    }
+    a.sched_groups = b->sched_groups;
+    a.seg_requests = b->seg_requests;
+    a.sched_lds_bytes = (int32_t)sched_bytes;
+    a.sched_spin_limit = 20000;  // waits of 127 x 64 cycles: about 70 ms, several segments
+    if (const char *env = std::getenv("MMSIM_SCHED_SPIN_LIMIT")) a.sched_spin_limit = std::max(0, std::atoi(env));  // tuning knob
     a.streams = b->streams.p;
     a.stream_off = b->stream_off.p;
     a.rep32 = reinterpret_cast<const uint4 *>(b->rep32.p);
@@ -902,15 +972,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.group_global = b->group_global;
     a.slot_cnt = b->slot_cnt.p;
     a.xcd_map = 1;
-    {   // bursty streams (most requests repeat the model of the one before) get the loop over runs
-        int64_t rep = 0, tot = 0;
-        for (int s = 0; s < n_seeds; ++s) {
-            rep += wls[s]->repeats;
-            tot += wls[s]->R;
-        }
-        a.runs = 5 * rep > 4 * tot ? 1 : 0;  // four in five (measured: at three in four the chunked loop is still ahead)
-        if (const char *env = std::getenv("MMSIM_RUNS")) a.runs = std::atoi(env) ? 1 : 0;  // tuning knob
-    }
+    a.runs = runs ? 1 : 0;
     a.skip_ahead = 1;
     if (const char *env = std::getenv("MMSIM_SKIP_AHEAD")) a.skip_ahead = std::atoi(env) ? 1 : 0;  // tuning knob
     if (const char *env = std::getenv("MMSIM_XCD_MAP")) a.xcd_map = std::atoi(env) ? 1 : 0;  // tuning knob
@@ -991,11 +1053,6 @@ int mmsim_ctx_create(int device, mmsim_ctx **out) {
         lds = (int)c->prop.sharedMemPerBlock;
     c->max_lds = lds;
     HIP_TRY(hipStreamCreate(&c->stream));  // default priority, like every stream of the library
-    for (int i = 0; i < kSideStreams; ++i) {
-        HIP_TRY(hipStreamCreate(&c->side[i]));
-        HIP_TRY(hipEventCreateWithFlags(&c->ev_join[i], hipEventDisableTiming));
-    }
-    HIP_TRY(hipEventCreateWithFlags(&c->ev_fork, hipEventDisableTiming));
     HIP_TRY(hipEventCreate(&c->ev_static[0]));
     HIP_TRY(hipEventCreate(&c->ev_static[1]));
     {   // address of this device's copy of the static scratch: once per device, with that device current
@@ -1021,14 +1078,6 @@ void mmsim_ctx_destroy(mmsim_ctx *ctx) {
         (void)hipStreamSynchronize(ctx->stream);
         (void)hipStreamDestroy(ctx->stream);
     }
-    for (int i = 0; i < kSideStreams; ++i) {
-        if (ctx->side[i]) {
-            (void)hipStreamSynchronize(ctx->side[i]);
-            (void)hipStreamDestroy(ctx->side[i]);
-        }
-        if (ctx->ev_join[i]) (void)hipEventDestroy(ctx->ev_join[i]);
-    }
-    if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
     for (hipEvent_t e : ctx->ev_static)
         if (e) (void)hipEventDestroy(e);
     delete ctx;
@@ -1140,38 +1189,14 @@ int mmsim_batch_run(mmsim_batch *b) {
         HIP_TRY(hipMemsetAsync(b->group_req.p, 0, b->group_req.bytes(), ctx->stream));
         HIP_TRY(hipMemsetAsync(b->group_good.p, 0, b->group_good.bytes(), ctx->stream));
     }
+    if (b->sched_groups > 0) HIP_TRY(hipMemsetAsync(b->kerr.p + 1, 0, sizeof(int32_t), ctx->stream));  // items completed
     HIP_TRY(hipEventRecord(b->ev_start, ctx->stream));
     std::string err;
-    b->launches = 0;
     if (b->flags & MMSIM_BATCHING) {
         if (launch_sim_batching(b->bargs, b->waves_per_block, b->lds_bytes, ctx->stream, &err) != hipSuccess) return fail(MMSIM_E_HIP, err);
-        b->launches = 1;
     } else {
-        // One launch per (class, segment).  A single class runs on the context's stream; several
-        // classes run side by side on the side streams, each class in segment order on its own.
-        const int nc = (int)b->classes.size();
-        const int used = nc > 1 ? std::min(nc, kSideStreams) : 0;
-        if (used) {
-            HIP_TRY(hipEventRecord(ctx->ev_fork, ctx->stream));
-            for (int i = 0; i < used; ++i) HIP_TRY(hipStreamWaitEvent(ctx->side[i], ctx->ev_fork, 0));
-        }
-        for (int seg = 0; seg < b->nseg; ++seg)
-            for (int ci = 0; ci < nc; ++ci) {
-                const mmsim_batch::TileClass &c = b->classes[ci];
-                MixedArgs a = b->args;
-                a.tile0 = c.tile0;
-                a.tile1 = c.tile1;
-                a.nslots = c.nslots;
-                a.wave_lds_bytes = (int32_t)c.wave_bytes;
-                a.seg = seg;
-                if (launch_sim_mixed(a, b->smax_bucket, c.wpb, c.lds_bytes, used ? ctx->side[ci % used] : ctx->stream, &err) != hipSuccess)
-                    return fail(MMSIM_E_HIP, err);
-                ++b->launches;
-            }
-        for (int i = 0; i < used; ++i) {
-            HIP_TRY(hipEventRecord(ctx->ev_join[i], ctx->side[i]));
-            HIP_TRY(hipStreamWaitEvent(ctx->stream, ctx->ev_join[i], 0));
-        }
+        if (launch_sim_mixed(b->args, b->smax_bucket, b->waves_per_block, b->lds_bytes, ctx->stream, &err) != hipSuccess)
+            return fail(MMSIM_E_HIP, err);
     }
     HIP_TRY(hipEventRecord(b->ev_stop, ctx->stream));
     b->ran = true;
@@ -1200,9 +1225,14 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
     HIP_TRY(hipStreamSynchronize(b->ctx->stream));
 
     if (!(b->flags & MMSIM_BATCHING)) {
-        int32_t kerr = 0;
-        HIP_TRY(hipMemcpy(&kerr, b->kerr.p, sizeof(int32_t), hipMemcpyDeviceToHost));
-        if (kerr != 0) return fail(MMSIM_E_HIP, "simulation kernel: dynamic LDS does not start at address 0; results are invalid");
+        int32_t kerrs[32] = {};
+        HIP_TRY(hipMemcpy(kerrs, b->kerr.p, sizeof(kerrs), hipMemcpyDeviceToHost));
+        const int32_t kerr = kerrs[0];
+        if (kerr == 1) return fail(MMSIM_E_HIP, "simulation kernel: dynamic LDS does not start at address 0; results are invalid");
+        if (kerr != 0) return fail(MMSIM_E_HIP, "simulation kernel: unexpected error flag; results are invalid");
+        if (b->sched_groups > 0 && kerrs[1] != b->waves)
+            return fail(MMSIM_E_HIP, "simulation kernel: the schedule completed " + std::to_string(kerrs[1]) + " of " +
+                                         std::to_string(b->waves) + " (tile, stream) items; results are invalid");
     }
     const int32_t B = b->B, M = b->M, Gmax = b->Gmax, tiles = b->tiles;
     const size_t lanes_padded = (size_t)b->waves * kWave;
@@ -1325,10 +1355,10 @@ int mmsim_batch_get_info(const mmsim_batch *b, mmsim_batch_info *out) {
     out->table_bytes = (int64_t)(b->rep32.bytes() + b->repx32.bytes() + b->rep8.bytes() + b->repx.bytes() + b->ginfo.bytes() +
                                  b->rmax.bytes() + b->lat.bytes() + b->lat_nb.bytes());
     out->stream_bytes = (int64_t)b->streams.bytes();
-    out->tile_classes = (int32_t)b->classes.size();
-    out->segments = b->nseg;
-    out->launches = (b->flags & MMSIM_BATCHING) ? 1 : (int32_t)b->classes.size() * b->nseg;
-    out->reserved = 0;
+    out->workgroups = b->sched_groups;
+    out->segments = b->max_nseg;
+    out->launches = 1;
+    out->waves_per_group = b->waves_per_block;
     return MMSIM_OK;
 }
 

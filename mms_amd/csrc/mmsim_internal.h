@@ -94,11 +94,24 @@ struct MixedArgs {
     const float *lat;            // [M][lat_row] compact stage latencies (batch size 1)
     int32_t M, lat_row, rep_extra;
     int32_t n_seeds, B, tiles, nslots, Gmax;
-    int32_t tile0, tile1;        // this launch covers tiles [tile0, tile1); nslots and wave_lds_bytes are theirs
-    int32_t seg, nseg;           // this launch covers segment seg of nseg of every stream
     int32_t slot_rows;           // row pitch of slot_group (most slots of any tile)
     int32_t state_rows;          // row pitch of state
-    double *state;               // [waves][state_rows][64] clocks between segments (nseg > 1)
+    double *state;               // [waves][state_rows][64] clocks parked between segments (scheduled launch)
+    // Scheduled launch (loop over runs): workgroup w owns the items wg_off[w] .. wg_off[w+1]-1, an item being one
+    // (tile, stream) pair cut into segments of seg_requests requests; its wavefronts take turns on them.
+    const int32_t *wg_off;       // [workgroups + 1]
+    const int32_t *item_tile;    // [items]
+    const int32_t *item_seed;    // [items]
+    const int32_t *item_nslots;  // [items] clock slots of the item's tile
+    const int32_t *item_bytes;   // [items] LDS bytes a wavefront needs to simulate the item
+    const int32_t *item_nseg;    // [items] segments of the item's stream (at least 1)
+    const int32_t *part_off;     // [workgroups][kMaxWavesPerBlock] byte offset of each wavefront's LDS region behind the
+                                 //   schedule state, -1: that wavefront has none and leaves at once
+    const int32_t *part_bytes;   // [workgroups][kMaxWavesPerBlock] size of that region
+    int32_t sched_groups;        // workgroups of the scheduled launch
+    int32_t seg_requests;        // requests per segment, a multiple of 64
+    int32_t sched_lds_bytes;     // LDS bytes of the schedule state (behind the latency table)
+    int32_t sched_spin_limit;    // a wavefront leaves after waiting this many times in a row for an item to be handed back
     int32_t lat_in_lds;          // 1: the block keeps a copy of lat in LDS
     int32_t uniform_stages;      // 1: all stages of a (model, config) have the same latency; lat is [M][C]
     int32_t pow2_depths;         // 1: every group of the batch has 1, 2, 4, 8 or 16 stages
@@ -133,13 +146,15 @@ struct MixedArgs {
 // LDS layout of the plain simulator, shared by the kernel and by the host code
 // that bakes LDS addresses into the replica descriptors:
 //   [latency table][wavefront 0][wavefront 1]...
-//   wavefront: [64 staged requests][replica bounds u8[M]]
+//   wavefront: [64 staged requests (chunked loop only)][replica bounds u8[M]]
 //              [clocks: nslots+1 rows of 64 f64][slot owners][group counters]
 // Row nslots of the clocks is the +inf row that empty descriptors point at.
 // rmax_lds_bytes is M rounded up to 16.
-__host__ __device__ inline uint32_t mixed_clock_offset(int32_t rmax_lds_bytes) {
-    return (uint32_t)(kStageBytes + rmax_lds_bytes);
+__host__ __device__ inline uint32_t mixed_clock_offset(int32_t rmax_lds_bytes, bool runs) {
+    return (uint32_t)((runs ? 0 : kStageBytes) + rmax_lds_bytes);  // the loop over runs keeps its requests in registers
 }
+constexpr int kMaxGroupItems = 256;   // items one workgroup of a scheduled launch can own
+constexpr int kSchedLdsBytes = 1024;  // LDS reserved for its schedule state
 
 // Arguments of the batching simulation kernel.  Replica lists and group
 // descriptors are shared with the plain kernel; on top come, per seed, the

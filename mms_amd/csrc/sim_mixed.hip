@@ -196,6 +196,14 @@ __device__ __forceinline__ uint32_t pick_desc(const uint4 &a, const uint4 &b) {
     return b.w;
 }
 
+// Schedule state of one workgroup (in LDS behind the latency table): one word per item, twice the segment
+// the item is at, plus one while a wavefront is simulating that segment.  A wavefront takes an item by
+// compare-and-swap on its word and hands it back with a plain atomic store, so there is no lock to hold.
+struct SchedLds {
+    uint32_t item[kMaxGroupItems];
+};
+static_assert(sizeof(SchedLds) <= kSchedLdsBytes, "schedule state outgrew its LDS reservation");
+
 // SMAX: most stages of a group (bucket).  LATLDS: the latency table is kept in LDS.  UNIFORM: one
 // latency per (model, configuration).  POW2: every group has 1, 2, 4, 8 or 16 stages.  OUT: what the
 // request loop produces beyond goodput and latency sum (a.flags says which of it): 0 nothing, 1
@@ -210,53 +218,139 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const int W = (int)(blockDim.x >> 6);
     const int wv = uniform((int)(threadIdx.x >> 6));
     const int lane = (int)(threadIdx.x & 63);
-    const unsigned bq = a.xcd_map ? blockIdx.x >> 3 : blockIdx.x;
-    const int seed = (int)(bq % (unsigned)a.n_seeds);
-    const int tgroup = a.xcd_map ? (int)(bq / (unsigned)a.n_seeds) * 8 + (int)(blockIdx.x & 7u) : (int)(bq / (unsigned)a.n_seeds);
-    const int tile = a.tile0 + tgroup * W + wv;
-    const bool live = tile < a.tile1;
     constexpr bool STATS = OUT > 0;
     const bool want_model = STATS && (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
     const bool want_group = STATS && (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = OUT == 2 && (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const bool want_ops = OUT == 2 && (a.flags & MMSIM_WANT_OP_COUNT) != 0;
     constexpr bool pow2 = POW2;
+    // The loop over runs is launched as a schedule (see the top of the file): its descriptors hold clock
+    // addresses relative to the wavefront's clock rows, wherever in LDS they are this time.
+    constexpr bool SCHED = RUNS;
 
-    // ---- LDS: [latency table][per wavefront: request block | replica bounds | clocks (+inf row last) |
-    //            slot owners | group counters].  The replica descriptors hold byte offsets into lds_raw.
+    // ---- LDS: [latency table][schedule state (SCHED)][per wavefront: request block (chunked loop) | replica
+    //            bounds | clocks (+inf row last) | slot owners | group counters | model counters].
     if (lds_addr(lds_raw) != 0u) {  // the descriptors assume the dynamic LDS starts at address 0
         if (threadIdx.x == 0) *a.error = 1;
         return;
     }
     float *lat_lds = reinterpret_cast<float *>(lds_raw);
     const int lat_floats = LATLDS ? a.M * a.lat_row : 0;
-    unsigned char *mine = lds_raw + a.lat_lds_bytes + wv * a.wave_lds_bytes;
-    uint8_t *rmax_lds = mine + kStageBytes;
-    const uint32_t clk_off = (uint32_t)(a.lat_lds_bytes + wv * a.wave_lds_bytes) + mixed_clock_offset(a.rmax_lds_bytes);
+    for (int i = (int)threadIdx.x; i < lat_floats; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
+
+    // Which (tile, stream) pairs this wavefront simulates, and where its LDS region is.
+    SchedLds *sched = reinterpret_cast<SchedLds *>(lds_raw + a.lat_lds_bytes);
+    int item0 = 0, n_items = 0;      // SCHED: this workgroup's items are item0 .. item0 + n_items - 1
+    int part_off = -1, part_bytes = 0;  // SCHED: this wavefront's LDS region (offset behind the schedule state), -1: none
+    int tile = 0, seed = 0;
+    bool live = true;
+    if constexpr (SCHED) {
+        item0 = a.wg_off[blockIdx.x];
+        n_items = a.wg_off[blockIdx.x + 1] - item0;
+        part_off = a.part_off[(size_t)blockIdx.x * kMaxWavesPerBlock + wv];
+        part_bytes = a.part_bytes[(size_t)blockIdx.x * kMaxWavesPerBlock + wv];
+        for (int k = (int)threadIdx.x; k < n_items; k += (int)blockDim.x) sched->item[k] = 0u;
+        live = wv < kMaxWavesPerBlock && part_off >= 0;
+    } else {
+        const unsigned bq = a.xcd_map ? blockIdx.x >> 3 : blockIdx.x;
+        seed = (int)(bq % (unsigned)a.n_seeds);
+        const int tgroup = a.xcd_map ? (int)(bq / (unsigned)a.n_seeds) * 8 + (int)(blockIdx.x & 7u) : (int)(bq / (unsigned)a.n_seeds);
+        tile = tgroup * W + wv;
+        live = tile < a.tiles;
+    }
+    unsigned char *mine = lds_raw + a.lat_lds_bytes + (SCHED ? a.sched_lds_bytes + part_off : wv * a.wave_lds_bytes);
+    uint8_t *rmax_lds = mine + (RUNS ? 0 : kStageBytes);
+    const uint32_t clk_off = (uint32_t)(mine - lds_raw) + mixed_clock_offset(a.rmax_lds_bytes, RUNS);
     double *clk = reinterpret_cast<double *>(lds_raw + clk_off) + lane;
+    const uint32_t rel_base = SCHED ? clk_off : 0u;  // what turns a descriptor's clock address into an LDS address
     const bool group_regs = want_group && a.group_global != 0;  // counts per lane in registers, flushed to global rows
     const bool group_lds = want_group && !group_regs;
-    const int own_bytes = group_lds ? ((a.nslots * kWave + 15) & ~15) : 0;
-    uint8_t *owner = lds_raw + clk_off + (a.nslots + 1) * kSlotBytes;  // owner[slot * 64 + lane]
-    uint32_t *gcnt = reinterpret_cast<uint32_t *>(owner + own_bytes) + lane;
     const bool model_lds = want_model && a.model_lds != 0;
-    uint32_t *mcnt = gcnt + (group_lds ? 2 * a.Gmax * kWave : 0);  // [M][64] accepted requests per model
-
-    for (int i = (int)threadIdx.x; i < lat_floats; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
-    if (live)
-        for (int i = lane; i < a.M; i += kWave) rmax_lds[i] = a.rmax[(size_t)tile * a.M + i];
+    if constexpr (!SCHED) {
+        if (live)
+            for (int i = lane; i < a.M; i += kWave) rmax_lds[i] = a.rmax[(size_t)tile * a.M + i];
+    }
     __syncthreads();
-    if (!live) return;  // padding wavefront of the last workgroup
+    if (!live) return;  // a wavefront without work: padding of the last workgroup, or no LDS region in this schedule
+
+    const float *lat_base = LATLDS ? lat_lds : a.lat;
+    const double overhead = a.fixed_overhead;
+
+  for (int spins = 0;;) {  // SCHED: one turn per (item, segment) this wavefront is given; otherwise a single turn
+    int seg = 0, item_k = 0;
+    if constexpr (SCHED) {
+        // Take the item of this workgroup that is furthest behind among those that fit this wavefront's LDS
+        // region and that nobody is simulating right now (ties: the largest, so that the large regions serve
+        // the large items).  One lane looks and claims the item with a compare-and-swap; if another
+        // wavefront was faster it looks again.
+        int got = -1;  // -1: nothing left for this wavefront, -2: what is left is being simulated by others right now
+        if (lane == 0) {
+            for (int tries = 0; tries < 64; ++tries) {
+                int best = -1, best_bytes = -1;
+                uint32_t best_word = 0xFFFFFFFFu;
+                bool pending = false;
+                for (int k = 0; k < n_items; ++k) {
+                    const uint32_t w = __hip_atomic_load(&sched->item[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    const int sg = (int)(w >> 1), nsg = a.item_nseg[item0 + k];
+                    const int bytes = a.item_bytes[item0 + k];
+                    if (sg >= nsg || bytes > part_bytes) continue;
+                    if (w & 1u) {  // worth waiting for only if a segment follows the one being simulated
+                        if (sg + 1 < nsg) pending = true;
+                        continue;
+                    }
+                    if (w < best_word || (w == best_word && bytes > best_bytes)) {
+                        best = k;
+                        best_word = w;
+                        best_bytes = bytes;
+                    }
+                }
+                if (best < 0) {
+                    got = pending ? -2 : -1;
+                    break;
+                }
+                uint32_t expect = best_word;
+                if (__hip_atomic_compare_exchange_strong(&sched->item[best], &expect, best_word | 1u, __ATOMIC_ACQUIRE,
+                                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) {
+                    got = best;
+                    break;
+                }
+                got = -2;  // lost the race for that item: look again (or, after many losses, sleep first)
+            }
+        }
+        got = uniform(got);
+        if (got == -1) break;
+        if (got == -2) {
+            // Everything left for this wavefront is in another wavefront's hands.  Wait a little for a segment to
+            // end; a wavefront that has waited long leaves: no item depends on it (an item is either being
+            // simulated or was just handed back by a wavefront that is about to look for work itself).
+            __builtin_amdgcn_s_sleep(127);
+            if (++spins > a.sched_spin_limit) break;
+            continue;
+        }
+        spins = 0;
+        item_k = got;
+        tile = a.item_tile[item0 + item_k];
+        seed = a.item_seed[item0 + item_k];
+        seg = uniform((int)(__hip_atomic_load(&sched->item[item_k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >> 1));
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // the state another wavefront parked for this item
+        for (int i = lane; i < a.M; i += kWave) rmax_lds[i] = a.rmax[(size_t)tile * a.M + i];
+    }
+    const int nslots = SCHED ? a.item_nslots[item0 + item_k] : a.nslots;
+    const int own_bytes = group_lds ? ((nslots * kWave + 15) & ~15) : 0;
+    uint8_t *owner = lds_raw + clk_off + (nslots + 1) * kSlotBytes;  // owner[slot * 64 + lane]
+    uint32_t *gcnt = reinterpret_cast<uint32_t *>(owner + own_bytes) + lane;
+    uint32_t *mcnt = gcnt + (group_lds ? 2 * a.Gmax * kWave : 0);  // [M][64] accepted requests per model
 
     const int wave = seed * a.tiles + tile;
     const size_t out = (size_t)wave * kWave + lane;
     const int64_t off = a.stream_off[seed];
     const int64_t R = a.stream_off[seed + 1] - off;
-    // This launch simulates requests [r0, r1) of the stream: segment a.seg of a.nseg.  Segments other
-    // than the first pick up the lane's state where the previous launch left it.
-    const int64_t r0 = a.seg == 0 ? 0 : ((R * a.seg / a.nseg) & ~(int64_t)(kWave - 1));
-    const int64_t r1 = a.seg == a.nseg - 1 ? R : ((R * (a.seg + 1) / a.nseg) & ~(int64_t)(kWave - 1));
-    const bool resume = a.seg > 0;
+    // This turn simulates requests [r0, r1) of the stream.  Segments other than the first pick up the lane's
+    // state where the wavefront that simulated the segment before parked it.
+    const int64_t r0 = SCHED ? (int64_t)seg * a.seg_requests : 0;
+    const int64_t r1 = SCHED && r0 + a.seg_requests < R ? r0 + a.seg_requests : R;
+    const bool resume = seg > 0;
+    const bool last_seg = r1 >= R;
     double *saved = a.state + (size_t)wave * a.state_rows * kWave + lane;
     int32_t *greq = a.group_req + (size_t)wave * a.Gmax * kWave + lane;
     int32_t *ggood = a.group_good + (size_t)wave * a.Gmax * kWave + lane;
@@ -265,16 +359,16 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     double lat_sum = 0.0;
     int64_t fp_ops = 0;
     if (resume) {
-        for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = saved[(size_t)s * kWave];
+        for (int s = 0; s < nslots; ++s) clk[s * kWave] = saved[(size_t)s * kWave];
         n_good = a.n_good[out];
         lat_sum = a.lat_sum[out];
         if (want_ops) fp_ops = a.fp_ops[out];
     } else {
-        for (int s = 0; s < a.nslots; ++s) clk[s * kWave] = 0.0;
+        for (int s = 0; s < nslots; ++s) clk[s * kWave] = 0.0;
     }
-    clk[a.nslots * kWave] = __builtin_inf();
+    clk[nslots * kWave] = __builtin_inf();
     if (group_lds) {
-        for (int s = 0; s < a.nslots; ++s) owner[s * kWave + lane] = a.slot_group[((size_t)tile * a.slot_rows + s) * kWave + lane];
+        for (int s = 0; s < nslots; ++s) owner[s * kWave + lane] = a.slot_group[((size_t)tile * a.slot_rows + s) * kWave + lane];
         for (int g = 0; g < a.Gmax; ++g) {
             gcnt[g * kWave] = resume ? (uint32_t)greq[g * kWave] : 0u;
             gcnt[(a.Gmax + g) * kWave] = resume ? (uint32_t)ggood[g * kWave] : 0u;
@@ -288,10 +382,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const int4 *__restrict__ reqs4 = reinterpret_cast<const int4 *>(a.streams + off);
     const uint4 *__restrict__ rep_tile = a.rep32 + (size_t)tile * a.M * 2 * kWave + lane;
     const uint32_t *__restrict__ repx_tile = a.repx32 + (size_t)tile * a.M * a.rep_extra * kWave + lane;
-    const float *lat_base = LATLDS ? lat_lds : a.lat;
     double *fin_out = a.finish + (size_t)wave * a.Rmax * kWave + lane;
     uint8_t *good_out = a.good + (size_t)wave * a.Rmax * kWave + lane;
-    const double overhead = a.fixed_overhead;
 
     // the group chosen for the last request, kept while it stays valid (see the request loop)
     int ch_model = -2;        // wave-uniform: model the choice was made for
@@ -339,7 +431,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             static_while<0, nj>([&](auto J) {
                 constexpr int j = decltype(J)::value;
                 k[j].d = pick_desc<j>(da, db);
-                k[j].c = lds_f64(rep_addr(k[j].d));
+                k[j].c = lds_f64(rep_addr(k[j].d) + rel_base);
                 k[j].l = lrow_m[rep_lat_last(k[j].d)];
                 return true;
             });
@@ -364,7 +456,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
                 for (int j = RREG; j < n; ++j) {
                     const uint32_t d = row[(size_t)(j - RREG) * kWave];
-                    win = first_min(win, Cand{lds_f64(rep_addr(d)), d, lrow_m[rep_lat_last(d)]});
+                    win = first_min(win, Cand{lds_f64(rep_addr(d) + rel_base), d, lrow_m[rep_lat_last(d)]});
                 }
             }
             // a clock that is infinite (a group that served a request with infinite latency) is never
@@ -379,7 +471,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         const uint32_t sel = ch_sel;
         const bool has = (int32_t)sel >= 0;
         const int sm1 = has ? (int)rep_stages_m1(sel) : -1;  // stages - 1
-        const uint32_t last_addr = rep_addr(sel);            // the lane's +inf clock when there is no replica
+        const uint32_t last_addr = rep_addr(sel) + rel_base;  // only used when the lane has a replica
         const uint32_t first_addr = last_addr - (uint32_t)(has ? sm1 : 0) * kSlotBytes;
         const float *lrow = lrow_m + (has ? (int)rep_lat_last(sel) - sm1 : 0);
         const double l_last = ch_l_last;
@@ -617,7 +709,7 @@ asm volatile(NAME##_TEXT                                                        
                             if (group_regs) {  // the lane's pending group is the one kept from the request before
                                 if ((int32_t)ch_sel >= 0) pg_req += (uint32_t)passed;
                             } else if (want_group && passed > 0 && (int32_t)ch_sel >= 0) {
-                                const uint32_t g = owner[(rep_addr(ch_sel) - clk_off) >> 3];
+                                const uint32_t g = owner[(rep_addr(ch_sel) + rel_base - clk_off) >> 3];
                                 __hip_atomic_fetch_add(&gcnt[g * kWave], (uint32_t)passed, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_WAVEFRONT);
                             }
@@ -690,8 +782,8 @@ asm volatile(NAME##_TEXT                                                        
     a.n_good[out] = n_good;
     a.lat_sum[out] = lat_sum;
     if (want_ops) a.fp_ops[out] = fp_ops;
-    if (a.seg < a.nseg - 1)
-        for (int s = 0; s < a.nslots; ++s) saved[(size_t)s * kWave] = clk[s * kWave];
+    if (!last_seg)
+        for (int s = 0; s < nslots; ++s) saved[(size_t)s * kWave] = clk[s * kWave];
     if (model_lds)
         for (int m = 0; m < a.M; ++m) model_good[(size_t)m * kWave] = (int32_t)mcnt[m * kWave];
     if (group_regs) flush_group();
@@ -701,6 +793,17 @@ asm volatile(NAME##_TEXT                                                        
             ggood[g * kWave] = (int32_t)gcnt[(a.Gmax + g) * kWave];
         }
     }
+    if constexpr (SCHED) {
+        // hand the item back: its parked state must be visible to whichever wavefront takes its next segment
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        if (lane == 0) {
+            __hip_atomic_store(&sched->item[item_k], (uint32_t)(seg + 1) << 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (last_seg) atomicAdd(a.error + 1, 1);  // items completed: the host checks that none is missing
+        }
+    } else {
+        break;
+    }
+  }
 }
 
 template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT, bool RUNS>
@@ -711,8 +814,14 @@ hipError_t launch_kernel(const MixedArgs &args, int wpb, size_t lds_bytes, hipSt
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return e;
     }
-    const unsigned tile_groups = (unsigned)((args.tile1 - args.tile0 + wpb - 1) / wpb);
-    const dim3 grid((args.xcd_map ? ((tile_groups + 7u) & ~7u) : tile_groups) * (unsigned)args.n_seeds);
+    unsigned blocks;
+    if (RUNS) {
+        blocks = (unsigned)args.sched_groups;
+    } else {
+        const unsigned tile_groups = (unsigned)((args.tiles + wpb - 1) / wpb);
+        blocks = (args.xcd_map ? ((tile_groups + 7u) & ~7u) : tile_groups) * (unsigned)args.n_seeds;
+    }
+    const dim3 grid(blocks);
     hipLaunchKernelGGL(kern, grid, dim3(wpb * kWave), lds_bytes, stream, args);
     return hipGetLastError();
 }

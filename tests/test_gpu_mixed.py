@@ -210,22 +210,28 @@ def test_stage_walk_variants(eng, depths, uniform):
 COUNTS_IN_REGISTERS = -1    # per-model and per-group counts, the latter in registers with adds to global rows
 
 
-@pytest.mark.parametrize("flags", [0, COUNTS_IN_REGISTERS, ALL])
-@pytest.mark.parametrize("segments", [1, 5])
-def test_tile_classes_and_stream_segments(eng, monkeypatch, flags, segments):
-    """Large batches are split into classes of tiles by clock-slot count (each launched with its own
-    LDS size, side by side) and their streams into segments with the clocks parked in between.
-    Forced here on a small batch: 420 placements using 4..56 devices, odd stream length."""
+COUNTS_IN_LDS = -2          # the same counts, per-group counters in LDS
+
+
+@pytest.mark.parametrize("flags", [0, COUNTS_IN_REGISTERS, COUNTS_IN_LDS, ALL])
+@pytest.mark.parametrize("groups,regions,segment", [(1, 1, 64), (3, 2, 256), (5, 8, 512), (64, 8, 16384)])
+def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, groups, regions, segment):
+    """The loop over runs is launched as a schedule: a workgroup owns several (tile, stream) items, its
+    LDS is cut into regions sized by the items' clock slots, and its wavefronts simulate the items a
+    segment at a time, clocks parked in device memory in between.  Forced here on a small batch with
+    few workgroups, few regions and short segments: 420 placements using 4..56 devices (7 tiles of
+    different sizes x 2 streams of odd, unequal lengths), every output level."""
     from types import SimpleNamespace
     from mms_amd.profiling import ParallelConfig
     from mms_amd.placement_policy.base_policy import ModelPlacement
     from mms_amd.profiling import synthetic_profile
-    monkeypatch.setenv("MMSIM_WAVES_PER_CU", "8")
-    monkeypatch.setenv("MMSIM_TILE_CLASSES", "1")
-    monkeypatch.setenv("MMSIM_SEGMENTS", str(segments))
-    if flags == COUNTS_IN_REGISTERS:
+    monkeypatch.setenv("MMSIM_RUNS", "1")
+    monkeypatch.setenv("MMSIM_SCHED_GROUPS", str(groups))
+    monkeypatch.setenv("MMSIM_WAVES_PER_CU", str(regions))
+    monkeypatch.setenv("MMSIM_SEGMENT_REQUESTS", str(segment))
+    if flags in (COUNTS_IN_REGISTERS, COUNTS_IN_LDS):
+        monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", "0" if flags == COUNTS_IN_REGISTERS else "1")
         flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
-        monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", "0")
     traces = bool(flags & _lib.WANT_PER_REQUEST)
     rng = np.random.default_rng(77)
     M, R = 24, 3001
@@ -243,7 +249,8 @@ def test_tile_classes_and_stream_segments(eng, monkeypatch, flags, segments):
     streams = []
     for seed in range(2):
         gaps = rng.exponential(0.01, size=R + seed * 70)
-        streams.append(SimpleNamespace(tstamps=np.cumsum(gaps), model_ids=rng.integers(-1, M, len(gaps)).astype(np.int32),
+        ids = np.repeat(rng.integers(-1, M, len(gaps)), rng.integers(1, 9, len(gaps)))[:len(gaps)]   # bursts of 1..8
+        streams.append(SimpleNamespace(tstamps=np.cumsum(gaps), model_ids=ids.astype(np.int32),
                                        slos=rng.uniform(0.2, 1.0, len(gaps)).astype(np.float32)))
     table = E.LatencyTable(profiles, [1])
     packed = E.pack_placements(sols, table)
@@ -251,8 +258,8 @@ def test_tile_classes_and_stream_segments(eng, monkeypatch, flags, segments):
     batch = E.Batch(eng, dws, table, packed, flags)
     info = batch.info()
     print(info, flush=True)
-    assert info["tile_classes"] >= 2 and info["segments"] == segments
-    assert info["launches"] == info["tile_classes"] * segments
+    assert info["workgroups"] == min(groups, 14) and info["waves_per_group"] <= regions and info["launches"] == 1
+    assert info["segments"] == (-(-(R + 70) // segment) if 14 > info["workgroups"] * info["waves_per_group"] else 1)
     for _ in range(2):                      # a re-run starts from scratch again
         batch.run()
         batch.sync()
@@ -272,7 +279,7 @@ def test_eight_wavefronts_per_workgroup(eng, monkeypatch):
     cfg = make_config(2, 520)
     for flags in (0, ALL):
         out, table, packed, streams, info = _run_config(eng, cfg, cfg.placements, [0, 3], flags)
-        assert info["tile_classes"] == 1 and info["waves"] == 18
+        assert info["waves"] == 18
         for s, st in enumerate(streams):
             ref = oracle_batch(st, table, packed, want_per_request=bool(flags))
             assert_batch_matches(out, ref, s, packed[0], per_request=bool(flags), where=f"8 waves, seed {s}")
