@@ -40,10 +40,12 @@ def narrow(k):
     return f"v_cmpx_le_i32_e32 vcc, {k}, %[walk]"
 
 
-def body(levels, flavour):
+def body(levels, flavour, lean=False):
     a = []
     a.append("s_mov_b64 %[sv], exec")
-    a.append("v_mov_b32_e32 %[acc], 0")
+    a.append("s_mov_b64 %[am], 0")
+    if not lean:
+        a.append("v_mov_b32_e32 %[acc], 0")
     # ---- fetch
     a.append(narrow(0))
     a.append("s_cbranch_execz .Lmmsim_end_%=")
@@ -79,8 +81,10 @@ def body(levels, flavour):
     a.append(narrow(0))
     a.append("v_add_f64 %[lat], %[fin], -%[ts]")
     a.append("v_cmpx_le_f64_e32 vcc, %[lat], %[slo]")
+    a.append("s_mov_b64 %[am], exec")
     a.append("s_cbranch_execz .Lmmsim_end_%=")
-    a.append("v_mov_b32_e32 %[acc], 1")
+    if not lean:
+        a.append("v_mov_b32_e32 %[acc], 1")
     a.append("v_add_u32_e32 %[ng], 1, %[ng]")
     a.append("v_add_f64 %[ls], %[ls], %[lat]")
     # ---- commit
@@ -109,28 +113,32 @@ def pairs(lo, hi):
     return out
 
 
-FT = 250      # v[FT:FT+1]: finish time of a lane that would end at the level just computed
-FSEL = 252    # v[FSEL:FSEL+1]: the lane's own finish time
+FSEL = 252    # v[FSEL:FSEL+1]: the clock of the lane's own last stage
 
 
-def body_pow2_straight(levels, flavour):
+def body_pow2_straight(levels, flavour, lean=False):
     """"P" walks: depths all powers of two.
 
     EXEC is written seven times at most instead of once per phase and exit: which lanes reach depth
     2, 4, 8, 16 is kept as four SGPR masks; the code is straight-line per wave depth D (the deepest
-    walking lane), every walking lane fetches and chains D levels (levels past a lane's own depth read
-    clocks and latencies that are not its group's and compute values nobody uses), the lane's own
-    finish time is selected with the masks, and only the commit narrows EXEC.  LDS reads are waited for
-    one by one, so the chain starts when the first arrives; the finish-time adds and selects sit in the
+    walking lane, tested deepest first: deep walks are the common and the expensive ones), every
+    walking lane fetches and chains D levels (levels past a lane's own depth read clocks and latencies
+    that are not its group's and compute values nobody uses), the clock of the lane's own last stage
+    is selected with the masks, one add gives its finish time, and only the commit narrows EXEC.  LDS
+    reads are waited for one by one, so the chain starts when the first arrives; the selects sit in the
     issue slots the dependent max/add chain leaves empty.
+
+    lean: the variant for callers that only need goodput and latency sums (no per-lane accept flag, no
+    finish time); %[am] always receives the mask of accepting lanes.
     """
     depths = [d for d in (1, 2, 4, 8, 16) if d <= levels]
     masks = {1: "%[m1]", 2: "%[m2]", 4: "%[m4]", 8: "%[m8]"}     # lanes with depth > key
-    fsel = f"v[{FSEL}:{FSEL + 1}]"
-    ft = f"v[{FT}:{FT + 1}]"
+    csel = f"v[{FSEL}:{FSEL + 1}]"
     a = []
     a.append("s_mov_b64 %[sv], exec")
-    a.append("v_mov_b32_e32 %[acc], 0")
+    a.append("s_mov_b64 %[am], 0")
+    if not lean:
+        a.append("v_mov_b32_e32 %[acc], 0")
     a.append(narrow(0))
     a.append("s_cbranch_execz .Lmmsim_end_%=")
     for e in depths[:-1]:
@@ -138,10 +146,10 @@ def body_pow2_straight(levels, flavour):
     a.append(f"ds_read_b64 {creg(0)}, %[cb]")
     if flavour == "N":
         a.append(f"ds_read_b32 v{L0}, %[lb]")
-    for e in depths[:-1]:                       # the wave's depth is the first e nobody goes beyond
-        a.append(f"s_cmp_eq_u64 {masks[e]}, 0")
-        a.append(f"s_cbranch_scc1 .Lmmsim_d{e}_%=")
-    for D in reversed(depths):                  # deepest first: falls through from the dispatch
+    for e in reversed(depths[:-1]):             # the wave's depth is 2e for the largest e somebody goes beyond
+        a.append(f"s_cmp_lg_u64 {masks[e]}, 0")
+        a.append(f"s_cbranch_scc1 .Lmmsim_d{2 * e}_%=")
+    for D in depths:                            # shallowest first: depth 1 falls through from the dispatch
         a.append(f".Lmmsim_d{D}_%=:")
         # reads in issue order, each with the levels it brings (clock k: ("c", k), latency k: ("l", k))
         issued = [[("c", 0)]] + ([[("l", 0)]] if flavour == "N" else [])
@@ -177,27 +185,26 @@ def body_pow2_straight(levels, flavour):
             a.append(f"v_add_f64 {creg(k)}, {creg(k)}, " + (f"v[{TMP}:{TMP + 1}]" if flavour == "N" else "%[lc]"))
             if fill:
                 a.append(fill.pop(0))
-            if k + 1 in depths:                 # a lane of depth k+1 finishes here
-                a.extend(fill)                  # the shared temporary is reused: flush what still reads it
-                fill = []
+            if k + 1 in depths and k + 1 > 1:   # a lane of depth k+1 ends here: its last-stage clock is c[k]
                 i = depths.index(k + 1)
-                if i == 0:
-                    fill.append(f"v_add_f64 {fsel}, {creg(k)}, %[oh]")
-                else:
-                    m = masks[depths[i - 1]]
-                    fill.append(f"v_add_f64 {ft}, {creg(k)}, %[oh]")
-                    fill.append(f"v_cndmask_b32_e64 v{FSEL}, v{FSEL}, v{FT}, {m}")
-                    fill.append(f"v_cndmask_b32_e64 v{FSEL + 1}, v{FSEL + 1}, v{FT + 1}, {m}")
+                m = masks[depths[i - 1]]
+                src = creg(0) if i == 1 else csel        # depth-1 lanes end at c[0]
+                lo, hi = (C0, C0 + 1) if i == 1 else (FSEL, FSEL + 1)
+                fill.append(f"v_cndmask_b32_e64 v{FSEL}, v{lo}, v{C0 + 2 * k}, {m}")
+                fill.append(f"v_cndmask_b32_e64 v{FSEL + 1}, v{hi}, v{C0 + 2 * k + 1}, {m}")
         a.extend(fill)
-        a.append(f"v_add_f64 %[lat], {fsel}, -%[ts]")
-        a.append(f"v_mov_b64_e32 %[fin], {fsel}")
-        if D != depths[0]:
+        last = creg(0) if D == 1 else csel
+        a.append(f"v_add_f64 %[fin], {last}, %[oh]")      # :610
+        a.append("v_add_f64 %[lat], %[fin], -%[ts]")
+        if D != depths[-1]:
             a.append("s_branch .Lmmsim_decide_%=")
     # ---- decide
     a.append(".Lmmsim_decide_%=:")
     a.append("v_cmpx_le_f64_e32 vcc, %[lat], %[slo]")
+    a.append("s_mov_b64 %[am], exec")
     a.append("s_cbranch_execz .Lmmsim_end_%=")
-    a.append("v_mov_b32_e32 %[acc], 1")
+    if not lean:
+        a.append("v_mov_b32_e32 %[acc], 1")
     a.append("v_add_u32_e32 %[ng], 1, %[ng]")
     a.append("v_add_f64 %[ls], %[ls], %[lat]")
     # ---- commit: accepted lanes, each its own depth
@@ -228,18 +235,19 @@ def main():
            "// Stage walk of the plain simulator as one inline-asm block per request.", ""]
     for levels in (4, 16):
         for flavour in ("U", "N", "PU", "PN"):
-            name = f"MMSIM_WALK_{flavour}{levels}"
-            straight = flavour[0] == "P"
-            flavour = flavour[-1]
-            lines = body_pow2_straight(levels, flavour) if straight else body(levels, flavour)
-            out.append(f"#define {name}_TEXT \\")
-            out.extend(f'    "{l}\\n" \\' for l in lines[:-1])
-            out.append(f'    "{lines[-1]}\\n"')
-            regs = clobbers(levels, flavour)
-            if straight:
-                regs += [f"v{FT}", f"v{FT + 1}", f"v{FSEL}", f"v{FSEL + 1}"]
-            out.append(f"#define {name}_CLOBBERS " + ", ".join(f'"{r}"' for r in regs))
-            out.append("")
+            for lean in (False, True):
+                name = f"MMSIM_WALK_{flavour}{levels}" + ("_LEAN" if lean else "")
+                straight = flavour[0] == "P"
+                fl = flavour[-1]
+                lines = body_pow2_straight(levels, fl, lean) if straight else body(levels, fl, lean)
+                out.append(f"#define {name}_TEXT \\")
+                out.extend(f'    "{l}\\n" \\' for l in lines[:-1])
+                out.append(f'    "{lines[-1]}\\n"')
+                regs = clobbers(levels, fl)
+                if straight:
+                    regs += [f"v{FSEL}", f"v{FSEL + 1}"]
+                out.append(f"#define {name}_CLOBBERS " + ", ".join(f'"{r}"' for r in regs))
+                out.append("")
     with open(os.path.join(here, "walk_asm.inc"), "w") as f:
         f.write("\n".join(out))
     print("wrote walk_asm.inc")

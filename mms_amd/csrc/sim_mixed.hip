@@ -102,23 +102,27 @@ __device__ __forceinline__ double vmin(double x, double y) {
     return r;
 }
 
-// Smallest value of x over the 64 lanes (never NaN), the same in every lane: butterflies inside rows of
-// 16 lanes (DPP), then the four row results through scalar registers.  All lanes must be active.
-template <int CTRL>
-__device__ __forceinline__ double dpp_f64(double x) {
-    const int lo = __builtin_amdgcn_update_dpp(__double2loint(x), __double2loint(x), CTRL, 0xF, 0xF, false);
-    const int hi = __builtin_amdgcn_update_dpp(__double2hiint(x), __double2hiint(x), CTRL, 0xF, 0xF, false);
-    return __hiloint2double(hi, lo);
-}
-__device__ __forceinline__ double lane_f64(double x, int l) {
-    return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(x), l), __builtin_amdgcn_readlane(__double2loint(x), l));
-}
-__device__ __forceinline__ double wave_min(double x) {
-    x = vmin(x, dpp_f64<0xB1>(x));   // quad_perm [1,0,3,2]
-    x = vmin(x, dpp_f64<0x4E>(x));   // quad_perm [2,3,0,1]
-    x = vmin(x, dpp_f64<0x141>(x));  // row_half_mirror
-    x = vmin(x, dpp_f64<0x140>(x));  // row_mirror
-    return vmin(vmin(lane_f64(x, 0), lane_f64(x, 16)), vmin(lane_f64(x, 32), lane_f64(x, 48)));
+// Smallest values of x and of y over the 64 lanes, as scalars: butterflies inside rows of 16 lanes, then the
+// row results carried to the last lane (row_bcast15 into rows 1 and 3, row_bcast31 into rows 2 and 3).
+// One DPP instruction per step and value: v_min_u32_dpp d, d, d = min(d of the lane the pattern names, d),
+// lanes the row mask leaves out keep d.  A DPP operand needs two wait states after the write of its
+// register; the two independent chains and one s_nop give them.  All lanes must be active.
+__device__ __forceinline__ void wave_min2_u32(uint32_t &x, uint32_t &y) {
+#define MMSIM_MIN_STEP(PATTERN)                         \
+    "s_nop 1\n"                                         \
+    "v_min_u32_dpp %0, %0, %0 " PATTERN " bank_mask:0xf\n" \
+    "v_min_u32_dpp %1, %1, %1 " PATTERN " bank_mask:0xf\n"
+    asm volatile(MMSIM_MIN_STEP("quad_perm:[1,0,3,2] row_mask:0xf")
+                 MMSIM_MIN_STEP("quad_perm:[2,3,0,1] row_mask:0xf")
+                 MMSIM_MIN_STEP("row_half_mirror row_mask:0xf")
+                 MMSIM_MIN_STEP("row_mirror row_mask:0xf")
+                 MMSIM_MIN_STEP("row_bcast:15 row_mask:0xa")
+                 MMSIM_MIN_STEP("row_bcast:31 row_mask:0xc")
+                 "s_nop 1\n"
+                 : "+v"(x), "+v"(y));
+#undef MMSIM_MIN_STEP
+    x = (uint32_t)__builtin_amdgcn_readlane((int)x, 63);
+    y = (uint32_t)__builtin_amdgcn_readlane((int)y, 63);
 }
 
 // LDS accesses by byte address (the replica descriptors carry addresses, not pointers).
@@ -388,8 +392,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     // the group chosen for the last request, kept while it stays valid (see the request loop)
     int ch_model = -2;        // wave-uniform: model the choice was made for
     bool ch_stale = true;     // wave-uniform: some lane accepted a request since
-    double ch_best = __builtin_inf(), ch_l_last = 0.0;
-    uint32_t ch_sel = kEmpty;
+    double ch_best = __builtin_inf(), ch_l_last = 0.0;  // its last-stage clock and the model's last-stage latency there
+    int ch_sm1 = -1;          // its stages - 1, or -1: the lane has no replica to send the request to
+    uint32_t ch_last = 0, ch_first = 0;  // LDS addresses of its last and first stage clocks
+    int ch_lrow = 0;          // where its stage latencies start in the model's row of the latency table
     constexpr bool SKIP = RUNS && OUT <= 1;  // per-request outputs and operation counts need every request
     bool ch_looked = false;   // wave-uniform: the block has been searched for requests that the current choice rejects
     uint64_t skip = 0;        // wave-uniform: requests of the block that every lane rejects while nobody accepts
@@ -407,7 +413,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
 
     // One request for the whole wavefront: `at` is its place in the stream, m / n the model and the tile's
     // replica bound for it (wave-uniform), da / db this lane's descriptors of the model's replicas.
-    auto simulate = [&](int64_t at, int m, int n, const uint4 &da, const uint4 &db, double tstamp, double slo) {
+    auto simulate = [&](int64_t at, int m, int n, const uint4 &da, const uint4 &db, double tstamp, double slo) -> uint64_t {
         const float *lrow_m = lat_base + (size_t)(m < 0 ? 0 : m) * a.lat_row;
 
         // ---- choose the replica group: strictly smallest last-stage clock (:590-598).
@@ -464,20 +470,28 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             ch_model = m;
             ch_looked = false;
             ch_best = win.c;
-            ch_sel = win.c < 1e100 ? win.d : kEmpty;
             ch_l_last = (double)win.l;
+            // what the walk needs of the chosen group, worked out once per choice
+            const bool found = (int32_t)win.d >= 0 && win.c < 1e100;
+            const int stages_m1 = (int)rep_stages_m1(win.d);
+            ch_sm1 = found ? stages_m1 : -1;
+            ch_last = rep_addr(win.d) + rel_base;
+            ch_first = ch_last - (uint32_t)(found ? stages_m1 : 0) * kSlotBytes;
+            ch_lrow = found ? (int)rep_lat_last(win.d) - stages_m1 : 0;
         }
         const double best = ch_best;
-        const uint32_t sel = ch_sel;
-        const bool has = (int32_t)sel >= 0;
-        const int sm1 = has ? (int)rep_stages_m1(sel) : -1;  // stages - 1
-        const uint32_t last_addr = rep_addr(sel) + rel_base;  // only used when the lane has a replica
-        const uint32_t first_addr = last_addr - (uint32_t)(has ? sm1 : 0) * kSlotBytes;
-        const float *lrow = lrow_m + (has ? (int)rep_lat_last(sel) - sm1 : 0);
+        const bool has = ch_sm1 >= 0;
+        const int sm1 = ch_sm1;
+        const uint32_t last_addr = ch_last;    // only used when the lane has a replica
+        const uint32_t first_addr = ch_first;
+        const float *lrow = lrow_m + ch_lrow;
         const double l_last = ch_l_last;
 
         double finish_time;
-        bool acc;
+        bool acc = false;
+        uint64_t acc_mask = 0;  // wave-uniform: lanes that accepted the request
+        constexpr bool LEAN = OUT == 0;  // scores only: nobody asks which lane accepted or when it finished
+        bool asm_walk = false;
         if constexpr (SMAX == 1) {
             // ---- single-stage groups: the clock read for the choice is the whole pipeline (:605-619)
             const double t = vmax(tstamp, best) + l_last;
@@ -492,7 +506,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         } else {
             // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
             const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
-            const int walk = (int)(has & !(bound > slo)) != 0 ? sm1 : -1;  // stages - 1 of lanes that walk (no per-lane branch)
+            const int walk = !(bound > slo) ? sm1 : -1;  // stages - 1 of lanes that walk (no per-lane branch; -1 without a replica)
             if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
                 // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
                 uint64_t saved_exec, mask1, mask2, mask4, mask8;  // masks: scratch of the power-of-two walk
@@ -503,38 +517,47 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
 asm volatile(NAME##_TEXT                                                                                        \
      : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [fin] "=&v"(finish_time), [lat] "=&v"(latency),   \
        [ng] "+v"(n_good), [ls] "+v"(lat_sum), [m1] "=&s"(mask1), [m2] "=&s"(mask2), [m4] "=&s"(mask4),  \
-       [m8] "=&s"(mask8)                                                                                \
+       [m8] "=&s"(mask8), [am] "=&s"(acc_mask)                                                          \
      : [walk] "v"(walk), [cb] "v"(cb_addr), [LATNAME] "v"(LATVAL), [ts] "v"(tstamp), [slo] "v"(slo),    \
        [oh] "s"(overhead)                                                                               \
      : "vcc", "scc", "memory", NAME##_CLOBBERS)
+#define MMSIM_WALK_PICK(NAME, LATNAME, LATVAL)                 \
+    do {                                                       \
+        if constexpr (LEAN)                                    \
+            MMSIM_WALK(NAME##_LEAN, LATNAME, LATVAL);          \
+        else                                                   \
+            MMSIM_WALK(NAME, LATNAME, LATVAL);                 \
+    } while (0)
                 if constexpr (UNIFORM) {
                     if (pow2) {
                         if constexpr (SMAX == 4)
-                            MMSIM_WALK(MMSIM_WALK_PU4, lc, l_last);
+                            MMSIM_WALK_PICK(MMSIM_WALK_PU4, lc, l_last);
                         else
-                            MMSIM_WALK(MMSIM_WALK_PU16, lc, l_last);
+                            MMSIM_WALK_PICK(MMSIM_WALK_PU16, lc, l_last);
                     } else {
                         if constexpr (SMAX == 4)
-                            MMSIM_WALK(MMSIM_WALK_U4, lc, l_last);
+                            MMSIM_WALK_PICK(MMSIM_WALK_U4, lc, l_last);
                         else
-                            MMSIM_WALK(MMSIM_WALK_U16, lc, l_last);
+                            MMSIM_WALK_PICK(MMSIM_WALK_U16, lc, l_last);
                     }
                 } else {
                     const uint32_t lb = lds_addr(lrow);
                     if (pow2) {
                         if constexpr (SMAX == 4)
-                            MMSIM_WALK(MMSIM_WALK_PN4, lb, lb);
+                            MMSIM_WALK_PICK(MMSIM_WALK_PN4, lb, lb);
                         else
-                            MMSIM_WALK(MMSIM_WALK_PN16, lb, lb);
+                            MMSIM_WALK_PICK(MMSIM_WALK_PN16, lb, lb);
                     } else {
                         if constexpr (SMAX == 4)
-                            MMSIM_WALK(MMSIM_WALK_N4, lb, lb);
+                            MMSIM_WALK_PICK(MMSIM_WALK_N4, lb, lb);
                         else
-                            MMSIM_WALK(MMSIM_WALK_N16, lb, lb);
+                            MMSIM_WALK_PICK(MMSIM_WALK_N16, lb, lb);
                     }
                 }
+#undef MMSIM_WALK_PICK
 #undef MMSIM_WALK
-                acc = accepted != 0;
+                if constexpr (!LEAN) acc = accepted != 0;
+                asm_walk = true;
             } else {
                 // ---- the same in plain C++ (other stage buckets, latency table in global memory):
                 //      fetch, then the dependent chain (:605-608)
@@ -573,8 +596,8 @@ asm volatile(NAME##_TEXT                                                        
             }
         }
         if constexpr (RUNS) {
-            ch_stale = __ballot(acc) != 0ull;
-            if (ch_stale) skip = 0;
+            if (!asm_walk) acc_mask = __ballot(acc);
+            ch_stale = acc_mask != 0ull;
         }
         if (group_regs) {  // :611, :618
             const uint32_t now = has ? last_addr : 0xFFFFFFFFu;
@@ -617,6 +640,7 @@ asm volatile(NAME##_TEXT                                                        
             fin_out[at * kWave] = acc ? finish_time : tstamp;
             good_out[at * kWave] = acc ? 1 : 0;
         }
+        return acc_mask;
     };
 
     int4 ahead = make_int4(0, 0, -1, 0);  // this lane's request of the next block
@@ -677,43 +701,55 @@ asm volatile(NAME##_TEXT                                                        
                 const uint64_t run = (s1 >= 64 ? ~0ull : ((1ull << s1) - 1ull)) & (~0ull << s0) & valid;
 
                 auto request = [&](int i) {
-                    simulate(blk + i, m, n, da, db,
-                             __hiloint2double(__builtin_amdgcn_readlane(r.y, i), __builtin_amdgcn_readlane(r.x, i)),
-                             (double)__int_as_float(__builtin_amdgcn_readlane(r.w, i)));
+                    return simulate(blk + i, m, n, da, db,
+                                    __hiloint2double(__builtin_amdgcn_readlane(r.y, i), __builtin_amdgcn_readlane(r.x, i)),
+                                    (double)__int_as_float(__builtin_amdgcn_readlane(r.w, i)));
                 };
 
                 if constexpr (SKIP) {
-                    for (int i = s0; i < s1;) {
-                        request(i);
+                    uint64_t later = run & (~1ull << s0);  // requests of the run that follow the one being simulated
+                    for (int i = s0;;) {
+                        const uint64_t accepted = request(i);
                         // Nobody accepted: until somebody does, a request of this model is rejected by every lane
                         // (before any walk) if  fl(fl(fl(max(t, best) + l_last) + overhead) - t) > slo  in every
                         // lane.  For t <= best in every lane the left side is fl(C - t) with
-                        // C = fl(fl(best + l_last) + overhead), and rounding is monotone, so the smallest C of
-                        // the wavefront decides for all lanes at once: lane j tests request j of the block, and
-                        // the requests found are not simulated: a rejected request changes nothing and counts
-                        // only as a request of the group its lane would have chosen (:611), which is the group
-                        // kept from the request before.
-                        if (a.skip_ahead && !ch_stale && !ch_looked && i + 1 < s1) {
+                        // C = fl(fl(best + l_last) + overhead), and rounding is monotone, so any lower bound of
+                        // the smallest C of the wavefront decides for all lanes at once (and any lower bound of
+                        // the smallest best guards t <= best): the bounds are the smallest high words over the
+                        // lanes, low words zero (non-negative doubles order like their high words).  Lane j
+                        // tests request j of the block, and the requests found are not simulated: a rejected
+                        // request changes nothing and counts only as a request of the group its lane would
+                        // have chosen (:611), which is the group kept from the request before.
+                        if (accepted) {
+                            skip = 0;
+                        } else if (a.skip_ahead && !ch_looked && later) {
                             ch_looked = true;
-                            const bool chosen = (int32_t)ch_sel >= 0;
-                            const double cmin = wave_min(chosen ? (ch_best + ch_l_last) + overhead : __builtin_inf());
-                            const double bmin = wave_min(chosen ? ch_best : __builtin_inf());
+                            const bool chosen = ch_sm1 >= 0;
+                            const uint32_t none = 0x7FF00000u;  // high word of +inf
+                            uint32_t chi = chosen ? (uint32_t)__double2hiint((ch_best + ch_l_last) + overhead) : none;
+                            uint32_t bhi = chosen ? (uint32_t)__double2hiint(ch_best) : none;
+                            wave_min2_u32(chi, bhi);
+                            const double clow = __hiloint2double((int)chi, 0);
+                            const double blow = __hiloint2double((int)bhi, 0);
                             const double tj = __hiloint2double(r.y, r.x);
-                            const bool rejected = r.z == w && tj <= bmin && (cmin - tj) > (double)__int_as_float(r.w);
+                            const bool rejected = r.z == w && tj <= blow && (clow - tj) > (double)__int_as_float(r.w);
                             skip |= __ballot(rejected);
                         }
-                        const uint64_t todo = run & ~skip & (i >= 63 ? 0ull : (~0ull << (i + 1)));
-                        const int next = todo ? (int)__builtin_ctzll(todo) : s1;
+                        const uint64_t todo = later & ~skip;
+                        const int next = todo ? (int)__builtin_ctzll(todo) : 64;
                         if constexpr (OUT == 1) {
-                            const int passed = next - (i + 1);  // requests of the run that are not simulated
+                            // requests of the run that are passed over for good
+                            const int passed = __builtin_popcountll(next < 64 ? later & ~(~0ull << next) : later);
                             if (group_regs) {  // the lane's pending group is the one kept from the request before
-                                if ((int32_t)ch_sel >= 0) pg_req += (uint32_t)passed;
-                            } else if (want_group && passed > 0 && (int32_t)ch_sel >= 0) {
-                                const uint32_t g = owner[(rep_addr(ch_sel) + rel_base - clk_off) >> 3];
+                                if (ch_sm1 >= 0) pg_req += (uint32_t)passed;
+                            } else if (want_group && passed > 0 && ch_sm1 >= 0) {
+                                const uint32_t g = owner[(ch_last - clk_off) >> 3];
                                 __hip_atomic_fetch_add(&gcnt[g * kWave], (uint32_t)passed, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_WAVEFRONT);
                             }
                         }
+                        if (!todo) break;
+                        later &= ~1ull << next;
                         i = next;
                     }
                 } else {
