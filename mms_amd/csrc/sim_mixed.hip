@@ -211,8 +211,9 @@ static_assert(sizeof(SchedLds) <= kSchedLdsBytes, "schedule state outgrew its LD
 // SMAX: most stages of a group (bucket).  LATLDS: the latency table is kept in LDS.  UNIFORM: one
 // latency per (model, configuration).  POW2: every group has 1, 2, 4, 8 or 16 stages.  OUT: what the
 // request loop produces beyond goodput and latency sum (a.flags says which of it): 0 nothing, 1
-// per-model / per-group counts, 2 also per-request results and operation counts; a level's loop
-// carries no trace of the higher levels' outputs.  RUNS: the loop walks runs of equal models (bursty
+// per-model / per-group counts kept in registers and global rows, 2 the same counts kept in LDS (small
+// batches), 3 also per-request results and operation counts; a level's loop carries no trace of the
+// higher levels' outputs.  RUNS: the loop walks runs of equal models (bursty
 // streams) instead of fixed chunks of four requests.
 template <int SMAX, bool LATLDS, bool UNIFORM, bool POW2, int OUT, bool RUNS>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(const MixedArgs a) {
@@ -225,8 +226,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     constexpr bool STATS = OUT > 0;
     const bool want_model = STATS && (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
     const bool want_group = STATS && (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
-    const bool want_req = OUT == 2 && (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
-    const bool want_ops = OUT == 2 && (a.flags & MMSIM_WANT_OP_COUNT) != 0;
+    const bool want_req = OUT == 3 && (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
+    const bool want_ops = OUT == 3 && (a.flags & MMSIM_WANT_OP_COUNT) != 0;
     constexpr bool pow2 = POW2;
     // The loop over runs is launched as a schedule (see the top of the file): its descriptors hold clock
     // addresses relative to the wavefront's clock rows, wherever in LDS they are this time.
@@ -267,9 +268,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const uint32_t clk_off = (uint32_t)(mine - lds_raw) + mixed_clock_offset(a.rmax_lds_bytes, RUNS);
     double *clk = reinterpret_cast<double *>(lds_raw + clk_off) + lane;
     const uint32_t rel_base = SCHED ? clk_off : 0u;  // what turns a descriptor's clock address into an LDS address
-    const bool group_regs = want_group && a.group_global != 0;  // counts per lane in registers, flushed to global rows
-    const bool group_lds = want_group && !group_regs;
-    const bool model_lds = want_model && a.model_lds != 0;
+    // Counter homes: output level 1 keeps no counters in LDS (its request loop carries no code for them)
+    const bool group_regs = want_group && (OUT == 1 || a.group_global != 0);  // counts per lane in registers, flushed to global rows
+    const bool group_lds = OUT >= 2 && want_group && !group_regs;
+    const bool model_lds = OUT >= 2 && want_model && a.model_lds != 0;
     if constexpr (!SCHED) {
         if (live)
             for (int i = lane; i < a.M; i += kWave) rmax_lds[i] = a.rmax[(size_t)tile * a.M + i];
@@ -396,20 +398,29 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     int ch_sm1 = -1;          // its stages - 1, or -1: the lane has no replica to send the request to
     uint32_t ch_last = 0, ch_first = 0;  // LDS addresses of its last and first stage clocks
     int ch_lrow = 0;          // where its stage latencies start in the model's row of the latency table
-    constexpr bool SKIP = RUNS && OUT <= 1;  // per-request outputs and operation counts need every request
+    constexpr bool SKIP = RUNS && OUT <= 2;  // per-request outputs and operation counts need every request
     bool ch_looked = false;   // wave-uniform: the block has been searched for requests that the current choice rejects
     uint64_t skip = 0;        // wave-uniform: requests of the block that every lane rejects while nobody accepts
 
-    // Per-group counts without LDS (group_regs): a lane's group changes about once per run of equal models, so the
-    // lane counts in registers and adds them to the global row of the group's last clock slot only when its group
-    // changes (relaxed adds that nobody waits for; every counter has one owner).
-    uint32_t pg_addr = 0xFFFFFFFFu, pg_req = 0, pg_good = 0;  // LDS address of the group's last-stage clock, or none
+    // Per-group counts without LDS (group_regs).  A lane's group changes only when the choice is made anew, and
+    // between two choices every request the wavefront handles (simulated or passed over) goes to that group, so a
+    // lane keeps, for its current group, how many requests of this turn had been handled (the request's place in the
+    // stream, wave-uniform) and where its own count of accepted requests stood when it chose the group, and adds
+    // the differences to the global row of the group's last
+    // clock slot when its group changes (one 64-bit relaxed add, requests in the low half, accepted requests in the
+    // high half; nobody waits for it; every counter has one owner).
+    uint32_t pg_addr = 0xFFFFFFFFu, pg_req0 = 0;  // LDS address of the group's last-stage clock (or none); requests handled then
+    int32_t pg_good0 = 0;                         // n_good then
     unsigned long long *slot_cnt = a.slot_cnt + (size_t)wave * a.slot_rows * kWave;
-    auto flush_group = [&]() {
-        if (pg_addr != 0xFFFFFFFFu && pg_req != 0)  // one 64-bit add: requests in the low half, accepted ones in the high half
-            __hip_atomic_fetch_add(&slot_cnt[(pg_addr - clk_off) >> 3], ((unsigned long long)pg_good << 32) | pg_req,
+    auto flush_group = [&](uint32_t handled) {  // handled: requests of this turn handled so far (wave-uniform)
+        const uint32_t reqs = handled - pg_req0, goods = (uint32_t)(n_good - pg_good0);
+        if (pg_addr != 0xFFFFFFFFu && reqs != 0)
+            __hip_atomic_fetch_add(&slot_cnt[(pg_addr - clk_off) >> 3], ((unsigned long long)goods << 32) | reqs,
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
+    // Per-model counts in global rows (no LDS for them): in the loop over runs a lane's accepted requests of a run
+    // are the growth of n_good over the run, added once at its end.
+    const bool model_per_run = RUNS && want_model && !model_lds;
 
     // One request for the whole wavefront: `at` is its place in the stream, m / n the model and the tile's
     // replica bound for it (wave-uniform), da / db this lane's descriptors of the model's replicas.
@@ -478,6 +489,15 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             ch_last = rep_addr(win.d) + rel_base;
             ch_first = ch_last - (uint32_t)(found ? stages_m1 : 0) * kSlotBytes;
             ch_lrow = found ? (int)rep_lat_last(win.d) - stages_m1 : 0;
+            if (group_regs) {  // requests handled up to here went to the group chosen before (:611, :618)
+                const uint32_t now = found ? ch_last : 0xFFFFFFFFu;
+                if (now != pg_addr) {
+                    flush_group((uint32_t)(at - r0));
+                    pg_addr = now;
+                    pg_req0 = (uint32_t)(at - r0);
+                    pg_good0 = n_good;
+                }
+            }
         }
         const double best = ch_best;
         const bool has = ch_sm1 >= 0;
@@ -599,16 +619,8 @@ asm volatile(NAME##_TEXT                                                        
             if (!asm_walk) acc_mask = __ballot(acc);
             ch_stale = acc_mask != 0ull;
         }
-        if (group_regs) {  // :611, :618
-            const uint32_t now = has ? last_addr : 0xFFFFFFFFu;
-            if (now != pg_addr) {
-                flush_group();
-                pg_addr = now;
-                pg_req = 0;
-                pg_good = 0;
-            }
-            pg_req += has ? 1u : 0u;
-            pg_good += acc ? 1u : 0u;
+        if (group_regs) {
+            // counted when the lane's group changes (above)
         } else if (want_group && has) {  // :611, :618
             const uint32_t g = owner[(last_addr - clk_off) >> 3];  // (slot * 512 + lane * 8) / 8
             // LDS adds that return nothing: the wavefront does not wait for them
@@ -633,7 +645,7 @@ asm volatile(NAME##_TEXT                                                        
         if (model_lds) {  // an LDS add that returns nothing
             if (m >= 0)
                 __hip_atomic_fetch_add(&mcnt[m * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-        } else if (want_model && m >= 0 && acc) {  // one owner per counter: a relaxed add that nobody waits for
+        } else if (want_model && !model_per_run && m >= 0 && acc) {  // one owner per counter: a relaxed add that nobody waits for
             __hip_atomic_fetch_add(&model_good[(size_t)m * kWave], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         if (want_req) {
@@ -699,6 +711,7 @@ asm volatile(NAME##_TEXT                                                        
                 const int m = w >= 0 ? (w & 0xFFFFFF) : -1;  // wave-uniform model id (or -1)
                 const int n = w >= 0 ? (w >> 24) : 0;        // replica bound of the tile; 0: nothing to simulate
                 const uint64_t run = (s1 >= 64 ? ~0ull : ((1ull << s1) - 1ull)) & (~0ull << s0) & valid;
+                const int32_t good_before = n_good;  // model_per_run
 
                 auto request = [&](int i) {
                     return simulate(blk + i, m, n, da, db,
@@ -737,12 +750,10 @@ asm volatile(NAME##_TEXT                                                        
                         }
                         const uint64_t todo = later & ~skip;
                         const int next = todo ? (int)__builtin_ctzll(todo) : 64;
-                        if constexpr (OUT == 1) {
+                        if constexpr (OUT == 2) {
                             // requests of the run that are passed over for good
                             const int passed = __builtin_popcountll(next < 64 ? later & ~(~0ull << next) : later);
-                            if (group_regs) {  // the lane's pending group is the one kept from the request before
-                                if (ch_sm1 >= 0) pg_req += (uint32_t)passed;
-                            } else if (want_group && passed > 0 && ch_sm1 >= 0) {
+                            if (group_lds && passed > 0 && ch_sm1 >= 0) {
                                 const uint32_t g = owner[(ch_last - clk_off) >> 3];
                                 __hip_atomic_fetch_add(&gcnt[g * kWave], (uint32_t)passed, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_WAVEFRONT);
@@ -754,6 +765,11 @@ asm volatile(NAME##_TEXT                                                        
                     }
                 } else {
                     for (int i = s0; i < s1; ++i) request(i);
+                }
+                if (model_per_run && m >= 0) {  // one owner per counter: a relaxed add that nobody waits for
+                    const int32_t grown = n_good - good_before;
+                    if (grown != 0)
+                        __hip_atomic_fetch_add(&model_good[(size_t)m * kWave], grown, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
                 s0 = s1;
             }
@@ -822,7 +838,7 @@ asm volatile(NAME##_TEXT                                                        
         for (int s = 0; s < nslots; ++s) saved[(size_t)s * kWave] = clk[s * kWave];
     if (model_lds)
         for (int m = 0; m < a.M; ++m) model_good[(size_t)m * kWave] = (int32_t)mcnt[m * kWave];
-    if (group_regs) flush_group();
+    if (group_regs) flush_group((uint32_t)(r1 - r0));
     if (group_lds) {
         for (int g = 0; g < a.Gmax; ++g) {
             greq[g * kWave] = (int32_t)gcnt[g * kWave];
@@ -872,17 +888,22 @@ hipError_t launch_one(const MixedArgs &args, int wpb, size_t lds_bytes, hipStrea
 // table in global memory only the general kernels exist.
 template <int SMAX, bool UNIFORM>
 hipError_t launch_u(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
-    // what the request loop has to produce: 0 scores only, 1 also per-model / per-group counts, 2 anything
-    const int out = (args.flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT)) ? 2
-                    : (args.flags & (MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) ? 1 : 0;
-    if (!args.lat_in_lds) return launch_one<SMAX, false, UNIFORM, false, 2>(args, wpb, lds_bytes, stream);
+    // what the request loop has to produce: 0 scores only, 1 also per-model / per-group counts without counters in
+    // LDS, 2 counts with counters in LDS (small batches), 3 anything
+    const bool lds_counters = ((args.flags & MMSIM_WANT_GROUP_COUNTS) && !args.group_global) ||
+                              ((args.flags & MMSIM_WANT_MODEL_COUNTS) && args.model_lds);
+    const int out = (args.flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT)) ? 3
+                    : (args.flags & (MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) ? (lds_counters ? 2 : 1) : 0;
+    if (!args.lat_in_lds) return launch_one<SMAX, false, UNIFORM, false, 3>(args, wpb, lds_bytes, stream);
     if constexpr (SMAX == 4 || SMAX == 16) {  // the stage buckets with a hand-scheduled walk
         if (args.pow2_depths)
-            return out == 2   ? launch_one<SMAX, true, UNIFORM, true, 2>(args, wpb, lds_bytes, stream)
+            return out == 3   ? launch_one<SMAX, true, UNIFORM, true, 3>(args, wpb, lds_bytes, stream)
+                   : out == 2 ? launch_one<SMAX, true, UNIFORM, true, 2>(args, wpb, lds_bytes, stream)
                    : out == 1 ? launch_one<SMAX, true, UNIFORM, true, 1>(args, wpb, lds_bytes, stream)
                               : launch_one<SMAX, true, UNIFORM, true, 0>(args, wpb, lds_bytes, stream);
     }
-    return out == 2   ? launch_one<SMAX, true, UNIFORM, false, 2>(args, wpb, lds_bytes, stream)
+    return out == 3   ? launch_one<SMAX, true, UNIFORM, false, 3>(args, wpb, lds_bytes, stream)
+           : out == 2 ? launch_one<SMAX, true, UNIFORM, false, 2>(args, wpb, lds_bytes, stream)
            : out == 1 ? launch_one<SMAX, true, UNIFORM, false, 1>(args, wpb, lds_bytes, stream)
                       : launch_one<SMAX, true, UNIFORM, false, 0>(args, wpb, lds_bytes, stream);
 }
