@@ -181,11 +181,56 @@ def _check(out, ref, s, per_request=False):
 def test_config5_subsample_counts(eng):
     cfg = make_config(5, 96)
     flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
-    out, table, packed, streams, info, ms = _run(eng, cfg, cfg.placements, [0, 1], flags)
+    out, table, packed, streams, info, ms = _run(eng, cfg, cfg.placements, cfg.base_seeds, flags)
+    assert len(streams) == 4
     print(info, f"kernel {ms:.1f} ms", flush=True)
     for s, st in enumerate(streams):
         ref = oracle_batch(st, table, packed, batching=True)
         _check(out, ref, s)
+
+
+def test_config5_full_size_properties(eng):
+    """Configuration 5 at full size (8192 candidates x 4 arrival seeds): no simulation runs out of event
+    slots, a placement's results do not depend on where it sits in the batch or on what shares its
+    wavefront, and the counts are consistent with each other and with the streams."""
+    cfg = make_config(5)
+    B = len(cfg.placements)
+    assert B == 8192
+    flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
+    base, table, packed, streams, info, ms = _run(eng, cfg, cfg.placements, cfg.base_seeds, flags)
+    print(info, f"kernel {ms:.1f} ms", flush=True)
+    assert info["lanes"] == 4 * B and np.all(base["status"] == 0)
+    # a permutation of the candidate list permutes the results
+    perm = np.random.default_rng(11).permutation(B)
+    shuffled, *_ = _run(eng, cfg, [cfg.placements[i] for i in perm], cfg.base_seeds, 0)
+    assert np.all(shuffled["status"] == 0)
+    assert np.array_equal(shuffled["n_good"], base["n_good"][:, perm])
+    assert np.array_equal(shuffled["latency_sum"], base["latency_sum"][:, perm])
+    # a small batch (other tile width, other LDS layout) agrees, and agrees with the oracle
+    pick = perm[:40]
+    small, t2, p2, *_ = _run(eng, cfg, [cfg.placements[i] for i in pick], cfg.base_seeds[:1], flags)
+    for k in ("n_good", "model_num_good"):
+        assert np.array_equal(small[k][0], base[k][0][pick]), k
+    for k in ("group_num_requests", "group_num_good"):      # the group axis is as wide as the batch's largest placement
+        g = small[k][0].shape[1]
+        assert np.array_equal(small[k][0], base[k][0][pick][:, :g]) and not base[k][0][pick][:, g:].any(), k
+    # batch members are summed in another order by tiles of another width: 1e-12 relative
+    np.testing.assert_allclose(small["latency_sum"][0], base["latency_sum"][0][pick], rtol=1e-12, atol=0)
+    ref = oracle_batch(streams[0], t2, p2, batching=True)
+    _check(small, ref, 0)
+    # counts: goodput = sum of per-model goods = sum of per-group goods; every request of a hosted model is
+    # served or dropped on exactly one group; models without a replica are not counted at all
+    assert np.array_equal(base["model_num_good"].sum(axis=2), base["n_good"])
+    assert np.array_equal(base["group_num_good"].sum(axis=2), base["n_good"])
+    assert np.array_equal(base["group_num_requests"].sum(axis=2), base["model_num_requests"].sum(axis=2))
+    hosted = np.zeros((B, cfg.num_models), bool)
+    for b, pl in enumerate(cfg.placements):
+        for ms_ in pl.group_models:
+            hosted[b, list(ms_)] = True
+    for s, st in enumerate(streams):
+        per_model = np.bincount(st.model_ids[st.model_ids >= 0], minlength=cfg.num_models)
+        assert np.array_equal(base["model_num_requests"][s], hosted * per_model[None, :])
+        assert np.all(base["n_good"][s] <= len(st.tstamps))
 
 
 def test_config5_full_traces_for_a_few_placements(eng):

@@ -129,12 +129,14 @@ def test_config2_ragged_batch_sizes(eng):
         assert_batch_matches(out, ref, 0, packed[0], per_request=True, where=f"cfg2 B={n}")
 
 
-def test_config3_greedy_step_candidates(eng):
+@pytest.mark.parametrize("flags", [0, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS])
+def test_config3_every_candidate_of_the_greedy_step(eng, flags):
+    """All 4096 candidates of configuration 3 (both base placements, every (group, model) move) against
+    the oracle: goodput and latency sums, and with counts every per-model and per-group counter."""
     cfg = make_config(3)
-    picks = list(range(0, 4096, 13))[:256]      # spread over both base placements
-    sols = [cfg.placements[i] for i in picks]
-    out, table, packed, streams, _ = _run_config(
-        eng, cfg, sols, [0], _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
+    assert len(cfg.placements) == 4096
+    out, table, packed, streams, info = _run_config(eng, cfg, cfg.placements, [0], flags)
+    assert info["lanes"] == 4096
     ref = oracle_batch(streams[0], table, packed)
     assert_batch_matches(out, ref, 0, packed[0], where="cfg3")
 
