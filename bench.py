@@ -34,6 +34,21 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def measured_traffic(kernel, workload):
+    """HBM bytes per launch of `kernel` on `workload` from the committed counter summary
+    (profiles/traffic.json: FETCH_SIZE / WRITE_SIZE of a rocprofv3 --pmc run, scaled by the same
+    counters of a device copy of known size), or None when the summary is for another kernel or workload."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    for e in json.load(open(path)):
+        if e["kernel"] == kernel and e["workload"] == workload:
+            fetch = e["fetch_size_kib"] * e["copy_bytes"] / 1024.0 / e["copy_fetch_size_kib"]
+            write = e["write_size_kib"] * e["copy_bytes"] / 1024.0 / e["copy_write_size_kib"]
+            return (fetch + write) * 1024.0
+    return None
+
+
 def cpu_baseline(cfg, table, stream, sols, n_threads):
     """Times the C oracle (single thread, then n_threads threads over placement
     slices) on `sols` x one stream.  Returns (result dict of 1-thread run, evals/s 1T, evals/s MT)."""
@@ -116,6 +131,8 @@ def main():
     batch = E.Batch(eng, dws, table, packed, flags)
     t_upload = time.perf_counter() - t0
     info = batch.info()
+    batch_kernel = batch.kernel_name()
+    log(f"[bench] kernel: {batch_kernel}")
     log(f"[bench] batch: {info}; python pack {t_pack:.2f}s, library pack+upload {t_upload:.2f}s")
 
     for _ in range(args.warmup):
@@ -136,10 +153,17 @@ def main():
     kernel_s = float(np.mean(kernel_ms)) / 1e3
     value = evals_per_step / sec_per_step
 
-    # exact operation count of the reference loop on these inputs: one untimed pass
-    # (plain simulator only; the batching loop has no fixed per-request operation count)
+    kernel = batch_kernel
+    workload = (f"config {cfg.index} ({cfg.name}): {cfg.num_models} models, {cfg.num_devices} devices, "
+                f"{B} candidate placements x {len(seeds)} seeds, {R_total // len(seeds)} requests/seed")
+    # Operations of the reference loop on these inputs.  Plain simulator: 2*stages + replicas + 3 per dispatched
+    # request, counted exactly by one untimed pass of the kernel itself (and cross-checked against the oracle on
+    # the CPU sample below).  Batching simulator: 2*stages + 2 per check_slo call (+1 for a head's deadline) and
+    # 2*stages + 1 per committed batch, counted by the oracle on the CPU sample and scaled to the batch.
     total_ops = None
     achieved_tops = None
+    ops_note = "achieved counts 2*stages+replicas+3 per dispatched request of the reference loop (what the " \
+               "reference executes on these inputs, not what this kernel executes: it keeps choices and skips requests)"
     if not cfg.batching:
         ops_batch = E.Batch(eng, dws, table, packed, _lib.WANT_OP_COUNT)
         ops_batch.run()
@@ -151,12 +175,10 @@ def main():
         achieved_tops = total_ops / kernel_s / 1e12
     else:
         assert np.all(out["status"] == 0), "a lane ran out of idle-event slots"
+        ops_note = "achieved counts 2*stages+2 per check_slo call (+1 per head deadline) and 2*stages+1 per committed " \
+                   "batch of the reference loop, counted by the oracle on the CPU sample and scaled to the batch"
 
-    # HBM bytes per launch from the committed rocprofv3 counter runs (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB,
-    # scaled by a 1 GiB device copy): only known for the workload those runs used.
-    traffic = None
-    if (cfg.index == 4 and args.placements is None and args.seeds is None and args.flags == "scores"):
-        traffic = 4.691e10 + 1.6e6      # bytes: the committed counter summary of this kernel on this workload (profiles/)
+    traffic = measured_traffic(kernel, workload) if args.flags == "scores" else None
 
     hbm_bytes = info["stream_bytes"] + info["table_bytes"] + 12 * lanes
     # dispatched requests = evaluations whose model has a replica: every one costs 3 operations beyond clocks
@@ -185,9 +207,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f64",
         "data": "synthetic",
-        "config": {"workload": f"config {cfg.index} ({cfg.name}): {cfg.num_models} models, "
-                               f"{cfg.num_devices} devices, {B} candidate placements x {len(seeds)} seeds, "
-                               f"{R_total // len(seeds)} requests/seed",
+        "config": {"workload": workload, "kernel": kernel,
+                   "workgroups": info["workgroups"], "wavefronts_per_workgroup": info["waves_per_group"],
+                   "lds_bytes_per_workgroup": info["lds_bytes"], "stream_segments": info["segments"],
                    "placements": B, "seeds": len(seeds), "requests_per_seed": R_total // len(seeds),
                    "lanes": lanes, "outputs": args.flags, "inputs_resident_in_hbm": True},
         "placements_per_sec": lanes / sec_per_step,
@@ -203,8 +225,7 @@ def main():
             "ops_per_launch": total_ops,
             "ops_per_eval": None if total_ops is None else total_ops / evals_per_step,
             "traffic": traffic,
-            "note": "fp64 add/max/compare only (no FMA): peak = published 78.6 TFLOP/s / 2; "
-                    "achieved counts 2*stages+replicas+3 per dispatched request",
+            "note": "fp64 add/max/compare only (no FMA): peak = published 78.6 TFLOP/s / 2; " + ops_note,
             # the two other ceilings of this path, for the record: compulsory HBM bytes (streams once per
             # wavefront group + tables + results) and algorithmic LDS bytes (8 per clock read or written:
             # 2*stages + replicas per dispatched request) against 8 TB/s and 256 CUs x 128 B/clk x 2.4 GHz
@@ -221,6 +242,15 @@ def main():
         sample = cfg.placements[:min(args.cpu_sample, B)]
         ref, spacked, c1, cm, t1 = cpu_baseline(cfg, table, streams[0], sample, n_threads)
         same = np.array_equal(out["n_good"][0, :len(sample)], ref["n_good"])
+        if cfg.batching:        # scale the sample's operation count to the whole batch
+            sample_evals = len(sample) * len(streams[0].tstamps)
+            total_ops = int(round(ref["fp_ops"] / sample_evals * evals_per_step))
+            rf = result["roofline"]
+            rf["achieved"] = total_ops / kernel_s / 1e12
+            rf["frac"] = rf["achieved"] / FP64_NON_FMA_PEAK_TOPS
+            rf["frac_of_published_fma_peak"] = rf["achieved"] / FP64_VECTOR_PEAK_FMA_TFLOPS
+            rf["ops_per_launch"] = total_ops
+            rf["ops_per_eval"] = total_ops / evals_per_step
         result["cpu_baseline"] = {
             "value": c1, "unit": "evals/s", "cores": 1, "kind": "port",
             "sample": f"first {len(sample)} placements x seed {seeds[0]} "

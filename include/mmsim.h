@@ -202,6 +202,9 @@ typedef struct {
     int32_t waves_per_group;  /* wavefronts of a workgroup that simulate side by side               */
 } mmsim_batch_info;
 int mmsim_batch_get_info(const mmsim_batch *batch, mmsim_batch_info *out);
+/* Name of the kernel template instance mmsim_batch_run launches for this batch, as a profiler prints it
+ * (e.g. "sim_mixed_kernel<16, true, true, true, 0, true>"); measurement aid, no counterpart in the reference. */
+int mmsim_batch_kernel_name(const mmsim_batch *batch, char *buf, size_t size);
 
 /* create + run + sync + fetch + destroy */
 int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,

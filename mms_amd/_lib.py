@@ -79,6 +79,7 @@ SIGNATURES = {
     "mmsim_batch_fetch": (C.c_int, [C.c_void_p, C.POINTER(Result)]),
     "mmsim_batch_destroy": (None, [C.c_void_p]),
     "mmsim_batch_get_info": (C.c_int, [C.c_void_p, C.POINTER(BatchInfo)]),
+    "mmsim_batch_kernel_name": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t]),
     "mmsim_eval_batch": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
                                     C.POINTER(Placements), C.c_uint32, C.POINTER(Result)]),
     "mmsim_eval_batch_static": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),

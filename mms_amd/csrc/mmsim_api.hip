@@ -1362,6 +1362,14 @@ int mmsim_batch_get_info(const mmsim_batch *b, mmsim_batch_info *out) {
     return MMSIM_OK;
 }
 
+int mmsim_batch_kernel_name(const mmsim_batch *b, char *buf, size_t size) {
+    if (!b || !buf || size == 0) return fail(MMSIM_E_INVALID, "batch_kernel_name: null pointer or empty buffer");
+    const std::string name = (b->flags & MMSIM_BATCHING) ? sim_batching_kernel_name(b->bargs)
+                                                         : sim_mixed_kernel_name(b->args, b->smax_bucket);
+    std::snprintf(buf, size, "%s", name.c_str());
+    return MMSIM_OK;
+}
+
 int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
                      const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
                      mmsim_result *out) {

@@ -215,6 +215,8 @@ hipError_t launch_sim_batching(const BatchingArgs &args, int waves_per_block, si
 // Launches the plain simulator with `waves_per_block` wavefronts per workgroup.
 hipError_t launch_sim_mixed(const MixedArgs &args, int smax_bucket, int waves_per_block, size_t lds_bytes,
                             hipStream_t stream, std::string *err);
+std::string sim_mixed_kernel_name(const MixedArgs &args, int smax_bucket);
+std::string sim_batching_kernel_name(const BatchingArgs &args);
 // Smallest compiled stage bucket >= value, or -1.
 int smax_bucket_for(int smax);
 constexpr int kMaxWavesPerBlock = 8;          // plain simulator

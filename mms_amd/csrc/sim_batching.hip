@@ -795,4 +795,12 @@ hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_byt
     return e;
 }
 
+// The template instance launch_sim_batching picks for these arguments, as profilers print it.
+std::string sim_batching_kernel_name(const BatchingArgs &args) {
+    const int nbt = args.NB <= 4 ? 4 : args.NB <= 8 ? 8 : 16;
+    auto tf = [](bool v) { return v ? "true" : "false"; };
+    return "sim_batching_kernel<" + std::to_string(nbt) + ", " + tf(args.lat_lds_bytes > 0) + ", " + tf(args.g2m_in_lds != 0) +
+           ", " + tf(args.lane_stride == 8) + ">";
+}
+
 }  // namespace mmsim

@@ -922,6 +922,20 @@ int smax_bucket_for(int smax) {
     return -1;
 }
 
+// The template instance launch_sim_mixed picks for these arguments, as profilers print it (same choices as
+// launch_u / launch_s above).
+std::string sim_mixed_kernel_name(const MixedArgs &args, int sb) {
+    const bool lds_counters = ((args.flags & MMSIM_WANT_GROUP_COUNTS) && !args.group_global) ||
+                              ((args.flags & MMSIM_WANT_MODEL_COUNTS) && args.model_lds);
+    int out = (args.flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT)) ? 3
+              : (args.flags & (MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) ? (lds_counters ? 2 : 1) : 0;
+    bool latlds = args.lat_in_lds != 0, pow2 = latlds && (sb == 4 || sb == 16) && args.pow2_depths;
+    if (!latlds) out = 3;
+    auto tf = [](bool v) { return v ? "true" : "false"; };
+    return "sim_mixed_kernel<" + std::to_string(sb) + ", " + tf(latlds) + ", " + tf(args.uniform_stages != 0) + ", " + tf(pow2) +
+           ", " + std::to_string(out) + ", " + tf(args.runs != 0) + ">";
+}
+
 hipError_t launch_sim_mixed(const MixedArgs &args, int sb, int wpb, size_t lds_bytes, hipStream_t stream,
                             std::string *err) {
     hipError_t e;

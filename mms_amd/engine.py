@@ -261,6 +261,12 @@ class Batch:
         _lib.check(self.engine.lib.mmsim_batch_get_info(self._h, C.byref(bi)))
         return {f[0]: getattr(bi, f[0]) for f in bi._fields_}
 
+    def kernel_name(self) -> str:
+        """The kernel template instance run() launches, as a profiler prints it."""
+        buf = C.create_string_buffer(256)
+        _lib.check(self.engine.lib.mmsim_batch_kernel_name(self._h, buf, len(buf)))
+        return buf.value.decode()
+
     def fetch(self):
         out, r = _result_arrays(self.flags, self.n_seeds, self.B, self.M, self.Gmax, self.Rmax)
         _lib.check(self.engine.lib.mmsim_batch_fetch(self._h, C.byref(r)))

@@ -229,6 +229,7 @@ typedef struct {
     ev_heap heap;
     int32_t *model_num_good_requests, *group_num_requests, *group_num_good_requests;
     int err;
+    int64_t ops;   /* fp64 operations of check_slo calls, deadlines and commits (measurement only) */
 } bsim;
 
 static inline int64_t qlen(const bsim *s, int32_t m) { return s->tail[m] - s->head[m]; }
@@ -273,6 +274,7 @@ static void b_handle(bsim *s, double tstamp, int32_t m, int32_t g)
         while (qlen(s, m) > 0) {
             const int64_t r = qfront(s, m);
             s->head[m] += 1;                                              /* pop(0) :678 */
+            s->ops += 2 * (int64_t)s->num_stages[g] + 3;  /* deadline add, S max + S add, overhead add, compare */
             if (b_check_slo(s, tstamp, g, lat_mg, s->tstamps[r] + (double)s->slos[r])) {
                 found = 1; first = r; break;
             }
@@ -293,11 +295,13 @@ static void b_handle(bsim *s, double tstamp, int32_t m, int32_t g)
             if ((int64_t)cand - 1 > qlen(s, m)) break;
             const int col = ilog2_i32(cand);
             if (col >= s->NB) { s->err = -2; return; }
+            s->ops += 2 * (int64_t)s->num_stages[g] + 2;
             if (b_check_slo(s, tstamp, g, lat_mg + col, deadline)) bs = cand; else break;
         }
         /* :715-732 */
         const int col = ilog2_i32(bs);
         double t = tstamp + s->fixed_overhead;
+        s->ops += 2 * (int64_t)s->num_stages[g] + 1;    /* the commit's overhead add and stage walk */
         double *clk = s->clocks + (size_t)g * s->Smax;
         const int32_t S = s->num_stages[g];
         for (int32_t k = 0; k < S; ++k) {
@@ -332,7 +336,9 @@ int oracle_simulate_requests_mixed_batching(
     double fixed_overhead,
     int32_t *model_num_requests, int32_t *model_num_good_requests,
     int32_t *group_num_requests, int32_t *group_num_good_requests,
-    int64_t *max_heap_len /* optional */)
+    int64_t *max_heap_len /* optional */,
+    int64_t *fp_ops /* optional: adds the fp64 operations of every check_slo call (2*S + 2, + 1 for a head's
+                       deadline) and of every committed batch (2*S + 1) */)
 {
     bsim s;
     memset(&s, 0, sizeof(s));
@@ -407,6 +413,7 @@ int oracle_simulate_requests_mixed_batching(
     for (int32_t m = 0; m < M; ++m)                                       /* :789-790 */
         if (qlen(&s, m) != 0) { rc = -4; break; }
     if (max_heap_len) *max_heap_len = s.heap.max_n;
+    if (fp_ops) *fp_ops += s.ops;
 done:
     free(s.clocks); free(s.tmp); free(s.order); free(s.qbase); free(s.head); free(s.tail);
     free(s.heap.a);
@@ -496,7 +503,7 @@ int oracle_eval_placements(
             if (batching)
                 rc = oracle_simulate_requests_mixed_batching(
                     finish, good, tstamps, model_ids, slos, m2g, g2m, nst, sl, batch_sizes,
-                    R, M, Gz, Smax, NB, fixed_overhead, mreq, mgood, greq, ggood, NULL);
+                    R, M, Gz, Smax, NB, fixed_overhead, mreq, mgood, greq, ggood, NULL, fp_ops);
             else
                 rc = oracle_simulate_requests_mixed(
                     finish, good, tstamps, model_ids, slos, m2g, nst, sl,

@@ -96,7 +96,7 @@ def simulate_requests_mixed_batching(tstamps, model_ids, slos, m2g, g2m, num_sta
         _p(sl, C.c_float), _p(m2g, C.c_int32), _p(g2m, C.c_int32), _p(ns, C.c_int32),
         _p(lat, C.c_float), _p(bss, C.c_int32),
         C.c_int64(R), C.c_int32(M), C.c_int32(G), C.c_int32(S), C.c_int32(NB),
-        C.c_double(fixed_overhead), *[_p(c, C.c_int32) for c in cnt], C.byref(mh))
+        C.c_double(fixed_overhead), *[_p(c, C.c_int32) for c in cnt], C.byref(mh), None)
     assert rc == 0, rc
     assert not (good == 255).any()
     return finish, good.astype(bool), tuple(cnt), mh.value
