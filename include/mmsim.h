@@ -171,6 +171,19 @@ int mmsim_batch_fetch(mmsim_batch *batch, mmsim_result *out);
 void mmsim_batch_destroy(mmsim_batch *batch);
 
 /*
+ * Like mmsim_eval_batch, but placement b is simulated on workloads[stream_of[b]]
+ * only: B simulations, results laid out [B][...] (finish / good rows are Rmax
+ * long, Rmax the longest of the streams).  This is the loop over the segments
+ * of a ModelPlacementWithReplacement in approximate_one_case
+ * (alpa_serve/simulator/controller.py:345-391): every (start time, placement)
+ * pair is simulated on its own slice of the arrivals from idle clocks; here all
+ * segments of all candidates are lanes of one launch.
+ */
+int mmsim_eval_pairs(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_streams,
+                     const mmsim_tables *tables, const mmsim_placements *placements,
+                     const int32_t *stream_of, uint32_t flags, mmsim_result *out);
+
+/*
  * mmsim_eval_batch without any device allocation.  It has no counterpart in
  * the reference; it is for callers that cannot allocate device memory: code
  * under HIP graph capture, tight search or serving loops, harnesses that

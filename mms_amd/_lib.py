@@ -82,6 +82,8 @@ SIGNATURES = {
     "mmsim_batch_kernel_name": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t]),
     "mmsim_eval_batch": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
                                     C.POINTER(Placements), C.c_uint32, C.POINTER(Result)]),
+    "mmsim_eval_pairs": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
+                                    C.POINTER(Placements), _p_i32, C.c_uint32, C.POINTER(Result)]),
     "mmsim_eval_batch_static": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
                                            C.POINTER(Placements), C.c_uint32, C.POINTER(Result)]),
     "mmsim_simulate_requests_mixed": (C.c_int, [

@@ -142,6 +142,12 @@ struct mmsim_batch {
     std::vector<int64_t> wl_R;                           // [n_seeds] stream lengths
     std::vector<std::vector<int32_t>> wl_model_requests;  // [n_seeds][M] requests per model of each stream
     std::vector<int32_t> pos;  // pos[placement] = tile * 64 + lane it is simulated on
+    // Paired batch (mmsim_eval_pairs): placement p is simulated on stream stream_of[p] only; a tile holds
+    // placements of one stream, and results are laid out as for a single seed.
+    bool paired = false;
+    std::vector<int32_t> stream_of;   // [B]
+    DevBuf<int32_t> tile_seed;        // [tiles]
+    int32_t out_seeds = 1;            // seeds of the result layout: n_seeds, or 1 for a paired batch
     size_t wave_bytes = 0;     // LDS bytes of one wavefront's region (chunked loop, batching simulator)
     // Plain simulator, loop over runs: one launch of `sched_groups` workgroups, each owning a set of (tile, stream)
     // items that its wavefronts simulate segment by segment (clocks parked in `state` between segments).
@@ -244,7 +250,7 @@ int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLi
 
 // Builds every device table of a batch from replica lists and launches nothing.
 int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seeds, const mmsim_tables *t,
-                const RepLists &rl, uint32_t flags, mmsim_batch **out) {
+                const RepLists &rl, uint32_t flags, mmsim_batch **out, const int32_t *stream_of = nullptr) {
     const bool batching = (flags & MMSIM_BATCHING) != 0;
     if (batching && (flags & MMSIM_WANT_OP_COUNT)) return fail(MMSIM_E_UNSUPPORTED, "operation counts are only available for the plain simulator");
     if (batching) {
@@ -276,6 +282,13 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     for (int s = 0; s < n_seeds; ++s) {  // copied: the batch does not depend on the workloads outliving it
         b->wl_R.push_back(wls[s]->R);
         b->wl_model_requests.push_back(wls[s]->model_num_requests);
+    }
+    b->paired = stream_of != nullptr;
+    b->out_seeds = b->paired ? 1 : n_seeds;
+    if (b->paired) {
+        b->stream_of.assign(stream_of, stream_of + B);
+        for (int32_t p = 0; p < B; ++p)
+            if (stream_of[p] < 0 || stream_of[p] >= n_seeds) return fail(MMSIM_E_INVALID, "stream_of names a stream outside 0..n_streams-1");
     }
 
     // ---- per placement: slot layout; per (placement, model): replica count
@@ -355,7 +368,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     // no more than fit in LDS.  MMSIM_WAVES_PER_CU (1..8) sets the number instead (tuning knob).
     int wpb_cap = kMaxWavesPerBlock;
     {
-        const int64_t waves_total = (int64_t)((B + kWave - 1) / kWave) * n_seeds;
+        const int64_t waves_total = (int64_t)((B + kWave - 1) / kWave) * b->out_seeds;
         const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
         wpb_cap = (int)std::min<int64_t>(wpb_cap, std::max<int64_t>(1, (waves_total + cus - 1) / cus));
     }
@@ -451,7 +464,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             for (;;) {
                 size_for(blanes);
                 const int64_t per_cu = heap_cap >= heap_min ? (int64_t)ctx->max_lds / (int64_t)wave_bytes : 0;
-                const int64_t waves = (int64_t)((B + blanes - 1) / blanes) * n_seeds;
+                const int64_t waves = (int64_t)((B + blanes - 1) / blanes) * b->out_seeds;
                 if (blanes == 8 || (per_cu >= 8 && waves >= 8 * cus)) break;
                 blanes /= 2;
             }
@@ -463,6 +476,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
 
     std::vector<int32_t> tile_nslots;  // most clock slots of a placement of each tile
+    std::vector<int32_t> tile_stream;  // paired batches: the stream of each tile
     // ---- lane assignment.  A wavefront walks as many pipeline stages as its deepest
     //      lane needs, so placements are ordered by depth before they are cut into
     //      tiles of 64: first by their deepest group, then by the expected depth of a
@@ -495,19 +509,27 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         std::vector<int32_t> order(B);
         for (int32_t p = 0; p < B; ++p) order[p] = p;
         std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
+            if (b->paired && stream_of[x] != stream_of[y]) return stream_of[x] < stream_of[y];
             if (deepest[x] != deepest[y]) return deepest[x] > deepest[y];
             if (by_slots && slots_of[x] != slots_of[y]) return slots_of[x] > slots_of[y];
             return expected[x] > expected[y];
         });
         const int32_t tl = batching ? blanes : kWave;  // placements per tile
         b->pos.assign(B, 0);
-        b->tiles = (B + tl - 1) / tl;
-        b->waves = b->tiles * n_seeds;
-        tile_nslots.assign(b->tiles, 1);
+        int32_t tile = -1, in_tile = tl;
         for (int32_t k = 0; k < B; ++k) {
-            b->pos[order[k]] = (k / tl) * kWave + k % tl;
-            tile_nslots[k / tl] = std::max(tile_nslots[k / tl], slots_of[order[k]]);
+            const int32_t p = order[k];
+            if (in_tile == tl || (b->paired && stream_of[p] != tile_stream.back())) {  // a tile holds one stream's placements
+                ++tile;
+                in_tile = 0;
+                tile_nslots.push_back(1);
+                tile_stream.push_back(b->paired ? stream_of[p] : 0);
+            }
+            b->pos[p] = tile * kWave + in_tile++;
+            tile_nslots[tile] = std::max(tile_nslots[tile], slots_of[p]);
         }
+        b->tiles = tile + 1;
+        b->waves = b->paired ? b->tiles : b->tiles * n_seeds;
         if (batching) {
             b->waves_per_block = std::min(wpb, b->tiles);
             b->wave_bytes = wave_bytes;
@@ -534,7 +556,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     if (!batching && runs) {
         const size_t cap = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail;
         struct Item { int32_t tile, seed, bytes; };
-        const int64_t n_items = (int64_t)b->tiles * n_seeds;
+        const int64_t n_items = (int64_t)b->waves;
         const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
         int64_t groups = std::min<int64_t>(cus, n_items);
         if (const char *env = std::getenv("MMSIM_SCHED_GROUPS")) groups = std::max<int64_t>(1, std::min<int64_t>(n_items, std::atoi(env)));  // tuning knob
@@ -548,7 +570,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         std::vector<std::vector<Item>> per_xcd(nx);
         for (int32_t i = 0; i < b->tiles; ++i) {
             const int r = i % (2 * nx), x = r < nx ? r : 2 * nx - 1 - r;
-            for (int s2 = 0; s2 < n_seeds; ++s2) per_xcd[x].push_back(Item{torder[i], s2, tile_bytes[torder[i]]});
+            if (b->paired)
+                per_xcd[x].push_back(Item{torder[i], tile_stream[torder[i]], tile_bytes[torder[i]]});
+            else
+                for (int s2 = 0; s2 < n_seeds; ++s2) per_xcd[x].push_back(Item{torder[i], s2, tile_bytes[torder[i]]});
         }
         std::vector<std::vector<Item>> per_group((size_t)groups);
         for (int x = 0; x < nx; ++x) {
@@ -844,6 +869,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         HIP_TRY(b->slot_group.alloc(slot_group.size()));
         HIP_TRY(hipMemcpyAsync(b->slot_group.p, slot_group.data(), slot_group.size(), hipMemcpyHostToDevice, st));
     }
+    if (b->paired) {
+        HIP_TRY(b->tile_seed.alloc(tile_stream.size()));
+        HIP_TRY(hipMemcpyAsync(b->tile_seed.p, tile_stream.data(), sizeof(int32_t) * tile_stream.size(), hipMemcpyHostToDevice, st));
+    }
     HIP_TRY(b->kerr.alloc(32));
     HIP_TRY(hipMemsetAsync(b->kerr.p, 0, 32 * sizeof(int32_t), st));
     HIP_TRY(b->rmax.alloc(rmax.size()));
@@ -935,6 +964,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         a.part_off = a.item_nseg + total;
         a.part_bytes = a.part_off + groups * kMaxWavesPerBlock;
     }
+    a.tile_seed = b->tile_seed.p;
+    a.paired = b->paired ? 1 : 0;
     a.sched_groups = b->sched_groups;
     a.seg_requests = b->seg_requests;
     a.sched_lds_bytes = (int32_t)sched_bytes;
@@ -1009,6 +1040,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         q.lat_lds_bytes = (int32_t)batching_lat_lds;
         q.g2m_in_lds = batching_g2m_lds;
         q.lane_stride = blanes;
+        q.tile_seed = b->tile_seed.p;
+        q.paired = b->paired ? 1 : 0;
         q.Rmax = b->Rmax;
         q.fixed_overhead = t->fixed_overhead;
         q.flags = flags;
@@ -1252,7 +1285,7 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
         ops.resize(lanes_padded);
         HIP_TRY(hipMemcpy(ops.data(), b->fp_ops.p, sizeof(int64_t) * lanes_padded, hipMemcpyDeviceToHost));
     }
-    for (int s = 0; s < b->n_seeds; ++s)
+    for (int s = 0; s < b->out_seeds; ++s)
         for (int32_t p = 0; p < B; ++p) {
             const size_t src = (size_t)s * tiles * kWave + b->pos[p];
             out->n_good[(size_t)s * B + p] = ng[src];
@@ -1265,7 +1298,7 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
     auto unpack_i32 = [&](const DevBuf<int32_t> &dev, int32_t width, int32_t *dst) -> int {
         std::vector<int32_t> h(dev.n);
         HIP_TRY(hipMemcpy(h.data(), dev.p, dev.bytes(), hipMemcpyDeviceToHost));
-        for (int s = 0; s < b->n_seeds; ++s)
+        for (int s = 0; s < b->out_seeds; ++s)
             for (int32_t p = 0; p < B; ++p) {
                 const size_t wave = (size_t)s * tiles + b->pos[p] / kWave;
                 for (int32_t x = 0; x < width; ++x)
@@ -1276,17 +1309,17 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
     if (wm) {
         int rc = unpack_i32(b->model_good, M, out->model_num_good);
         if (rc) return rc;
-        for (int s = 0; s < b->n_seeds; ++s)
+        for (int s = 0; s < b->out_seeds; ++s)
             for (int32_t p = 0; p < B; ++p)
                 for (int32_t m = 0; m < M; ++m)  // the batching loop only counts requests of hosted models (:754-757, :773)
                     out->model_num_requests[((size_t)s * B + p) * M + m] =
-                        (b->hosted.empty() || b->hosted[(size_t)p * M + m]) ? b->wl_model_requests[s][m] : 0;
+                        (b->hosted.empty() || b->hosted[(size_t)p * M + m]) ? b->wl_model_requests[(size_t)(b->paired ? b->stream_of[p] : s)][m] : 0;
     }
     if (wg && b->group_global) {  // counted per last clock slot of the group: map slots back to groups
         std::vector<unsigned long long> h(b->slot_cnt.n);
         HIP_TRY(hipMemcpy(h.data(), b->slot_cnt.p, b->slot_cnt.bytes(), hipMemcpyDeviceToHost));
         const size_t rows = (size_t)b->slot_rows;
-        for (int s = 0; s < b->n_seeds; ++s)
+        for (int s = 0; s < b->out_seeds; ++s)
             for (int32_t p = 0; p < B; ++p) {
                 const size_t wave = (size_t)s * tiles + b->pos[p] / kWave;
                 for (int32_t g = 0; g < Gmax; ++g) {
@@ -1308,15 +1341,15 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
         std::vector<uint8_t> hg(Rm * kWave);
         std::vector<int32_t> owner((size_t)tiles * kWave, -1);  // placement simulated on each lane
         for (int32_t p = 0; p < B; ++p) owner[b->pos[p]] = p;
-        for (int s = 0; s < b->n_seeds; ++s)
+        for (int s = 0; s < b->out_seeds; ++s)
             for (int32_t tile = 0; tile < tiles; ++tile) {
                 const size_t wave = (size_t)s * tiles + tile;
                 HIP_TRY(hipMemcpy(hf.data(), b->finish.p + wave * Rm * kWave, sizeof(double) * Rm * kWave, hipMemcpyDeviceToHost));
                 HIP_TRY(hipMemcpy(hg.data(), b->good.p + wave * Rm * kWave, Rm * kWave, hipMemcpyDeviceToHost));
-                const size_t Rs = (size_t)b->wl_R[s];
                 for (int l = 0; l < kWave; ++l) {
                     const int32_t p = owner[(size_t)tile * kWave + l];
                     if (p < 0) continue;
+                    const size_t Rs = (size_t)b->wl_R[(size_t)(b->paired ? b->stream_of[p] : s)];
                     const size_t row = ((size_t)s * B + (size_t)p) * Rm;
                     for (size_t i = 0; i < Rs; ++i) {
                         out->finish[row + i] = hf[i * kWave + l];
@@ -1343,7 +1376,7 @@ void mmsim_batch_destroy(mmsim_batch *b) {
 
 int mmsim_batch_get_info(const mmsim_batch *b, mmsim_batch_info *out) {
     if (!b || !out) return fail(MMSIM_E_INVALID, "batch_get_info: null pointer");
-    out->lanes = b->B * b->n_seeds;
+    out->lanes = b->B * b->out_seeds;
     out->waves = b->waves;
     out->n_seeds = b->n_seeds;
     out->B = b->B;
@@ -1376,6 +1409,24 @@ int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
     if (!out) return fail(MMSIM_E_INVALID, "eval_batch: out is null");
     mmsim_batch *b = nullptr;
     int rc = mmsim_batch_create(ctx, workloads, n_seeds, tables, placements, flags, &b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
+    if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
+    if (rc == MMSIM_OK) rc = mmsim_batch_fetch(b, out);
+    mmsim_batch_destroy(b);
+    return rc;
+}
+
+int mmsim_eval_pairs(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_streams,
+                     const mmsim_tables *tables, const mmsim_placements *placements, const int32_t *stream_of,
+                     uint32_t flags, mmsim_result *out) {
+    if (!ctx || !out || !stream_of) return fail(MMSIM_E_INVALID, "eval_pairs: null pointer");
+    int rc = check_tables(tables);
+    if (rc) return rc;
+    RepLists rl;
+    rc = lists_from_placements(placements, tables->M, tables->C, &rl);
+    if (rc) return rc;
+    mmsim_batch *b = nullptr;
+    rc = build_batch(ctx, workloads, n_streams, tables, rl, flags, &b, stream_of);
     if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
     if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
     if (rc == MMSIM_OK) rc = mmsim_batch_fetch(b, out);

@@ -94,6 +94,9 @@ struct MixedArgs {
     const float *lat;            // [M][lat_row] compact stage latencies (batch size 1)
     int32_t M, lat_row, rep_extra;
     int32_t n_seeds, B, tiles, nslots, Gmax;
+    const int32_t *tile_seed;    // paired batches: the one stream each tile is simulated on (see `paired`)
+    int32_t paired;              // 1: every tile has its own stream and results are laid out as for one seed;
+                                 // 0: every tile is simulated on every stream
     int32_t slot_rows;           // row pitch of slot_group (most slots of any tile)
     int32_t state_rows;          // row pitch of state
     double *state;               // [waves][state_rows][64] clocks parked between segments (scheduled launch)
@@ -178,6 +181,8 @@ struct BatchingArgs {
     int32_t lat_lds_bytes;       // > 0: the workgroup keeps a copy of lat in LDS (that many bytes, 16-aligned)
     int32_t g2m_in_lds;          // 1: each wavefront keeps its g2m_off / g2m_idx rows in LDS
     int32_t lane_stride;         // 64, 32 or 16: lanes of a wavefront that simulate; pitch of the per-lane LDS arrays
+    const int32_t *tile_seed;    // as in MixedArgs
+    int32_t paired;
     int64_t Rmax;
     double fixed_overhead;
     uint32_t flags;

@@ -135,8 +135,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const int W = (int)(blockDim.x >> 6);
     const int wv = uniform_i((int)(threadIdx.x >> 6));
     const int lane = (int)(threadIdx.x & 63);
-    const int seed = (int)(blockIdx.x % (unsigned)a.n_seeds);
-    const int tile = (int)(blockIdx.x / (unsigned)a.n_seeds) * W + wv;
+    const unsigned grid_seeds = a.paired ? 1u : (unsigned)a.n_seeds;
+    const int tile = (int)(blockIdx.x / grid_seeds) * W + wv;
+    // paired batches: the tile's own stream; otherwise every tile on every stream
+    const int seed = a.paired ? (tile < a.tiles ? a.tile_seed[tile] : 0) : (int)(blockIdx.x % grid_seeds);
     const bool want_model = (a.flags & MMSIM_WANT_MODEL_COUNTS) != 0;
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     __syncthreads();  // the latency table is complete; wavefronts run independently from here
     if (!live) return;
 
-    const int wave = seed * a.tiles + tile;
+    const int wave = a.paired ? tile : seed * a.tiles + tile;  // where this (tile, stream) pair's results go
     const int64_t off = a.stream_off[seed];
     const int64_t R = a.stream_off[seed + 1] - off;
     const Req *__restrict__ reqs = a.streams + off;
@@ -752,7 +754,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     }
 
     if (oj == 0) {
-        const size_t out = (size_t)seed * a.tiles * kWave + (size_t)tile * kWave + sl;
+        const size_t out = (size_t)wave * kWave + sl;
         a.n_good[out] = n_good;
         a.lat_sum[out] = lat_sum;
         a.status[out] = dead;
@@ -787,7 +789,7 @@ hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_byt
                                     (int)lds_bytes);
         if (e == hipSuccess) {
             const unsigned tile_groups = (unsigned)((args.tiles + wpb - 1) / wpb);
-            hipLaunchKernelGGL(kern, dim3(tile_groups * (unsigned)args.n_seeds), dim3(wpb * kWave), lds_bytes, stream, args);
+            hipLaunchKernelGGL(kern, dim3(tile_groups * (unsigned)(args.paired ? 1 : args.n_seeds)), dim3(wpb * kWave), lds_bytes, stream, args);
             e = hipGetLastError();
         }
     }

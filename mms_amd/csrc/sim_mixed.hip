@@ -257,11 +257,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         for (int k = (int)threadIdx.x; k < n_items; k += (int)blockDim.x) sched->item[k] = 0u;
         live = wv < kMaxWavesPerBlock && part_off >= 0;
     } else {
+        const unsigned grid_seeds = a.paired ? 1u : (unsigned)a.n_seeds;
         const unsigned bq = a.xcd_map ? blockIdx.x >> 3 : blockIdx.x;
-        seed = (int)(bq % (unsigned)a.n_seeds);
-        const int tgroup = a.xcd_map ? (int)(bq / (unsigned)a.n_seeds) * 8 + (int)(blockIdx.x & 7u) : (int)(bq / (unsigned)a.n_seeds);
+        seed = (int)(bq % grid_seeds);
+        const int tgroup = a.xcd_map ? (int)(bq / grid_seeds) * 8 + (int)(blockIdx.x & 7u) : (int)(bq / grid_seeds);
         tile = tgroup * W + wv;
         live = tile < a.tiles;
+        if (a.paired && live) seed = a.tile_seed[tile];
     }
     unsigned char *mine = lds_raw + a.lat_lds_bytes + (SCHED ? a.sched_lds_bytes + part_off : wv * a.wave_lds_bytes);
     uint8_t *rmax_lds = mine + (RUNS ? 0 : kStageBytes);
@@ -347,7 +349,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     uint32_t *gcnt = reinterpret_cast<uint32_t *>(owner + own_bytes) + lane;
     uint32_t *mcnt = gcnt + (group_lds ? 2 * a.Gmax * kWave : 0);  // [M][64] accepted requests per model
 
-    const int wave = seed * a.tiles + tile;
+    const int wave = a.paired ? tile : seed * a.tiles + tile;  // where this (tile, stream) pair's results go
     const size_t out = (size_t)wave * kWave + lane;
     const int64_t off = a.stream_off[seed];
     const int64_t R = a.stream_off[seed + 1] - off;
@@ -871,7 +873,7 @@ hipError_t launch_kernel(const MixedArgs &args, int wpb, size_t lds_bytes, hipSt
         blocks = (unsigned)args.sched_groups;
     } else {
         const unsigned tile_groups = (unsigned)((args.tiles + wpb - 1) / wpb);
-        blocks = (args.xcd_map ? ((tile_groups + 7u) & ~7u) : tile_groups) * (unsigned)args.n_seeds;
+        blocks = (args.xcd_map ? ((tile_groups + 7u) & ~7u) : tile_groups) * (unsigned)(args.paired ? 1 : args.n_seeds);
     }
     const dim3 grid(blocks);
     hipLaunchKernelGGL(kern, grid, dim3(wpb * kWave), lds_bytes, stream, args);

@@ -231,6 +231,23 @@ def eval_batch(engine: "Engine", workloads, table: "LatencyTable", packed, flags
     return _shape_results(out, n_seeds, B)
 
 
+def eval_pairs(engine: "Engine", workloads, table: "LatencyTable", packed, stream_of, flags: int = 0,
+               fixed_overhead: float = FIXED_OVERHEAD):
+    """One call of ``mmsim_eval_pairs``: placement b on ``workloads[stream_of[b]]`` only.
+    Result arrays are [B][...]."""
+    workloads = list(workloads)
+    t, p, wl, keep = _abi_inputs(workloads, table, packed, fixed_overhead)
+    so = _lib.carray(stream_of, np.int32)
+    assert len(so) == p.B
+    out, r = _result_arrays(flags, 1, p.B, t.M, p.Gmax, max(w.R for w in workloads))
+    _lib.check(engine.lib.mmsim_eval_pairs(engine._h, wl, len(workloads), C.byref(t), C.byref(p),
+                                           _lib.ptr(so, C.c_int32), int(flags), C.byref(r)))
+    del keep
+    if "good" in out:
+        out["good"] = out["good"].astype(bool)
+    return out
+
+
 class Batch:
     """Device-resident batch of placements x seeds; run() may be repeated."""
 

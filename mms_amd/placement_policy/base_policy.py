@@ -219,14 +219,38 @@ class PlacementEvaluator:
     def _is_plain(sols):
         return all(isinstance(s, ModelPlacement) for s in sols)
 
+    @staticmethod
+    def _num_replicas(sol):
+        if isinstance(sol, ModelPlacement):
+            return sum(len(x) for x in sol.group_models)
+        return sum(len(x) for p in sol.placements for x in p.group_models)
+
+    def _mixed_stats(self, sols):
+        """Fast statistics (controller.py:393-403) of a list that holds ModelPlacementWithReplacement
+        entries: every segment of every entry (a plain placement being one segment over the whole
+        workload) is a lane of one GPU launch (controller.py:345-391 evaluated as a batch)."""
+        from mms_amd.simulator.controller import replacement_fast_stats, simulate_replacements
+        self._prepare()
+        wl = self.workload
+        model_ids, slos, names, profs = wl.cached_data
+        as_replacements = [s if isinstance(s, ModelPlacementWithReplacement)
+                           else ModelPlacementWithReplacement([0], [s]) for s in sols]
+        if not hasattr(self, "_segment_workloads"):
+            self._segment_workloads = {}
+        res = simulate_replacements(as_replacements, names, profs, model_ids, slos, wl.arrivals,
+                                    _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS,
+                                    enable_batching=self.enable_batching, table=self._table,
+                                    workload_cache=self._segment_workloads)
+        return [replacement_fast_stats(names, wl.arrivals, r) for r in res]
+
     # -- public API ---------------------------------------------------------------
     def get_scores(self, sols: List[ModelPlacement]):
         """goodput - latency_mean/10000 + num_replicas/1e6 per placement (:225-226)."""
         if len(sols) == 0:
             return []
         if not self._is_plain(sols):
-            return [self.get_goodput_simulation(s, self.model_datas, self.cluster_env,
-                                                self.workload, self.method) for s in sols]
+            return [st.goodput - st.latency_mean / 10000 + self._num_replicas(sol) / 1000000
+                    for sol, st in zip(sols, self._mixed_stats(sols))]
         out = self._run(sols, 0)
         R = len(self.workload)
         goodput = out["n_good"][0] / R
@@ -241,8 +265,8 @@ class PlacementEvaluator:
         if len(sols) == 0:
             return []
         if not self._is_plain(sols):
-            return [self.get_stats_simulation(s, self.model_datas, self.cluster_env,
-                                              self.workload, self.method) for s in sols]
+            return [(st.goodput, [x.goodput for x in st.per_model_stats], st.group_num_requests, st)
+                    for st in self._mixed_stats(sols)]
         out = self._run(sols, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
         arrivals = self.workload.arrivals
         R = len(arrivals)

@@ -140,6 +140,69 @@ def approximate_one_case_one_placement(placement, model_names, prof_ress, model_
     return (start, finish, good) + tuple(counts)
 
 
+def replacement_cuts(placement, arrivals):
+    """Index ranges of the segments of a ModelPlacementWithReplacement: a new segment starts at the
+    first arrival strictly later than the next change time (controller.py:345-365)."""
+    change_times = list(placement.start_times[1:]) + [inf]
+    cuts = [0]
+    pt = 0
+    for i in range(len(arrivals)):
+        if arrivals[i] > change_times[pt]:
+            cuts.append(i)
+            pt += 1
+    cuts.append(len(arrivals))
+    return list(zip(cuts[:-1], cuts[1:]))
+
+
+def simulate_replacements(sols, model_names, prof_ress, model_ids, slos, arrivals, flags=0,
+                          enable_batching=False, table=None, workload_cache=None):
+    """All segments of all ``ModelPlacementWithReplacement`` in ``sols`` as lanes of ONE GPU launch
+    (``mmsim_eval_pairs``): segment k of candidate n is its placement simulated from idle clocks on
+    its slice of the arrivals, as the reference does one after another (controller.py:345-391).
+
+    Returns one dict per candidate: ``n_good``, ``latency_sum`` and, with the count flags,
+    ``model_num_requests`` / ``model_num_good`` / ``group_num_requests`` / ``group_num_good`` summed
+    over its segments (:385-391; the group axis is as wide as the candidate's widest placement), and
+    with ``WANT_PER_REQUEST`` ``finish`` / ``good`` concatenated (:381-383).
+    """
+    eng = _engine.Engine.default()
+    arrivals = np.asarray(arrivals, dtype=np.float64)
+    if table is None:
+        table = _engine.LatencyTable(prof_ress, list(batchsize_config) if enable_batching else [1])
+    if enable_batching:
+        flags |= _lib.BATCHING
+    cache = {} if workload_cache is None else workload_cache
+    streams, stream_index, lanes, stream_of, owner = [], {}, [], [], []
+    for n, sol in enumerate(sols):
+        for seg, (lo, hi) in enumerate(replacement_cuts(sol, arrivals)):
+            if (lo, hi) not in stream_index:
+                if (lo, hi) not in cache:
+                    cache[(lo, hi)] = _engine.DeviceWorkload(eng, arrivals[lo:hi], model_ids[lo:hi], slos[lo:hi],
+                                                             len(model_names))
+                stream_index[(lo, hi)] = len(streams)
+                streams.append(cache[(lo, hi)])
+            lanes.append(sol.placements[seg])
+            stream_of.append(stream_index[(lo, hi)])
+            owner.append((n, lo, hi))
+    out = _engine.eval_pairs(eng, streams, table, _engine.pack_placements(lanes, table), stream_of, flags)
+    results = [None] * len(sols)
+    for n, sol in enumerate(sols):
+        mine = [k for k, o in enumerate(owner) if o[0] == n]
+        res = {"n_good": int(out["n_good"][mine].sum()), "latency_sum": float(np.sum(out["latency_sum"][mine]))}
+        for key in ("model_num_requests", "model_num_good"):
+            if key in out:
+                res[key] = out[key][mine].sum(axis=0)
+        gmax = max(len(p.group_configs) for p in sol.placements)
+        for key in ("group_num_requests", "group_num_good"):
+            if key in out:
+                res[key] = out[key][mine][:, :gmax].sum(axis=0)
+        if "finish" in out:
+            res["finish"] = np.concatenate([out["finish"][k, :owner[k][2] - owner[k][1]] for k in mine])
+            res["good"] = np.concatenate([out["good"][k, :owner[k][2] - owner[k][1]] for k in mine])
+        results[n] = res
+    return results
+
+
 def approximate_one_case(case: ServingCase, seed: int = 0, warmup: int = DEFAULT_WARMUP,
                          debug: bool = False, fast_stats: bool = False,
                          enable_batching: bool = False):
@@ -175,28 +238,17 @@ def approximate_one_case(case: ServingCase, seed: int = 0, warmup: int = DEFAULT
              placement, model_names, prof_ress, model_ids, slos, arrivals,
              enable_batching=enable_batching)
     elif isinstance(placement, ModelPlacementWithReplacement):
-        # A new segment starts at the first arrival strictly later than the next
-        # change time; every segment starts from idle clocks (:345-391).
-        change_times = list(placement.start_times[1:]) + [inf]
-        cuts = [0]
-        pt = 0
-        for i in range(len(arrivals)):
-            if arrivals[i] > change_times[pt]:
-                cuts.append(i)
-                pt += 1
-        cuts.append(len(arrivals))
-        pieces = []
-        for seg, (lo, hi) in enumerate(zip(cuts[:-1], cuts[1:])):
-            pieces.append(approximate_one_case_one_placement(
-                placement.placements[seg], model_names, prof_ress, model_ids[lo:hi],
-                slos[lo:hi], arrivals[lo:hi], enable_batching=enable_batching))
-        start = np.concatenate([p[0] for p in pieces])
-        finish = np.concatenate([p[1] for p in pieces])
-        good = np.concatenate([p[2] for p in pieces])
-        model_num_requests = np.sum([p[3] for p in pieces], axis=0)
-        model_num_good_requests = np.sum([p[4] for p in pieces], axis=0)
-        group_num_requests = np.sum([p[5] for p in pieces], axis=0)
-        group_num_good_requests = np.sum([p[6] for p in pieces], axis=0)
+        # every segment starts from idle clocks on its own slice of the arrivals (:345-391); all segments are
+        # lanes of one launch
+        counts = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
+        res = simulate_replacements([placement], model_names, prof_ress, model_ids, slos, arrivals,
+                                    counts if fast_stats else counts | _lib.WANT_PER_REQUEST,
+                                    enable_batching=enable_batching)[0]
+        model_num_requests, model_num_good_requests = res["model_num_requests"], res["model_num_good"]
+        group_num_requests, group_num_good_requests = res["group_num_requests"], res["group_num_good"]
+        if fast_stats:      # the fast statistics only need the sums (:393-403)
+            return replacement_fast_stats(model_names, arrivals, res), placement
+        start, finish, good = arrivals, res["finish"], res["good"]
     else:
         raise TypeError(f"unsupported placement type: {type(placement)}")
 
@@ -207,6 +259,18 @@ def approximate_one_case(case: ServingCase, seed: int = 0, warmup: int = DEFAULT
         stats = workload.compute_stats(start, finish, good, warmup)
         stats.group_num_requests = tuple(group_num_requests)
     return stats, placement
+
+
+def replacement_fast_stats(model_names, arrivals, res):
+    """fast_stats_result from the sums over a candidate's segments: mean(good) = accepted / requests,
+    mean(finish - start) = latency sum / requests (rejected requests contribute 0, :613-622)."""
+    R = len(arrivals)
+    interval = arrivals[-1] - arrivals[0]
+    mreq, mgood = res["model_num_requests"], res["model_num_good"]
+    per_model = [PerModelStatsResult(model_names[i], mreq[i], mgood[i] / (mreq[i] + eps), mreq[i] / interval,
+                                     0, 0, 0, 0, [], [], []) for i in range(len(model_names))]
+    return StatsResult(per_model, tuple(res["group_num_requests"]), np.float64(res["n_good"]) / R,
+                       res["latency_sum"] / R, R, R / interval)
 
 
 def fast_stats_result(model_names, start, finish, good, model_num_requests,

@@ -93,6 +93,26 @@ def main():
                                         "best": dump(sols[best]), "best_score": scores[best]}
         print(name, dump(placement)["group_models"], score, flush=True)
 
+    def record_replacement(name, interval, model_spec, cluster_spec):
+        """SelectiveReplicationReplacement (selective_replication.py:206-244): one greedy placement per interval
+        of the workload; the composite is then scored by the reference's own approximate_one_case, segment by
+        segment (simulator/controller.py:345-391)."""
+        model_datas = models(*model_spec)
+        cluster_env = pp.ClusterEnv(*cluster_spec)
+        rep, _ = pp.SelectiveReplicationReplacement(interval).solve_placement(model_datas, cluster_env)
+        wl = pp.base_policy.gen_train_workload(model_datas)
+        ev = pp.base_policy.PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+        # (get_scores of the reference cannot take the composite: base_policy.py:225 reads sol.group_models)
+        stats = ev.get_stats([rep])[0]
+        cases.append({"name": name, "policy": "SelectiveReplicationReplacement", "kwargs": {"replacement_interval": interval},
+                      "models": list(model_spec), "cluster": list(cluster_spec),
+                      "start_times": [float(t) for t in rep.start_times],
+                      "placements": [dump(p) for p in rep.placements],
+                      "goodput": float(stats[0]), "model_goodput": [float(x) for x in stats[1]],
+                      "latency_mean": float(stats[3].latency_mean),
+                      "group_num_requests": [int(x) for x in stats[2]]})
+        print(name, len(rep.placements), "segments", float(stats[0]), flush=True)
+
     # the three situations of the reference's own test
     record("ref_test_sr_greedy", "SelectiveReplicationGreedy", {}, (4, 1, 5, 1), (4, 4.5 * GB))
     record("ref_test_sr_search", "SelectiveReplicationSearch", {}, (4, 1, 5, 1), (4, 4.5 * GB))
@@ -106,6 +126,9 @@ def main():
     # two kinds of models: the search also splits the devices between them (model_parallelism.py:356-456)
     record("separation_mp_search", "ModelParallelismSearch", {"use_separation": True},
            [(3, 0.5, 5, 3, "test-2GB-100ms"), (2, 0.9, 3, 2, "test-4GB-150ms")], (6, 8.5 * GB))
+
+    # a placement per 150 s of a loaded workload (5 models do not all fit 4 devices at once)
+    record_replacement("replacement_sr", 150, (5, 0.5, 7, 4), (4, 4.5 * GB))
 
     path = os.path.join(HERE, "search_vectors.json")
     with open(path, "w") as f:

@@ -53,6 +53,36 @@ def _evaluate(engine, workloads, table, sols, flags=0, fixed_overhead=0.011):
     return res
 
 
+def _eval_pairs(engine, workloads, table, packed, stream_of, flags=0, fixed_overhead=0.011):
+    """Placement b on workloads[stream_of[b]] only; result arrays [B][...]."""
+    lat, pp = table.arrays()
+    num_groups, group_cfg, gm_off, gm_idx = packed
+    B, Gmax = group_cfg.shape
+    M = lat.shape[0]
+    Rmax = max(w.R for w in workloads)
+    res = {"n_good": np.zeros(B, np.int64), "latency_sum": np.zeros(B), "status": np.zeros(B, np.int32),
+           "model_num_requests": np.zeros((B, M), np.int32), "model_num_good": np.zeros((B, M), np.int32),
+           "group_num_requests": np.zeros((B, Gmax), np.int32), "group_num_good": np.zeros((B, Gmax), np.int32)}
+    if flags & _lib.WANT_PER_REQUEST:
+        res["finish"] = np.zeros((B, Rmax))
+        res["good"] = np.zeros((B, Rmax), bool)
+    for b in range(B):
+        w = workloads[stream_of[b]]
+        off = gm_off[b:b + 1] - gm_off[b, 0]
+        idx = gm_idx[gm_off[b, 0]:gm_off[b, -1]]
+        o = oracle_c.eval_placements(
+            w.tstamps, w.model_ids, w.slos, lat, pp, table.batch_sizes, num_groups[b:b + 1], group_cfg[b:b + 1],
+            off, idx, batching=bool(flags & _lib.BATCHING), fixed_overhead=fixed_overhead,
+            want_counts=True, want_per_request=bool(flags & _lib.WANT_PER_REQUEST))
+        for k in ("n_good", "latency_sum", "model_num_requests", "model_num_good", "group_num_requests",
+                  "group_num_good"):
+            res[k][b] = o[k][0]
+        if flags & _lib.WANT_PER_REQUEST:
+            res["finish"][b, :w.R] = o["finish"][0]
+            res["good"][b, :w.R] = o["good"][0]
+    return res
+
+
 def _simulate_requests_mixed(engine, finish, good, tstamps, model_ids, slos, m2g, num_stages, lat,
                              num_requests=None, fixed_overhead=0.011):
     f, g, cnt, _ = oracle_c.simulate_requests_mixed(tstamps, model_ids, slos, m2g, num_stages, lat, fixed_overhead)
@@ -83,6 +113,7 @@ def install(monkeypatch):
     monkeypatch.setattr(E.Engine, "default", classmethod(lambda cls: host))
     monkeypatch.setattr(E, "DeviceWorkload", _HostWorkload)
     monkeypatch.setattr(E, "evaluate", _evaluate)
+    monkeypatch.setattr(E, "eval_pairs", _eval_pairs)
     monkeypatch.setattr(E, "simulate_requests_mixed", _simulate_requests_mixed)
     monkeypatch.setattr(E, "simulate_requests", _simulate_requests)
     monkeypatch.setattr(E, "simulate_requests_mixed_batching", _simulate_requests_mixed_batching)

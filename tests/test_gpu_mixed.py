@@ -274,6 +274,39 @@ def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, group
             assert out["fp_ops"][s].sum() == ref["fp_ops"]
 
 
+@pytest.mark.parametrize("mode", ["chunks", "runs", "batching"])
+def test_paired_placements_and_streams(eng, monkeypatch, mode):
+    """mmsim_eval_pairs simulates placement b on stream stream_of[b] only (the segments of placements that
+    replace one another).  Every result must equal the [stream][placement] entry of the full cross product
+    that mmsim_eval_batch computes: 150 placements over 3 streams of different lengths, tiles ragged at the
+    stream boundaries, both request loops of the plain simulator and the batching simulator."""
+    cfg = make_config(5 if mode == "batching" else 2, 150)
+    if mode != "batching":
+        monkeypatch.setenv("MMSIM_RUNS", "1" if mode == "runs" else "0")
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(cfg.placements, table)
+    lens = (2500, 1700, 3001)
+    streams = [cfg.stream(s) for s in cfg.base_seeds[:3]]
+    dws = [E.DeviceWorkload(eng, st.tstamps[:n], st.model_ids[:n], st.slos[:n], cfg.num_models)
+           for st, n in zip(streams, lens)]
+    stream_of = np.random.default_rng(3).integers(0, 3, len(cfg.placements)).astype(np.int32)
+    flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS | _lib.WANT_PER_REQUEST
+    if mode == "batching":
+        flags |= _lib.BATCHING
+    full = E.eval_batch(eng, dws, table, packed, flags)
+    for fl in (flags, flags & ~_lib.WANT_PER_REQUEST, flags & _lib.BATCHING):
+        got = E.eval_pairs(eng, dws, table, packed, stream_of, fl)
+        for b, sidx in enumerate(stream_of):
+            for k in got:
+                if k == "status":
+                    continue
+                want = full[k][sidx, b]
+                if k in ("finish", "good"):
+                    assert np.array_equal(got[k][b][:lens[sidx]], want[:lens[sidx]]), (k, b)
+                else:
+                    assert np.array_equal(got[k][b], want), (k, b)
+
+
 def test_eight_wavefronts_per_workgroup(eng, monkeypatch):
     """Large batches of small placements run 8 wavefronts per workgroup (two per SIMD); forced here on
     520 placements of configuration 2 (16 clock slots)."""

@@ -46,7 +46,7 @@ def _golden_cases():
         return json.load(f)["cases"]
 
 
-@pytest.mark.parametrize("case", _golden_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("case", [c for c in _golden_cases() if "placement" in c], ids=lambda c: c["name"])
 def test_policies_return_what_the_reference_returns(backend, case):
     """Final placement, its score, goodput and per-group request counts as
     recorded from the reference's own policies (tests/golden/make_search_vectors.py)."""
@@ -84,6 +84,39 @@ def test_policies_return_what_the_reference_returns(backend, case):
         best = sols[int(np.argmax(scores))]
         assert [list(c) for c in best.group_configs] == case["separations"]["best"]["group_configs"]
         assert [[int(m) for m in ms] for ms in best.group_models] == case["separations"]["best"]["group_models"]
+
+
+@pytest.mark.parametrize("case", [c for c in _golden_cases() if "placements" in c], ids=lambda c: c["name"])
+def test_replacement_policy_returns_what_the_reference_returns(backend, case):
+    """SelectiveReplicationReplacement (selective_replication.py:206-244): the placement of every interval
+    and its start time as the reference's policy returned them, and the composite's statistics as the
+    reference's approximate_one_case computed them segment by segment (controller.py:345-391) -- here all
+    segments are lanes of one launch."""
+    import mms_amd.placement_policy as pp
+    n, slo, rate, cv = case["models"][:4]
+    model_datas = [ModelData(f"m{i}", slo, rate, cv, load_test_prof_result("test-2GB-100ms")) for i in range(n)]
+    cluster_env = ClusterEnv(*case["cluster"])
+    rep, _ = getattr(pp, case["policy"])(**case["kwargs"]).solve_placement(model_datas, cluster_env)
+    assert isinstance(rep, ModelPlacementWithReplacement)
+    assert [float(t) for t in rep.start_times] == case["start_times"]
+    assert len(rep.placements) == len(case["placements"])
+    for got, want in zip(rep.placements, case["placements"]):
+        assert [list(c) for c in got.group_configs] == want["group_configs"]
+        assert [[int(m) for m in ms] for ms in got.group_models] == want["group_models"]
+    wl = gen_train_workload(model_datas)
+    ev = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+    goodput, model_goodput, group_num_requests, stats = ev.get_stats([rep])[0]
+    assert goodput == case["goodput"]
+    np.testing.assert_allclose(model_goodput, case["model_goodput"], rtol=1e-15, atol=0)
+    assert [int(x) for x in group_num_requests] == case["group_num_requests"]
+    assert abs(stats.latency_mean - case["latency_mean"]) <= 1e-12 * case["latency_mean"]
+    # the same through approximate_one_case with the full statistics (per-request results of every segment)
+    full, _ = approximate_one_case(_case(rep, model_datas, wl), fast_stats=False)
+    assert [int(x) for x in full.group_num_requests] == case["group_num_requests"]
+    # a list of composites and plain placements is one batch too
+    both = ev.get_stats([rep, rep.placements[0], rep])
+    assert both[0][0] == goodput and both[2][0] == goodput
+    assert both[1][0] == ev.get_stats([rep.placements[0]])[0][0]
 
 
 def test_assertions_of_the_reference_test_file(backend):
