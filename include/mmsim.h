@@ -149,7 +149,8 @@ typedef struct {
     int32_t *group_num_requests; /* [L][Gmax]  */
     int32_t *group_num_good;     /* [L][Gmax]  */
     double *finish;              /* [L][Rmax]  Rmax = longest stream of the batch; row tail unspecified */
-    uint8_t *good;               /* [L][Rmax]  */
+    uint8_t *good;               /* [L][Rmax]  both may be NULL: the per-request outputs then stay on the
+                                               device (mmsim_batch_model_stats reads them there) */
     int32_t *status;             /* [L]        0, or MMSIM_E_OVERFLOW for a lane whose results are invalid */
     int64_t *fp_ops;             /* [L]        sum over dispatched requests of 2*stages + replicas + 3:
                                                the fp64 max/add/compare operations the reference's loop
@@ -168,6 +169,44 @@ int mmsim_batch_run(mmsim_batch *batch);
 int mmsim_batch_sync(mmsim_batch *batch, float *kernel_ms);
 /* Copies results of the last completed run into caller memory. */
 int mmsim_batch_fetch(mmsim_batch *batch, mmsim_result *out);
+
+/* Serving statistics per (simulation, model), computed on the device from the
+ * per-request outputs of the last run, which stay there: what
+ * Workload.compute_stats (alpa_serve/simulator/workload.py:308-354) derives
+ * from start / finish / good, start being the arrival times.  All arrays are
+ * [L][M], L as in mmsim_result; all are required.
+ *
+ * Only requests skip[s] <= i < R_s - skip[s] of stream s count (the caller
+ * computes skip as workload.py:313 does: int(warmup / (last - first arrival) *
+ * R); 0 keeps every request).  Of the accepted requests of a model inside that
+ * window: their number, the arrival times of the first and the last one
+ * (throughput = number / (last - first), :337), the sum, mean and standard
+ * deviation of their latencies finish - arrival (np.mean / np.std, :349) and
+ * the order statistics sorted[int(0.90 * n)], sorted[int(0.99 * n)] (:344-346).
+ * A model none of whose requests was accepted reports 0 for all of them, as
+ * the reference's latency = [0] does (:340-342).
+ *
+ * Counts, times and the two percentiles are exact.  Sum, mean and deviation
+ * are compensated sums: within 1e-14 relative of the exact value, hence within
+ * 1e-12 of numpy's pairwise sums, but not bit-equal to them.
+ *
+ * The batch must have been created with MMSIM_WANT_PER_REQUEST and run;
+ * `workloads` are the n_streams streams it was created with (their per-model
+ * request lists are read; the batch keeps no copy of them).  Call
+ * mmsim_batch_fetch as well to learn of simulations that failed. */
+typedef struct {
+    int32_t *model_num_requests; /* requests of the model inside the window     */
+    int32_t *model_num_good;     /* accepted ones among them                     */
+    double *first_start;         /* arrival of the first accepted request        */
+    double *last_start;          /* arrival of the last accepted request         */
+    double *latency_sum;
+    double *latency_mean;
+    double *latency_std;
+    double *latency_p90;
+    double *latency_p99;
+} mmsim_model_stats;
+int mmsim_batch_model_stats(mmsim_batch *batch, const mmsim_workload *const *workloads, int32_t n_streams,
+                            const int64_t *skip, mmsim_model_stats *out);
 void mmsim_batch_destroy(mmsim_batch *batch);
 
 /*

@@ -54,6 +54,13 @@ class DeviceInfo(C.Structure):
                 ("clock_khz", C.c_int32), ("lds_bytes_per_block", C.c_int32), ("hbm_bytes", C.c_int64)]
 
 
+class ModelStats(C.Structure):
+    _fields_ = [("model_num_requests", _p_i32), ("model_num_good", _p_i32),
+                ("first_start", _p_f64), ("last_start", _p_f64), ("latency_sum", _p_f64),
+                ("latency_mean", _p_f64), ("latency_std", _p_f64), ("latency_p90", _p_f64),
+                ("latency_p99", _p_f64)]
+
+
 class BatchInfo(C.Structure):
     _fields_ = [("lanes", C.c_int32), ("waves", C.c_int32), ("n_seeds", C.c_int32), ("B", C.c_int32),
                 ("smax_bucket", C.c_int32), ("max_replicas", C.c_int32), ("slots", C.c_int32),
@@ -77,6 +84,8 @@ SIGNATURES = {
     "mmsim_batch_run": (C.c_int, [C.c_void_p]),
     "mmsim_batch_sync": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
     "mmsim_batch_fetch": (C.c_int, [C.c_void_p, C.POINTER(Result)]),
+    "mmsim_batch_model_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(C.c_int64),
+                                           C.POINTER(ModelStats)]),
     "mmsim_batch_destroy": (None, [C.c_void_p]),
     "mmsim_batch_get_info": (C.c_int, [C.c_void_p, C.POINTER(BatchInfo)]),
     "mmsim_batch_kernel_name": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t]),

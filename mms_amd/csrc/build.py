@@ -16,7 +16,7 @@ PKG = os.path.dirname(HERE)
 OUT = os.path.join(PKG, "libmmsim.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["mmsim_api.hip", "sim_mixed.hip", "sim_batching.hip", "sim_scalar.hip"]
+SOURCES = ["mmsim_api.hip", "sim_mixed.hip", "sim_batching.hip", "sim_scalar.hip", "stats.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -48,7 +48,7 @@ def build(verbose=False, extra_flags=(), src_dir=HERE, out=OUT):
     """Compiles SOURCES from `src_dir` and links them into `out`."""
     obj_dir = os.path.join(src_dir, "build")
     os.makedirs(obj_dir, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as pool:
         results = list(pool.map(lambda s: _compile(s, list(extra_flags), src_dir, obj_dir), SOURCES))
     objs = [o for o, _ in results]
     if verbose:

@@ -1134,6 +1134,7 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
     *out = nullptr;
     if (R < 0 || M < 1) return fail(MMSIM_E_INVALID, "workload_create: R must be >= 0 and M >= 1");
     if (R > 0 && (!tstamps || !model_ids || !slos)) return fail(MMSIM_E_INVALID, "workload_create: null array");
+    if (R > 0x7FFFFFFF) return fail(MMSIM_E_UNSUPPORTED, "workload_create: more than 2^31-1 requests");
     std::unique_ptr<mmsim_workload> w(new (std::nothrow) mmsim_workload);
     if (!w) return fail(MMSIM_E_NOMEM, "host allocation failed");
     w->ctx = ctx;
@@ -1141,6 +1142,7 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
     w->M = M;
     w->model_num_requests.assign(M, 0);
     std::vector<Req> host((size_t)R);
+    bool sorted = true;
     for (int64_t i = 0; i < R; ++i) {
         if (model_ids[i] >= M) return fail(MMSIM_E_INVALID, "workload_create: model id >= M");
         if (tstamps[i] != tstamps[i]) return fail(MMSIM_E_INVALID, "workload_create: arrival time is NaN");
@@ -1149,20 +1151,26 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
         host[i].slo = slos[i];
         if (model_ids[i] >= 0) w->model_num_requests[model_ids[i]] += 1;
         if (i > 0 && host[i].m == host[i - 1].m) w->repeats += 1;
+        if (i > 0 && tstamps[i] < tstamps[i - 1]) sorted = false;
     }
     w->mq_off.assign((size_t)M + 1, 0);
     for (int32_t m = 0; m < M; ++m) w->mq_off[m + 1] = w->mq_off[m] + w->model_num_requests[m];
     const size_t known = (size_t)w->mq_off[M];
     std::vector<MqEntry> mq(known);
     {
-        // dense rank of every arrival time (streams are normally sorted; this does not rely on it)
-        std::vector<int32_t> order((size_t)R), rank((size_t)R, 0);
-        for (int64_t i = 0; i < R; ++i) order[(size_t)i] = (int32_t)i;
-        std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) { return tstamps[x] < tstamps[y]; });
-        int32_t r = 0;
-        for (int64_t k = 0; k < R; ++k) {
-            if (k > 0 && tstamps[order[(size_t)k]] != tstamps[order[(size_t)k - 1]]) ++r;
-            rank[(size_t)order[(size_t)k]] = r;
+        // dense rank of every arrival time: one pass over a sorted stream (the normal case), a sort otherwise
+        std::vector<int32_t> rank((size_t)R, 0);
+        if (sorted) {
+            for (int64_t i = 1; i < R; ++i) rank[(size_t)i] = rank[(size_t)i - 1] + (tstamps[i] != tstamps[i - 1] ? 1 : 0);
+        } else {
+            std::vector<int32_t> order((size_t)R);
+            for (int64_t i = 0; i < R; ++i) order[(size_t)i] = (int32_t)i;
+            std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) { return tstamps[x] < tstamps[y]; });
+            int32_t r = 0;
+            for (int64_t k = 0; k < R; ++k) {
+                if (k > 0 && tstamps[order[(size_t)k]] != tstamps[order[(size_t)k - 1]]) ++r;
+                rank[(size_t)order[(size_t)k]] = r;
+            }
         }
         std::vector<int64_t> fill(w->mq_off.begin(), w->mq_off.end() - 1);
         for (int64_t i = 0; i < R; ++i)
@@ -1175,7 +1183,6 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
                 e.pad[0] = e.pad[1] = 0;
             }
     }
-    if (R > 0x7FFFFFFF) return fail(MMSIM_E_UNSUPPORTED, "workload_create: more than 2^31-1 requests");
     HIP_TRY(hipSetDevice(ctx->device));
     HIP_TRY(w->reqs.alloc((size_t)R));
     HIP_TRY(w->mq.alloc(known));
@@ -1250,10 +1257,9 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
     if (!b->ran) return fail(MMSIM_E_INVALID, "batch_fetch: batch was never run");
     if (!out->n_good || !out->latency_sum) return fail(MMSIM_E_INVALID, "batch_fetch: n_good and latency_sum are required");
     const bool wm = b->flags & MMSIM_WANT_MODEL_COUNTS, wg = b->flags & MMSIM_WANT_GROUP_COUNTS,
-               wr = b->flags & MMSIM_WANT_PER_REQUEST;
+               wr = (b->flags & MMSIM_WANT_PER_REQUEST) && out->finish && out->good;  // left on the device if not asked for
     if (wm && (!out->model_num_requests || !out->model_num_good)) return fail(MMSIM_E_INVALID, "batch_fetch: model count arrays missing");
     if (wg && (!out->group_num_requests || !out->group_num_good)) return fail(MMSIM_E_INVALID, "batch_fetch: group count arrays missing");
-    if (wr && (!out->finish || !out->good)) return fail(MMSIM_E_INVALID, "batch_fetch: per-request arrays missing");
     HIP_TRY(hipSetDevice(b->ctx->device));
     HIP_TRY(hipStreamSynchronize(b->ctx->stream));
 
@@ -1362,6 +1368,89 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
         return fail(any_bad, any_bad == MMSIM_E_OVERFLOW
                                  ? "a simulation ran out of idle-event slots; its results are invalid (pass status[] to see which)"
                                  : "a simulation hit an input the batching simulator does not support (all replica clocks infinite)");
+    return MMSIM_OK;
+}
+
+int mmsim_batch_model_stats(mmsim_batch *b, const mmsim_workload *const *workloads, int32_t n_streams,
+                            const int64_t *skip, mmsim_model_stats *out) {
+    if (!b || !workloads || !skip || !out) return fail(MMSIM_E_INVALID, "batch_model_stats: null pointer");
+    if (!b->ran) return fail(MMSIM_E_INVALID, "batch_model_stats: batch was never run");
+    if (!(b->flags & MMSIM_WANT_PER_REQUEST))
+        return fail(MMSIM_E_INVALID, "batch_model_stats: the batch was created without MMSIM_WANT_PER_REQUEST");
+    if (n_streams != b->n_seeds) return fail(MMSIM_E_INVALID, "batch_model_stats: pass the request streams the batch was created with");
+    if (!out->model_num_requests || !out->model_num_good || !out->first_start || !out->last_start || !out->latency_sum ||
+        !out->latency_mean || !out->latency_std || !out->latency_p90 || !out->latency_p99)
+        return fail(MMSIM_E_INVALID, "batch_model_stats: every result array is required");
+    const int32_t B = b->B, M = b->M, tiles = b->tiles;
+    std::vector<const MqEntry *> mq((size_t)n_streams);
+    std::vector<int64_t> mqo((size_t)n_streams * (M + 1)), lo((size_t)n_streams), hi((size_t)n_streams);
+    for (int s = 0; s < n_streams; ++s) {
+        const mmsim_workload *w = workloads[s];
+        if (!w || w->ctx != b->ctx || w->M != M || w->R != b->wl_R[(size_t)s])
+            return fail(MMSIM_E_INVALID, "batch_model_stats: pass the request streams the batch was created with");
+        if (skip[s] < 0) return fail(MMSIM_E_INVALID, "batch_model_stats: negative skip");
+        mq[(size_t)s] = w->mq.p;
+        for (int32_t m = 0; m <= M; ++m) mqo[(size_t)s * (M + 1) + m] = w->mq_off[(size_t)m];
+        lo[(size_t)s] = std::min<int64_t>(skip[s], w->R);   // start[skip:-skip], workload.py:315-318
+        hi[(size_t)s] = std::max<int64_t>(lo[(size_t)s], w->R - skip[s]);
+    }
+    HIP_TRY(hipSetDevice(b->ctx->device));
+    hipStream_t st = b->ctx->stream;
+    const size_t cells = (size_t)b->waves * (size_t)M * kWave;
+    DevBuf<const MqEntry *> d_mq;
+    DevBuf<int64_t> d_i64;   // mq_off | lo | hi
+    DevBuf<int32_t> d_i32;   // model_req | model_good
+    DevBuf<double> d_f64;    // the seven double results
+    HIP_TRY(d_mq.alloc(mq.size()));
+    HIP_TRY(d_i64.alloc(mqo.size() + 2 * (size_t)n_streams));
+    HIP_TRY(d_i32.alloc(2 * cells));
+    HIP_TRY(d_f64.alloc(7 * cells));
+    HIP_TRY(hipMemcpyAsync(d_mq.p, mq.data(), sizeof(mq[0]) * mq.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_i64.p, mqo.data(), sizeof(int64_t) * mqo.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_i64.p + mqo.size(), lo.data(), sizeof(int64_t) * lo.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_i64.p + mqo.size() + lo.size(), hi.data(), sizeof(int64_t) * hi.size(), hipMemcpyHostToDevice, st));
+    StatsArgs a{};
+    a.finish = b->finish.p;
+    a.good = b->good.p;
+    a.mq = d_mq.p;
+    a.mq_off = d_i64.p;
+    a.lo = d_i64.p + mqo.size();
+    a.hi = a.lo + n_streams;
+    a.tile_seed = b->tile_seed.p;
+    a.paired = b->paired ? 1 : 0;
+    a.tiles = tiles;
+    a.M = M;
+    a.Rmax = b->Rmax;
+    a.model_req = d_i32.p;
+    a.model_good = d_i32.p + cells;
+    double *f = d_f64.p;
+    a.first_start = f;
+    a.last_start = f + cells;
+    a.latency_sum = f + 2 * cells;
+    a.latency_mean = f + 3 * cells;
+    a.latency_std = f + 4 * cells;
+    a.latency_p90 = f + 5 * cells;
+    a.latency_p99 = f + 6 * cells;
+    std::string err;
+    hipError_t e = launch_model_stats(a, b->waves, st, &err);
+    if (e != hipSuccess) return fail(MMSIM_E_HIP, err.empty() ? std::string("model_stats launch: ") + hipGetErrorString(e) : err);
+    std::vector<int32_t> h32(2 * cells);
+    std::vector<double> h64(7 * cells);
+    HIP_TRY(hipMemcpyAsync(h32.data(), d_i32.p, sizeof(int32_t) * h32.size(), hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipMemcpyAsync(h64.data(), d_f64.p, sizeof(double) * h64.size(), hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    int32_t *const o32[2] = {out->model_num_requests, out->model_num_good};
+    double *const o64[7] = {out->first_start, out->last_start, out->latency_sum, out->latency_mean,
+                            out->latency_std, out->latency_p90, out->latency_p99};
+    for (int s = 0; s < b->out_seeds; ++s)
+        for (int32_t p = 0; p < B; ++p) {
+            const size_t wave = (size_t)s * tiles + b->pos[p] / kWave, lane = (size_t)(b->pos[p] % kWave);
+            for (int32_t m = 0; m < M; ++m) {
+                const size_t src = (wave * M + m) * kWave + lane, dst = ((size_t)s * B + p) * M + m;
+                for (int k = 0; k < 2; ++k) o32[k][dst] = h32[(size_t)k * cells + src];
+                for (int k = 0; k < 7; ++k) o64[k][dst] = h64[(size_t)k * cells + src];
+            }
+        }
     return MMSIM_OK;
 }
 

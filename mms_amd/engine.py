@@ -284,10 +284,26 @@ class Batch:
         _lib.check(self.engine.lib.mmsim_batch_kernel_name(self._h, buf, len(buf)))
         return buf.value.decode()
 
-    def fetch(self):
-        out, r = _result_arrays(self.flags, self.n_seeds, self.B, self.M, self.Gmax, self.Rmax)
+    def fetch(self, per_request=True):
+        """Results of the last run.  ``per_request=False`` leaves finish / good of a
+        ``WANT_PER_REQUEST`` batch on the device (for ``model_stats``)."""
+        flags = self.flags if per_request else self.flags & ~_lib.WANT_PER_REQUEST
+        out, r = _result_arrays(flags, self.n_seeds, self.B, self.M, self.Gmax, self.Rmax)
         _lib.check(self.engine.lib.mmsim_batch_fetch(self._h, C.byref(r)))
         return _shape_results(out, self.n_seeds, self.B)
+
+    def model_stats(self, skip):
+        """Per (simulation, model) statistics of the last run's per-request outputs, computed on
+        the device (``mmsim_batch_model_stats``; workload.py:308-354).  ``skip[s]`` requests are
+        trimmed at either end of stream ``s``.  Arrays are [n_seeds][B][M]."""
+        L = self.n_seeds * self.B
+        out = {f[0]: np.zeros((L, self.M), np.int32 if f[1] is _lib._p_i32 else np.float64)
+               for f in _lib.ModelStats._fields_}
+        r = _lib.ModelStats(*[_lib.ptr(out[f[0]], f[1]._type_) for f in _lib.ModelStats._fields_])
+        wl = (C.c_void_p * self.n_seeds)(*[w._h for w in self.workloads])
+        sk = (C.c_int64 * self.n_seeds)(*[int(x) for x in skip])
+        _lib.check(self.engine.lib.mmsim_batch_model_stats(self._h, wl, self.n_seeds, sk, C.byref(r)))
+        return {k: v.reshape(self.n_seeds, self.B, self.M) for k, v in out.items()}
 
     def close(self):
         if self._h:

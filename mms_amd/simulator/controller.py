@@ -205,10 +205,15 @@ def simulate_replacements(sols, model_names, prof_ress, model_ids, slos, arrival
 
 def approximate_one_case(case: ServingCase, seed: int = 0, warmup: int = DEFAULT_WARMUP,
                          debug: bool = False, fast_stats: bool = False,
-                         enable_batching: bool = False):
+                         enable_batching: bool = False, per_request_arrays: bool = False):
     """Score one serving case with the approximate simulator
     (controller.py:308-407).  ``seed`` and ``debug`` are accepted and unused,
-    as in the reference; ``warmup`` only matters when ``fast_stats`` is off."""
+    as in the reference; ``warmup`` only matters when ``fast_stats`` is off.
+
+    With ``fast_stats`` off the statistics of a ``ModelPlacement`` are computed on the GPU
+    (``device_compute_stats``) and finish / good are never copied to the host;
+    ``per_request_arrays=True`` takes the host path instead (``Workload.compute_stats`` on the copied
+    arrays), which also fills the per-request arrays of each ``PerModelStatsResult``."""
     from mms_amd.placement_policy.base_policy import (ModelPlacement,
                                                       ModelPlacementWithReplacement)
 
@@ -232,6 +237,9 @@ def approximate_one_case(case: ServingCase, seed: int = 0, warmup: int = DEFAULT
             workload.cached_data = (model_ids, slos, model_names, prof_ress)
 
     arrivals = workload.arrivals
+    if isinstance(placement, ModelPlacement) and not fast_stats and not per_request_arrays:
+        return device_compute_stats(workload, [placement], model_names, prof_ress, model_ids, slos, warmup,
+                                    enable_batching=enable_batching)[0], placement
     if isinstance(placement, ModelPlacement):
         (start, finish, good, model_num_requests, model_num_good_requests,
          group_num_requests, group_num_good_requests) = approximate_one_case_one_placement(
@@ -259,6 +267,87 @@ def approximate_one_case(case: ServingCase, seed: int = 0, warmup: int = DEFAULT
         stats = workload.compute_stats(start, finish, good, warmup)
         stats.group_num_requests = tuple(group_num_requests)
     return stats, placement
+
+
+def warmup_skip(arrivals, warmup):
+    """Requests that Workload.compute_stats trims at either end (workload.py:312-314); 0: none."""
+    if len(arrivals) > 1:
+        return max(int(warmup / (arrivals[-1] - arrivals[0]) * len(arrivals)), 0)
+    return 0
+
+
+def device_compute_stats(workload, sols, model_names, prof_ress, model_ids, slos, warmup,
+                         enable_batching=False, table=None, device_workload=None):
+    """``Workload.compute_stats`` (workload.py:308-354) for every placement in ``sols``, with the
+    per-request outputs left on the GPU: one launch simulates all placements, a second one
+    (``mmsim_batch_model_stats``) reduces finish / good to per-model counts, first and last
+    accepted arrival, latency mean / deviation and the two percentiles inside the warm-up window.
+
+    Returns one ``StatsResult`` per placement.  Counts, goodput, throughput, p90 and p99 equal the
+    reference's; means and deviations are within 1e-12 relative (compensated sums on the device,
+    pairwise sums in numpy).  The per-request arrays of ``PerModelStatsResult`` (``latency``,
+    ``request_starts``, ``request_finishes``) are ``None``: they never leave the device.
+    """
+    eng = _engine.Engine.default()
+    arrivals = np.asarray(workload.arrivals, dtype=np.float64)
+    R = len(arrivals)
+    if table is None:
+        table = _engine.LatencyTable(prof_ress, list(batchsize_config) if enable_batching else [1])
+    flags = _lib.WANT_GROUP_COUNTS | _lib.WANT_PER_REQUEST | (_lib.BATCHING if enable_batching else 0)
+    own = device_workload is None
+    dw = _engine.DeviceWorkload(eng, arrivals, model_ids, slos, len(model_names)) if own else device_workload
+    batch = _engine.Batch(eng, [dw], table, _engine.pack_placements(sols, table), flags)
+    try:
+        batch.run()
+        batch.sync()
+        out = batch.fetch(per_request=False)
+        skip = warmup_skip(arrivals, warmup)
+        ms = batch.model_stats([skip])
+    finally:
+        batch.close()
+        if own:
+            dw.close()
+
+    lo, hi = (skip, R - skip) if skip > 0 else (0, R)
+    ids = np.asarray(model_ids[lo:hi])
+    n_window = len(ids)
+    # models in the order of their first request inside the window, then (stable) by request count
+    # (workload.py:321-327); a request of a model that was never registered (id -1) is listed under its name
+    entries = {}
+    placed, first_at = np.unique(ids[ids >= 0], return_index=True)
+    first_at = np.nonzero(ids >= 0)[0][first_at] if len(placed) else first_at
+    for m, at in zip(placed, first_at):
+        entries[model_names[m]] = [int(at), 0, int(m)]
+    for i in np.nonzero(ids < 0)[0]:
+        name = workload.requests[lo + int(i)].model_name
+        if name not in entries:
+            entries[name] = [int(i), 0, -1]
+        entries[name][1] += 1
+    ordered = sorted(entries.items(), key=lambda kv: kv[1][0])
+    interval = arrivals[hi - 1] - arrivals[lo]
+
+    results = []
+    for b, sol in enumerate(sols):
+        st = {k: v[0, b] for k, v in ms.items()}
+        rows = []
+        for name, (_, count, m) in ordered:
+            if m < 0:
+                rows.append(PerModelStatsResult(name, count, np.float64(0), 0, np.float64(0), np.float64(0),
+                                                0, 0, None, None, None))
+                continue
+            n_req, n_good = int(st["model_num_requests"][m]), int(st["model_num_good"][m])
+            goodput = np.float64(n_good) / n_req
+            throughput = n_good / (st["last_start"][m] - st["first_start"][m]) if n_good > 0 else 0
+            rows.append(PerModelStatsResult(name, n_req, goodput, throughput, st["latency_mean"][m],
+                                            st["latency_std"][m], st["latency_p90"][m], st["latency_p99"][m],
+                                            None, None, None))
+        rows.sort(key=lambda r: r.num_requests)     # stable
+        total_good = int(st["model_num_good"].sum())
+        stats = StatsResult(rows, tuple(out["group_num_requests"][0, b][:len(sol.group_configs)]),
+                            np.float64(total_good) / n_window, np.sum(st["latency_sum"]) / n_window,
+                            n_window, n_window / interval)
+        results.append(stats)
+    return results
 
 
 def replacement_fast_stats(model_names, arrivals, res):

@@ -83,6 +83,76 @@ def _eval_pairs(engine, workloads, table, packed, stream_of, flags=0, fixed_over
     return res
 
 
+def model_stats_numpy(tstamps, model_ids, finish, good, skip, M):
+    """What mmsim_batch_model_stats returns for one simulation, restated with numpy from the
+    conventions of Workload.compute_stats (workload.py:308-354): window [skip, R - skip), order
+    statistics sorted[int(q * n)], np.mean / np.std of the accepted requests' latencies."""
+    R = len(tstamps)
+    lo, hi = min(skip, R), max(min(skip, R), R - skip)
+    out = {k: np.zeros(M, np.int32) for k in ("model_num_requests", "model_num_good")}
+    out.update({k: np.zeros(M) for k in ("first_start", "last_start", "latency_sum", "latency_mean",
+                                         "latency_std", "latency_p90", "latency_p99")})
+    ids = model_ids[lo:hi]
+    for m in range(M):
+        sel = np.nonzero(ids == m)[0] + lo
+        ok = sel[np.asarray(good[sel], bool)]
+        out["model_num_requests"][m] = len(sel)
+        out["model_num_good"][m] = len(ok)
+        if len(ok):
+            lat = np.sort(finish[ok] - tstamps[ok])
+            out["first_start"][m], out["last_start"][m] = tstamps[ok[0]], tstamps[ok[-1]]
+            out["latency_sum"][m] = np.sum(lat)
+            out["latency_mean"][m], out["latency_std"][m] = np.mean(lat), np.std(lat)
+            out["latency_p90"][m] = lat[int(0.90 * len(lat))]
+            out["latency_p99"][m] = lat[int(0.99 * len(lat))]
+    return out
+
+
+class _HostBatch:
+    """Stand-in for engine.Batch: run / sync / fetch / model_stats on the oracle's outputs."""
+
+    def __init__(self, engine, workloads, table, packed, flags, fixed_overhead=0.011):
+        self.workloads, self.table, self.packed = list(workloads), table, packed
+        self.flags, self.fixed_overhead = int(flags), fixed_overhead
+        self.n_seeds, self.B, self.M = len(self.workloads), packed[1].shape[0], table.arrays()[0].shape[0]
+        self.out = None
+
+    def run(self):
+        lat, pp = self.table.arrays()
+        num_groups, group_cfg, gm_off, gm_idx = self.packed
+        outs = [oracle_c.eval_placements(
+            w.tstamps, w.model_ids, w.slos, lat, pp, self.table.batch_sizes, num_groups, group_cfg, gm_off,
+            gm_idx, batching=bool(self.flags & _lib.BATCHING), fixed_overhead=self.fixed_overhead,
+            want_counts=True, want_per_request=bool(self.flags & _lib.WANT_PER_REQUEST)) for w in self.workloads]
+        Rmax = max(w.R for w in self.workloads)
+        self.out = {}
+        for k in outs[0]:
+            if k in ("finish", "good"):
+                arr = np.zeros((self.n_seeds, self.B, Rmax), outs[0][k].dtype)
+                for s, o in enumerate(outs):
+                    arr[s, :, :o[k].shape[1]] = o[k]
+                self.out[k] = arr
+            else:
+                self.out[k] = np.stack([o[k] for o in outs])
+        self.out["status"] = np.zeros((self.n_seeds, self.B), np.int32)
+
+    def sync(self):
+        return 0.0
+
+    def fetch(self, per_request=True):
+        return {k: v for k, v in self.out.items() if per_request or k not in ("finish", "good")}
+
+    def model_stats(self, skip):
+        per = [[model_stats_numpy(w.tstamps, w.model_ids, self.out["finish"][s, b, :w.R],
+                                  self.out["good"][s, b, :w.R], int(skip[s]), self.M)
+                for b in range(self.B)] for s, w in enumerate(self.workloads)]
+        return {k: np.array([[per[s][b][k] for b in range(self.B)] for s in range(self.n_seeds)])
+                for k in per[0][0]}
+
+    def close(self):
+        pass
+
+
 def _simulate_requests_mixed(engine, finish, good, tstamps, model_ids, slos, m2g, num_stages, lat,
                              num_requests=None, fixed_overhead=0.011):
     f, g, cnt, _ = oracle_c.simulate_requests_mixed(tstamps, model_ids, slos, m2g, num_stages, lat, fixed_overhead)
@@ -113,6 +183,7 @@ def install(monkeypatch):
     monkeypatch.setattr(E.Engine, "default", classmethod(lambda cls: host))
     monkeypatch.setattr(E, "DeviceWorkload", _HostWorkload)
     monkeypatch.setattr(E, "evaluate", _evaluate)
+    monkeypatch.setattr(E, "Batch", _HostBatch)
     monkeypatch.setattr(E, "eval_pairs", _eval_pairs)
     monkeypatch.setattr(E, "simulate_requests_mixed", _simulate_requests_mixed)
     monkeypatch.setattr(E, "simulate_requests", _simulate_requests)

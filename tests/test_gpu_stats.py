@@ -1,0 +1,94 @@
+"""GPU parity of the statistics kernel (mmsim_batch_model_stats) with
+Workload.compute_stats' conventions (workload.py:308-354).
+
+The kernel reduces the per-request outputs that the simulation kernels left in
+device memory; the check fetches those same outputs and reduces them with
+numpy (``model_stats_numpy``: sort, ``sorted[int(q * n)]``, ``np.mean``,
+``np.std``).  Bars: counts, first / last accepted arrival and both percentiles
+bit-exact; sum, mean and deviation within 1e-12 relative (compensated sums on
+the device, pairwise sums in numpy).
+"""
+import numpy as np
+import pytest
+
+from mms_amd import _lib, engine as E
+from mms_amd.synthetic import make_config
+from oracle_backend import model_stats_numpy
+
+pytestmark = pytest.mark.gpu
+
+EXACT = ("model_num_requests", "model_num_good", "first_start", "last_start", "latency_p90", "latency_p99")
+CLOSE = ("latency_sum", "latency_mean", "latency_std")
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return E.Engine.default()
+
+
+def _check(eng, cfg, sols, seeds, skips, flags=0):
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    streams = [cfg.stream(s) for s in seeds]
+    dws = [E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models) for st in streams]
+    batch = E.Batch(eng, dws, table, E.pack_placements(sols, table), flags | _lib.WANT_PER_REQUEST)
+    batch.run()
+    batch.sync()
+    out = batch.fetch()
+    for skip in skips:
+        got = batch.model_stats(skip)
+        for s, st in enumerate(streams):
+            for b in range(len(sols)):
+                R = len(st.tstamps)
+                want = model_stats_numpy(st.tstamps, st.model_ids, out["finish"][s, b, :R], out["good"][s, b, :R],
+                                         skip[s], cfg.num_models)
+                for k in EXACT:
+                    assert np.array_equal(got[k][s, b], want[k]), (k, s, b, skip)
+                for k in CLOSE:
+                    np.testing.assert_allclose(got[k][s, b], want[k], rtol=1e-12, atol=1e-300, err_msg=f"{k} {s} {b}")
+    batch.close()
+    return out
+
+
+def test_plain_simulator_two_streams_every_window(eng):
+    cfg = make_config(2, 64)
+    R = min(len(cfg.stream(s).tstamps) for s in (0, 1))
+    out = _check(eng, cfg, cfg.placements, (0, 1),
+                 [(0, 0), (1, 7), (R // 10, R // 7), (R // 2 - 1, R // 2 - 1), (R // 2 + 5, R), (3 * R, 0)])
+    assert 0 < out["good"].mean() < 1       # both accepted and rejected requests took part
+
+
+def test_more_placements_than_one_wavefront_and_deep_pipelines(eng):
+    cfg = make_config(4, 96)
+    cfg.duration *= 0.02        # about 20000 requests
+    R = len(cfg.stream(3).tstamps)
+    _check(eng, cfg, cfg.placements, (3,), [(0,), (R // 20,)])
+
+
+def test_batching_simulator(eng):
+    cfg = make_config(5, 24)
+    cfg.duration *= 0.05
+    R = len(cfg.stream(0).tstamps)
+    _check(eng, cfg, cfg.placements, (0,), [(0,), (R // 9,)], flags=_lib.BATCHING)
+
+
+def test_requires_per_request_outputs_and_the_same_streams(eng):
+    cfg = make_config(2, 4)
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    st = cfg.stream(0)
+    dw = E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models)
+    batch = E.Batch(eng, [dw], table, E.pack_placements(cfg.placements, table), 0)
+    batch.run()
+    batch.sync()
+    with pytest.raises(_lib.MmsimError, match="MMSIM_WANT_PER_REQUEST"):
+        batch.model_stats([0])
+    batch.close()
+    batch = E.Batch(eng, [dw], table, E.pack_placements(cfg.placements, table), _lib.WANT_PER_REQUEST)
+    with pytest.raises(_lib.MmsimError, match="never run"):
+        batch.model_stats([0])
+    batch.run()
+    batch.sync()
+    other = E.DeviceWorkload(eng, st.tstamps[:-1], st.model_ids[:-1], st.slos[:-1], cfg.num_models)
+    batch.workloads = [other]
+    with pytest.raises(_lib.MmsimError, match="streams the batch was created with"):
+        batch.model_stats([0])
+    batch.close()

@@ -219,6 +219,45 @@ def test_approximate_one_case_full_stats_and_unknown_model(backend):
     assert fast.num_requests == len(wl)
 
 
+@pytest.mark.parametrize("enable_batching", [False, True], ids=["plain", "batching"])
+def test_device_statistics_equal_compute_stats(backend, monkeypatch, enable_batching):
+    """approximate_one_case(fast_stats=False) reduces finish / good on the device; the reference
+    copies them and calls Workload.compute_stats (controller.py:405, workload.py:308-354).  Same
+    models in the same order, counts, goodput, throughput and percentiles equal; means and
+    deviations to 1e-12 (compensated sums against numpy's pairwise sums)."""
+    import mms_amd.util as U
+    import mms_amd.simulator.controller as ctl
+    from mms_amd.profiling import synthetic_profile
+    monkeypatch.setattr(U, "batchsize_config", [1, 2, 4])
+    monkeypatch.setattr(ctl, "batchsize_config", [1, 2, 4])
+    pcs = [ParallelConfig(1, 1, 1), ParallelConfig(1, 1, 2)]
+    model_datas = [ModelData(f"m{i}", 0.5, rate, 2, synthetic_profile(f"m{i}", 0.1 + 0.01 * i, pcs, (1, 2, 4), 0.2))
+                   for i, rate in enumerate((9, 3, 6, 1))]
+    wl = gen_train_workload(model_datas, simulation_min_samples=4000)
+    extra = [GammaProcess(r, 1).generate_workload(name, 0, wl.arrivals[-1], slo=1.0, seed=s)
+             for name, r, s in (("ghost-a", 0.5, 5), ("ghost-b", 2.0, 6))]
+    wl = Workload.merge(wl, *extra)
+    sol = ModelPlacement([ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 1), ParallelConfig(1, 1, 1)],
+                         [[0, 1, 2], [0, 3], [2]])
+    for warmup in (0, 10, 37.5):
+        got, _ = approximate_one_case(_case(sol, model_datas, wl), warmup=warmup, enable_batching=enable_batching)
+        want, _ = approximate_one_case(_case(sol, model_datas, wl), warmup=warmup, enable_batching=enable_batching,
+                                       per_request_arrays=True)
+        assert [m.name for m in got.per_model_stats] == [m.name for m in want.per_model_stats]
+        assert any(m.latency_p99 > m.latency_p90 > 0 for m in want.per_model_stats)
+        for g, w in zip(got.per_model_stats, want.per_model_stats):
+            assert g.num_requests == w.num_requests
+            for field in ("goodput", "throughput", "latency_p90", "latency_p99"):
+                assert getattr(g, field) == getattr(w, field), (field, g.name, warmup)
+            for field in ("latency_mean", "latency_std"):
+                assert abs(getattr(g, field) - getattr(w, field)) <= 1e-12 * abs(getattr(w, field)), (field, g.name)
+            assert g.latency is None and len(w.latency) >= 1
+        assert got.group_num_requests == want.group_num_requests
+        assert got.goodput == want.goodput and got.num_requests == want.num_requests
+        assert got.request_rate == want.request_rate
+        assert abs(got.latency_mean - want.latency_mean) <= 1e-12 * want.latency_mean
+
+
 def test_placement_with_replacement_is_simulated_per_segment(backend):
     model_datas = four_models(0.5, 6, 2)
     wl = gen_train_workload(model_datas, simulation_min_samples=3000)
