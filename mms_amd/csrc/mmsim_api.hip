@@ -887,8 +887,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             for (int32_t m = 0; m <= M; ++m) mqo[(size_t)s * (M + 1) + m] = total + wls[s]->mq_off[m];
             total += wls[s]->mq_off[M];
         }
-        HIP_TRY(b->mq.alloc((size_t)total + 1));  // one padding entry: the kernel looks one entry past a popped head
-        HIP_TRY(hipMemsetAsync(b->mq.p + total, 0, sizeof(MqEntry), st));
+        // padding entries: the kernel looks one entry past a popped head, and fetches the sixteen entries from a
+        // queue's head on at once, whether they have arrived or not
+        HIP_TRY(b->mq.alloc((size_t)total + kMqPadding));
+        HIP_TRY(hipMemsetAsync(b->mq.p + total, 0, sizeof(MqEntry) * kMqPadding, st));
         int64_t at = 0;
         for (int s = 0; s < n_seeds; ++s) {
             const size_t n = (size_t)wls[s]->mq_off[M];

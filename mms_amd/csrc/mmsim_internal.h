@@ -32,6 +32,7 @@ struct __attribute__((aligned(32))) MqEntry {
     int32_t pad[2];
 };
 static_assert(sizeof(MqEntry) == 32, "MqEntry must be 32 bytes");
+constexpr int kMqPadding = 16;  // zeroed entries behind the last stream's lists
 
 // Group descriptor of the batching simulator: one 32-bit word per (placement,
 // group), kept per lane in LDS; replicas are listed as group indices.
@@ -167,7 +168,7 @@ struct BatchingArgs {
     const Req *streams;          // all seeds' requests, back to back
     const int64_t *stream_off;   // [n_seeds+1]
     const int64_t *mq_off;       // [n_seeds][M+1] offsets into mq of the arrivals of each model
-    const MqEntry *mq;           // model-ordered arrivals of all seeds, plus one padding entry at the end
+    const MqEntry *mq;           // model-ordered arrivals of all seeds, plus kMqPadding zeroed entries at the end
     const uint64_t *rep8;        // as in MixedArgs
     const uint8_t *repx;
     const uint32_t *ginfo;       // [tiles][Gmax+1][64]

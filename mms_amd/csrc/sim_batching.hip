@@ -86,6 +86,7 @@ __device__ __forceinline__ uint32_t oct_get(uint32_t v, int k) {
 __device__ __forceinline__ double oct_get(double v, int k) {
     return __hiloint2double((int)oct_get((uint32_t)__double2hiint(v), k), (int)oct_get((uint32_t)__double2loint(v), k));
 }
+__device__ __forceinline__ float oct_get(float v, int k) { return __uint_as_float(oct_get(__float_as_uint(v), k)); }
 // The lanes of an octet run in lockstep; this marks the places where that matters (all have read a
 // value before any of them overwrites it).  No instruction.
 __device__ __forceinline__ void oct_sync() { __builtin_amdgcn_wave_barrier(); }
@@ -98,6 +99,12 @@ __device__ __forceinline__ double oct_min(double v) {
     v = w < v ? w : v;
     w = oct_swap<2>(v);
     return w < v ? w : v;
+}
+// sum over the octet, in all of its lanes (the same order of additions in every lane)
+__device__ __forceinline__ double oct_sum(double v) {
+    v += oct_swap<0>(v);
+    v += oct_swap<1>(v);
+    return v + oct_swap<2>(v);
 }
 __device__ __forceinline__ uint32_t oct_min(uint32_t v) {
     uint32_t w = oct_swap<0>(v);
@@ -321,7 +328,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     };
 
     // the same for one latency column (the octet's lanes take one column each)
-    auto batch_time_col = [&](double t0, const double *gclk, int stages, uint32_t lat_mg, int col) -> double {
+    // c0 / l0: the clocks and this column's latencies of the first four stages as read (the commit reuses them)
+    auto batch_time_col = [&](double t0, const double *gclk, int stages, uint32_t lat_mg, int col, double(&c0)[4],
+                              float(&l0)[4]) -> double {
         double t = t0;
         for (int k0 = 0; k0 < stages; k0 += 4) {
             double c[4];
@@ -331,6 +340,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 const int k = k0 + u < stages ? k0 + u : stages - 1;
                 c[u] = gclk[k * LS];
                 l[u] = lat_at(lat_mg + (uint32_t)(k * NB + col));
+            }
+            if (k0 == 0) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    c0[u] = c[u];
+                    l0[u] = l[u];
+                }
             }
 #pragma unroll
             for (int u = 1; u < 4; ++u)
@@ -365,27 +381,38 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             int64_t first = 0;
             double deadline = 0.0, first_t = 0.0;
             int bs = 1;
+            // COOP: what this lane fetched of the queue (entry q0 + oj: arrival time, deadline, index, rank; and the
+            // rank of entry q0 + oj + 8), the head that leads the batch, the first four stages as batch_time_col read them
+            double2 hv = {0.0, 0.0};
+            int2 ir = {0, 0};
+            int32_t rank8 = 0;
+            int kfirst = 0;
+            double c0[4] = {0.0, 0.0, 0.0, 0.0};
+            float l0[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             if constexpr (COOP) {
-                // lane j of the octet takes head j of the queue and latency column j
-                double2 hv = *reinterpret_cast<const double2 *>(&a.mq[q0 + (oj < avail ? oj : avail - 1)]);
-                const double tcol = batch_time_col(t0, gclk, stages, lat_mg, oj < NB ? oj : NB - 1);
+                // lane j of the octet takes entry j from the head of the queue on -- all of it, whether it has arrived
+                // yet or not, so that a batch made of these eight needs no further fetch -- and latency column j
+                const MqEntry *ep = &a.mq[q0 + oj];
+                hv = *reinterpret_cast<const double2 *>(ep);
+                ir = *reinterpret_cast<const int2 *>(&ep->idx);
+                rank8 = ep[8].rank;
+                const double tcol = batch_time_col(t0, gclk, stages, lat_mg, oj < NB ? oj : NB - 1, c0, l0);
                 const double alone = oct_get(tcol, 0) + overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
                 for (;;) {
                     const uint32_t pass = oct_ballot(oj < avail && alone <= hv.y);
                     const int k = pass ? __ffs((int)pass) - 1 : avail;  // the heads before k are dropped
                     if (oj < k) {
                         if (want_req) {
-                            const MqEntry e = a.mq[q0 + oj];
-                            fin_out[(size_t)e.idx * kWave] = e.t;
-                            good_out[(size_t)e.idx * kWave] = 0;
+                            fin_out[(size_t)ir.x * kWave] = hv.x;
+                            good_out[(size_t)ir.x * kWave] = 0;
                         }
                     }
                     if (want_group && oj == 0) group_req[g * kWave] += k;
                     if (pass) {
                         found = true;
+                        kfirst = k;
                         first = q0 + k;
                         deadline = oct_get(hv.y, k);
-                        first_t = oct_get(hv.x, k);
                         h += (uint32_t)(k + 1);
                         break;
                     }
@@ -393,7 +420,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                     if (h == arr) break;
                     q0 = base + h;
                     avail = (int)(arr - h) < 8 ? (int)(arr - h) : 8;
-                    hv = *reinterpret_cast<const double2 *>(&a.mq[q0 + (oj < avail ? oj : avail - 1)]);
+                    ep = &a.mq[q0 + oj];
+                    hv = *reinterpret_cast<const double2 *>(ep);
+                    ir = *reinterpret_cast<const int2 *>(&ep->idx);
+                    rank8 = ep[8].rank;
                 }
                 if (found) {
                     // grow the batch while the first request still meets its deadline (:693-702): lane b tests
@@ -468,19 +498,34 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 if (m < 0) return;
                 continue;
             }
-            // run it (:715-732); the rank of the arrival after the batch is fetched meanwhile
-            const int32_t next_rank = a.mq[first + bs].rank;
+            // run it (:715-732).  The rank of the arrival after the batch: one of the sixteen the octet fetched, or
+            // fetched while the stages are walked
             const int col = ilog2i(bs);
+            int32_t next_rank;
+            if constexpr (COOP) {
+                const int kb = kfirst + bs;
+                next_rank = (int32_t)oct_get((uint32_t)(kb < 8 ? ir.y : rank8), kb & 7);
+            } else {
+                next_rank = a.mq[first + bs].rank;
+            }
             double t = t0 + overhead;
             double idle_at = 0.0;
             for (int k0 = 0; k0 < stages; k0 += 4) {
                 double c[4];
                 float l[4];
+                if (COOP && k0 == 0) {  // as batch_time_col read them; the latencies are those of the lane that took this column
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int k = k0 + u < stages ? k0 + u : stages - 1;
-                    c[u] = gclk[k * LS];
-                    l[u] = lat_at(lat_mg + (uint32_t)(k * NB + col));
+                    for (int u = 0; u < 4; ++u) {
+                        c[u] = c0[u];
+                        l[u] = oct_get(l0[u], col);
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int k = k0 + u < stages ? k0 + u : stages - 1;
+                        c[u] = gclk[k * LS];
+                        l[u] = lat_at(lat_mg + (uint32_t)(k * NB + col));
+                    }
                 }
                 if constexpr (OCT) oct_sync();
 #pragma unroll
@@ -493,6 +538,27 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             }
             head[m * LS] = h + (uint32_t)(bs - 1);  // the batch is the arrivals first .. first+bs-1 of the model
             hrank[m * LS] = next_rank;
+            if constexpr (COOP) {
+                // the batch is the entries kfirst .. kfirst + bs - 1 of those fetched: each lane accounts for its own
+                // (the octet's latency sums are added up at the end)
+                if (oj >= kfirst && oj < kfirst + bs) {
+                    lat_sum += t - hv.x;
+                    if (want_req) {
+                        fin_out[(size_t)ir.x * kWave] = t;
+                        good_out[(size_t)ir.x * kWave] = 1;
+                    }
+                }
+                for (int u = 8 - kfirst; u < bs; ++u) {  // members behind those eight (heads were dropped first): rare
+                    const MqEntry e = a.mq[first + u];
+                    if (oj == 0) {
+                        lat_sum += t - e.t;
+                        if (want_req) {
+                            fin_out[(size_t)e.idx * kWave] = t;
+                            good_out[(size_t)e.idx * kWave] = 1;
+                        }
+                    }
+                }
+            } else {
             lat_sum += t - first_t;  // the first member's arrival time came with its deadline
             if (want_req) {
                 const int32_t r = a.mq[first].idx;
@@ -511,6 +577,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                         good_out[(size_t)r * kWave] = 1;
                     }
                 }
+            }
             }
             n_good += bs;
             if (want_group && oj == 0) {  // the lanes of an octet would all add
@@ -753,6 +820,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         handle(ti, m2, g);
     }
 
+    if constexpr (COOP) lat_sum = oct_sum(lat_sum);  // each lane summed the batch members it had fetched
     if (oj == 0) {
         const size_t out = (size_t)wave * kWave + sl;
         a.n_good[out] = n_good;
