@@ -91,36 +91,36 @@ __device__ __forceinline__ float oct_get(float v, int k) { return __uint_as_floa
 // value before any of them overwrites it).  No instruction.
 __device__ __forceinline__ void oct_sync() { __builtin_amdgcn_wave_barrier(); }
 // </octet primitives>
-// minimum over the octet, in all of its lanes (doubles are never NaN here)
+// Minimum over the octet, in all of its lanes.  One DPP instruction per step: v_min_u32_dpp d, d, d =
+// min(d of the lane the pattern names, d); a DPP operand needs two wait states after the write of its
+// register (s_nop 1).
+__device__ __forceinline__ uint32_t oct_min(uint32_t v) {
+    asm("s_nop 1\n"
+        "v_min_u32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n"
+        "s_nop 1\n"
+        "v_min_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n"
+        "s_nop 1\n"
+        "v_min_u32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n"
+        : "+v"(v));
+    return v;
+}
+// 64 bits: the smallest high word, then the smallest low word among the lanes that have it
+__device__ __forceinline__ uint64_t oct_min(uint64_t v) {
+    const uint32_t hi = (uint32_t)(v >> 32), lo = (uint32_t)v;
+    const uint32_t mh = oct_min(hi);
+    const uint32_t ml = oct_min(hi == mh ? lo : 0xFFFFFFFFu);
+    return ((uint64_t)mh << 32) | ml;
+}
+// Doubles that are never negative nor NaN (clocks and event times: they start at +0 and only ever
+// grow by latencies >= 0; +inf is allowed) order as their bit patterns do.
 __device__ __forceinline__ double oct_min(double v) {
-    double w = oct_swap<0>(v);
-    v = w < v ? w : v;
-    w = oct_swap<1>(v);
-    v = w < v ? w : v;
-    w = oct_swap<2>(v);
-    return w < v ? w : v;
+    return __longlong_as_double((long long)oct_min((uint64_t)__double_as_longlong(v)));
 }
 // sum over the octet, in all of its lanes (the same order of additions in every lane)
 __device__ __forceinline__ double oct_sum(double v) {
     v += oct_swap<0>(v);
     v += oct_swap<1>(v);
     return v + oct_swap<2>(v);
-}
-__device__ __forceinline__ uint32_t oct_min(uint32_t v) {
-    uint32_t w = oct_swap<0>(v);
-    v = w < v ? w : v;
-    w = oct_swap<1>(v);
-    v = w < v ? w : v;
-    w = oct_swap<2>(v);
-    return w < v ? w : v;
-}
-__device__ __forceinline__ uint64_t oct_min(uint64_t v) {
-    uint64_t w = oct_swap<0>(v);
-    v = w < v ? w : v;
-    w = oct_swap<1>(v);
-    v = w < v ? w : v;
-    w = oct_swap<2>(v);
-    return w < v ? w : v;
 }
 
 typedef volatile __attribute__((address_space(3))) uint32_t lds_vu32;
