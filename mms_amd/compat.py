@@ -21,6 +21,7 @@ _ALIASES = {
     "alpa_serve.simulator.workload": "mms_amd.simulator.workload",
     "alpa_serve.simulator.controller": "mms_amd.simulator.controller",
     "alpa_serve.simulator.executable": "mms_amd.simulator.executable",
+    "alpa_serve.trace": "mms_amd.trace",
     "alpa_serve.placement_policy": "mms_amd.placement_policy",
     "alpa_serve.placement_policy.base_policy": "mms_amd.placement_policy.base_policy",
     "alpa_serve.placement_policy.model_parallelism": "mms_amd.placement_policy.model_parallelism",

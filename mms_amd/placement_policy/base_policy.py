@@ -158,17 +158,17 @@ class PlacementEvaluator:
     reused across calls, which is what ``workload.cached_data`` does for the
     reference's per-placement loop (:155, :170, controller.py:323-339).
 
-    ``method`` must be "fast_simulator": the event-driven simulator is not
-    part of this package.  ``parallel`` selected one Ray task per placement
-    in the reference; the GPU batch already evaluates placements in parallel,
-    so the flag is accepted and has no effect.
+    ``method`` "fast_simulator" is the GPU path.  Any other method is, as in the
+    reference (:172-174, :199-224), the event-driven simulator
+    (``mms_amd.simulator.event_sim``): host code, one placement after another,
+    meant as a slower cross-check of a few placements, not for searches.
+    ``parallel`` selected one Ray task per placement in the reference; the GPU
+    batch already evaluates placements in parallel, so the flag is accepted and
+    has no effect.
     """
 
     def __init__(self, model_datas: List[ModelData], cluster_env: ClusterEnv, workload: Workload,
                  method: str, parallel: bool, enable_batching: bool = False):
-        if method != "fast_simulator":
-            raise NotImplementedError(
-                f"evaluator method {method!r}: only 'fast_simulator' is available")
         self.parallel = parallel
         self.model_datas = model_datas
         self.cluster_env = cluster_env
@@ -248,6 +248,9 @@ class PlacementEvaluator:
         """goodput - latency_mean/10000 + num_replicas/1e6 per placement (:225-226)."""
         if len(sols) == 0:
             return []
+        if self.method != "fast_simulator":
+            return [self.get_goodput_simulation(sol, self.model_datas, self.cluster_env, self.workload, self.method)
+                    for sol in sols]
         if not self._is_plain(sols):
             return [st.goodput - st.latency_mean / 10000 + self._num_replicas(sol) / 1000000
                     for sol, st in zip(sols, self._mixed_stats(sols))]
@@ -264,6 +267,9 @@ class PlacementEvaluator:
         placement (:263-264) with the fast statistics of controller.py:393-403."""
         if len(sols) == 0:
             return []
+        if self.method != "fast_simulator":
+            return [self.get_stats_simulation(sol, self.model_datas, self.cluster_env, self.workload, self.method)
+                    for sol in sols]
         if not self._is_plain(sols):
             return [(st.goodput, [x.goodput for x in st.per_model_stats], st.group_num_requests, st)
                     for st in self._mixed_stats(sols)]
@@ -287,10 +293,7 @@ class PlacementEvaluator:
 
     # -- one placement at a time, same signatures as the reference's static methods -----
     @staticmethod
-    def _serving_case(sol, model_datas, workload, method):
-        if method != "fast_simulator":
-            raise NotImplementedError("only 'fast_simulator' is available")
-
+    def _serving_case(sol, model_datas, cluster_env, workload, method):
         def register_models(controller):
             for data in model_datas:
                 controller.register_model.remote(
@@ -300,14 +303,24 @@ class PlacementEvaluator:
             return workload
 
         def place_models(controller):
-            return sol
+            if method == "fast_simulator":
+                return sol
+            # the event-driven simulator builds the groups and replicas on its controller (:216-218)
+            BasePlacementPolicy().place_models_impl(controller, cluster_env, model_datas, sol)
 
         return ServingCase(register_models, generate_workload, place_models)
 
     @staticmethod
+    def _one_case(sol, model_datas, cluster_env, workload, method):
+        case = PlacementEvaluator._serving_case(sol, model_datas, cluster_env, workload, method)
+        if method == "fast_simulator":
+            return approximate_one_case(case, fast_stats=True)[0]
+        from mms_amd.simulator.event_sim import simulate_one_case
+        return simulate_one_case(case)[0]
+
+    @staticmethod
     def get_goodput_simulation(sol, model_datas, cluster_env, workload, method):
-        case = PlacementEvaluator._serving_case(sol, model_datas, workload, method)
-        stats, _ = approximate_one_case(case, fast_stats=True)
+        stats = PlacementEvaluator._one_case(sol, model_datas, cluster_env, workload, method)
         if isinstance(sol, ModelPlacement):
             num_replicas = sum(len(x) for x in sol.group_models)
         else:
@@ -316,8 +329,7 @@ class PlacementEvaluator:
 
     @staticmethod
     def get_stats_simulation(sol, model_datas, cluster_env, workload, method):
-        case = PlacementEvaluator._serving_case(sol, model_datas, workload, method)
-        stats, _ = approximate_one_case(case, fast_stats=True)
+        stats = PlacementEvaluator._one_case(sol, model_datas, cluster_env, workload, method)
         return (stats.goodput, [x.goodput for x in stats.per_model_stats],
                 stats.group_num_requests, stats)
 

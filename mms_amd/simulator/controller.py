@@ -8,8 +8,9 @@ reference JIT-compiles with numba (:561-628, :631-798) run as HIP kernels
 behind ``libmmsim``; nothing here computes a simulation on the CPU.
 
 The event-driven simulator of the same reference file (``Controller``,
-``GroupManager``, ``Client``, ``simulate_one_case``, :30-279) is a different,
-slow path and is not provided.
+``GroupManager``, ``Client``, ``simulate_one_case``, :30-279) is host code in
+``mms_amd.simulator.event_sim``; its names are re-exported here, where the
+reference has them.
 """
 from functools import partial
 from typing import Callable
@@ -21,6 +22,7 @@ from mms_amd.profiling import ProfilingResult
 from mms_amd.simulator.workload import (DEFAULT_WARMUP, PerModelStatsResult,
                                         StatsResult, Workload)
 from mms_amd.util import ServingCase, batchsize_config, eps, inf
+from mms_amd.simulator.event_sim import Client, Controller, GroupManager, simulate_one_case  # noqa: F401
 
 
 def install_remote_methods(obj):

@@ -3,9 +3,10 @@
 The placement evaluator registers models as ``partial(Executable, profile)``
 (reference base_policy.py:202-205) and the approximate simulator only reads
 the ``ProfilingResult`` back out of that partial (controller.py:290-296).  The
-reference's class additionally replays stage latencies on an event loop
-(simulator/executable.py:7-46); that behaviour belongs to the event-driven
-simulator and is not provided here.
+reference's class additionally replays stage latencies on its event loop
+(simulator/executable.py:31-46); here that replay is part of
+``mms_amd.simulator.event_sim.Client.submit_workload``, which needs the
+profile only.
 """
 from mms_amd.profiling import ProfilingResult
 
@@ -18,7 +19,3 @@ class Executable:
         if parallel_config is not None:
             self.stage_latency = profiling_result.para_dict[parallel_config].latency
 
-    async def handle_request(self, request):
-        raise NotImplementedError(
-            "mms_amd provides the approximate simulator only; the event-driven "
-            "simulator that would call this is outside its scope")

@@ -1,0 +1,116 @@
+"""The event-driven simulator (mms_amd/simulator/event_sim.py) against what the
+reference's own classes returned on the same seeded cases
+(tests/golden/make_event_sim_vectors.py -> event_sim_vectors.json): finish
+times bit for bit, good flags, per-group request counts and the statistics.
+Host code; no GPU involved.  Plus the TraceReplay -> Workload input format.
+"""
+import json
+import os
+from functools import partial
+
+import numpy as np
+import pytest
+
+from mms_amd.placement_policy import ClusterEnv, ModelData, ModelPlacement, PlacementEvaluator
+from mms_amd.placement_policy.base_policy import BasePlacementPolicy
+from mms_amd.profiling import ParallelConfig, load_test_prof_result
+from mms_amd.simulator.controller import Client, Controller, simulate_one_case
+from mms_amd.simulator.executable import Executable
+from mms_amd.simulator.workload import GammaProcess, Workload
+from mms_amd.util import GB, ServingCase
+
+with open(os.path.join(os.path.dirname(__file__), "golden", "event_sim_vectors.json")) as f:
+    CASES = json.load(f)["cases"]
+
+
+def _serving_case(c):
+    profile = load_test_prof_result(c["profile"])
+    model_datas = [ModelData(f"m{i}", slo, rate, cv, profile) for i, (rate, cv, slo) in enumerate(c["models"])]
+    placement = ModelPlacement([ParallelConfig(1, 1, p) for p, _ in c["groups"]], [list(ms) for _, ms in c["groups"]])
+    cluster_env = ClusterEnv(sum(p for p, _ in c["groups"]), 64 * GB)
+
+    def register_models(controller):
+        for md in model_datas:
+            controller.register_model.remote(md.name, partial(Executable, md.profiling_result))
+
+    def generate_workload(start=0):
+        ws = [GammaProcess(md.rate, md.cv).generate_workload(md.name, start, c["duration"], slo=md.slo,
+                                                              seed=c["seed"] * 100 + i)
+              for i, md in enumerate(model_datas)]
+        return Workload.merge(*ws)
+
+    def place_models(controller):
+        BasePlacementPolicy().place_models_impl(controller, cluster_env, model_datas, placement)
+
+    return ServingCase(register_models, generate_workload, place_models), model_datas, placement, cluster_env
+
+
+@pytest.mark.parametrize("c", CASES, ids=lambda c: c["name"])
+def test_per_request_outcomes_equal_the_reference(c):
+    case, _, _, _ = _serving_case(c)
+    register_models, generate_workload, place_models = case
+    np.random.seed(c["seed"])                      # the same order of draws as simulate_one_case
+    controller = Controller()
+    register_models(controller)
+    place_models(controller)
+    client = Client(controller)
+    workload = generate_workload()
+    assert [float(x).hex() for x in workload.arrivals] == c["arrivals_hex"]
+    client.submit_workload(workload)
+    start, finish, good = client.res_dict[workload]
+    assert np.array_equal(start, workload.arrivals)
+    assert [float(x).hex() for x in finish] == c["finish_hex"]
+    assert [int(x) for x in good] == c["good"]
+    assert [controller.num_total_requests[g] for g in controller.managers] == c["group_num_requests"]
+    assert 0 < sum(c["good"]) and (c["name"] == "light_two_stage" or sum(c["good"]) < len(c["good"]))
+
+
+@pytest.mark.parametrize("c", CASES, ids=lambda c: c["name"])
+def test_simulate_one_case_statistics_equal_the_reference(c):
+    case, _, _, _ = _serving_case(c)
+    np.random.seed(c["seed"])
+    stats, placement = simulate_one_case(case, warmup=c["warmup"])
+    assert placement is None                       # place_models applies the placement and returns nothing
+    assert stats.group_num_requests == tuple(c["group_num_requests"])
+    assert stats.goodput == c["goodput"]
+    assert abs(stats.latency_mean - c["latency_mean"]) <= 1e-15 * c["latency_mean"]
+    assert [[s.name, int(s.num_requests), float(s.goodput), float(s.latency_p99)] for s in stats.per_model_stats] == c["per_model"]
+
+
+def test_evaluator_with_the_event_driven_method_and_the_approximation_agree_roughly():
+    """PlacementEvaluator(method != "fast_simulator") goes through simulate_one_case (base_policy.py:172-224 of the
+    reference).  The two simulators model different overheads, so they only agree roughly -- which is the use of the
+    slow one: a fidelity check of the fast one."""
+    import oracle_backend
+    mp = pytest.MonkeyPatch()
+    try:
+        oracle_backend.install(mp)
+        model_datas = [ModelData(f"m{i}", 1.0, 4, 1, load_test_prof_result("test-2GB-100ms")) for i in range(3)]
+        cluster_env = ClusterEnv(4, 64 * GB)
+        sol = ModelPlacement([ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 2)], [[0, 1, 2], [0, 1, 2]])
+        ws = [GammaProcess(md.rate, md.cv).generate_workload(md.name, 0, 60, slo=md.slo, seed=i)
+              for i, md in enumerate(model_datas)]
+        wl = Workload.merge(*ws)
+        np.random.seed(3)
+        slow = PlacementEvaluator(model_datas, cluster_env, wl, "simulator", False)
+        fast = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+        g_slow, per_model, groups, stats = slow.get_stats([sol])[0]
+        g_fast = fast.get_stats([sol])[0][0]
+        assert sum(groups) == len(wl) and len(per_model) == 3
+        assert abs(g_slow - g_fast) < 0.05
+        assert abs(slow.get_scores([sol])[0] - fast.get_scores([sol])[0]) < 0.05
+    finally:
+        mp.undo()
+
+
+def test_trace_replay_to_workload():
+    from mms_amd.trace import TraceReplay
+    arrivals = np.array([0.5, 1.0, 1.25, 4.0])
+    tr = TraceReplay("m0", arrivals, "azure_v1", "0.0.0", "0.0.1", 60, "gamma")
+    wl = tr.to_workload(slo=0.7)
+    assert isinstance(wl, Workload) and len(wl) == 4
+    assert np.array_equal(wl.arrivals, arrivals)
+    assert [r.model_name for r in wl.requests] == ["m0"] * 4 and [r.idx for r in wl.requests] == [0, 1, 2, 3]
+    assert all(r.slo == 0.7 and r.data is None for r in wl.requests)
+    merged = Workload.merge(wl, TraceReplay("m1", np.array([0.75]), "azure_v1", "0.0.0", "0.0.1", 60, "gamma").to_workload(1.0))
+    assert [r.model_name for r in merged.requests] == ["m0", "m1", "m0", "m0", "m0"]

@@ -198,8 +198,6 @@ def test_evaluator_batch_equals_one_by_one(backend):
     s0 = PlacementEvaluator.get_goodput_simulation(sols[0], model_datas, cluster_env, wl, "fast_simulator")
     assert abs(s0 - scores[0]) <= 1e-12 * abs(s0)
     assert ev.get_scores([]) == [] and ev.get_stats([]) == []
-    with pytest.raises(NotImplementedError):
-        PlacementEvaluator(model_datas, cluster_env, wl, "simulator", False)
 
 
 def test_approximate_one_case_full_stats_and_unknown_model(backend):
