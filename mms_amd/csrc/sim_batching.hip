@@ -194,6 +194,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     o += (size_t)(Gmax + 1) * LS * 2;
     uint16_t *g2m_idx_lds = reinterpret_cast<uint16_t *>(mine + o) + sl;  // [members_max][64]
 
+    bool sizes_pow2 = true;  // wave-uniform: batch size q is 1 << q
+    for (int q = 0; q < NB; ++q) sizes_pow2 = sizes_pow2 && a.batch_sizes[q] == (1 << q);
+
     const bool live = tile < a.tiles;
     const bool sim = sl < LS;  // the other lanes of a narrow tile only help fetching requests
     if (live && sim) {
@@ -258,18 +261,35 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     auto select_model = [&](uint32_t g) -> int {
         const int lo = g2m_off_at(g), hi = g2m_off_at(g + 1u);
         if constexpr (OCT) {
-            // one model per lane; the key orders by rank of the head's arrival, then by place in the list
+            // The models of the group are dealt to the lanes of the octet (model x to lane x mod 8), two per lane
+            // and round so that their reads overlap; every lane keeps the smallest key of its own models and the
+            // octet takes one minimum at the end.  The key orders by rank of the head's arrival, then by place in
+            // the list.
+            constexpr int kPerLane = 2;
             uint64_t best = ~0ull;
-            for (int x0 = lo; x0 < hi; x0 += 8) {
-                const int x = x0 + oj;
-                const int mm = g2m_idx_at(x < hi ? x : hi - 1);
-                const uint32_t rk = (uint32_t)hrank[mm * LS];
-                const uint32_t hd = head[mm * LS], ar = arrived[mm];
-                const bool waiting = x < hi && (int)(ar - hd) > 0;
-                const uint64_t key = waiting ? ((uint64_t)rk << 32) | ((uint64_t)(uint32_t)(x - lo) << 16) | (uint32_t)mm : ~0ull;
-                const uint64_t k = oct_min(key);
-                best = k < best ? k : best;
+            for (int xb = lo; xb < hi; xb += 8 * kPerLane) {
+                int mm[kPerLane];
+                uint32_t rk[kPerLane], hd[kPerLane], ar[kPerLane];
+#pragma unroll
+                for (int u = 0; u < kPerLane; ++u) {
+                    const int x = xb + 8 * u + oj;
+                    mm[u] = g2m_idx_at(x < hi ? x : hi - 1);
+                }
+#pragma unroll
+                for (int u = 0; u < kPerLane; ++u) {
+                    rk[u] = (uint32_t)hrank[mm[u] * LS];
+                    hd[u] = head[mm[u] * LS];
+                    ar[u] = arrived[mm[u]];
+                }
+#pragma unroll
+                for (int u = 0; u < kPerLane; ++u) {
+                    const int x = xb + 8 * u + oj;
+                    const bool waiting = x < hi && (int)(ar[u] - hd[u]) > 0;
+                    const uint64_t key = waiting ? ((uint64_t)rk[u] << 32) | ((uint64_t)(uint32_t)(x - lo) << 16) | (uint32_t)mm[u] : ~0ull;
+                    best = key < best ? key : best;
+                }
             }
+            best = oct_min(best);
             return best == ~0ull ? -1 : (int)(best & 0xFFFFu);
         }
         int min_rank = 0x7FFFFFFF;
@@ -362,8 +382,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     constexpr bool COOP = OCT && NBT <= 8;  // batch attempts split over the octet (one latency column per lane)
 
     // :706-732 with :674-704 inlined; the reference's recursion on "nothing servable" is the outer loop
-    auto handle = [&](double t0, int m, uint32_t g) {
-        const uint32_t d = ginfo[g * LS];
+    // d: the group's descriptor (its index is desc_group(d))
+    auto handle = [&](double t0, int m, uint32_t d) {
+        const uint32_t g = desc_group(d);
         const int stages = (int)desc_stages_m1(d) + 1;
         double *gclk = clk + (desc_last_slot(d) - desc_stages_m1(d)) * LS;
         for (;;) {
@@ -427,13 +448,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 }
                 if (found) {
                     // grow the batch while the first request still meets its deadline (:693-702): lane b tests
-                    // batch size b, the batch is the last size before the first one that fails
-                    const int cand = bsz[oj < NB ? oj : NB - 1];
-                    const double tc = oct_get(tcol, ilog2i(cand));
+                    // batch size b, the batch is the last size before the first one that fails.  When the sizes are
+                    // 1, 2, 4, ... (size b is 1 << b and has latency column b) nothing needs to be looked up.
+                    const int cand = sizes_pow2 ? 1 << (oj < NB ? oj : NB - 1) : bsz[oj < NB ? oj : NB - 1];
+                    const double tc = sizes_pow2 ? tcol : oct_get(tcol, ilog2i(cand));
                     const bool ok = oj == 0 || (oj < NB && cand - 1 <= (int)(arr - h) && (tc + overhead) <= deadline);
                     const uint32_t fail = ~oct_ballot(ok) & 0xFFu;
                     const int nb_ok = fail ? __ffs((int)fail) - 1 : 8;
-                    bs = bsz[nb_ok - 1];
+                    bs = sizes_pow2 ? 1 << (nb_ok - 1) : bsz[nb_ok - 1];
                 }
             } else {
             double dl[8], tq[8];  // deadlines and arrival times (one 16-byte load per head)
@@ -592,7 +614,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             nfree -= 1;
             const int slot = fstack[nfree * LS];
             ev_t[slot * LS] = idle_at;
-            ev_g[slot * LS] = g;
+            ev_g[slot * LS] = d;  // the descriptor, not the index: it orders like the index and saves the look-up when the event is due
             double *cm = cm_t + (slot >> 3) * LS;
             *cm = fmin(*cm, idle_at);
             next_due = fmin(next_due, idle_at);
@@ -638,7 +660,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         }
     };
     // removes the lexicographically smallest (time, group) event, whose time T and chunk cj chunk_scan
-    // found (others as returned by it); returns its group and sets next_due to the earliest time left
+    // found (others as returned by it); returns its word (the group's descriptor, which orders like the group's
+    // index) and sets next_due to the earliest time left
     auto take_event = [&](double T, int cj, double others) -> uint32_t {
         uint32_t bg = 0xFFFFFFFFu;
         int be = cj << 3;
@@ -731,10 +754,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                     next_due = ti;
                     break;
                 }
-                const uint32_t g = take_event(ti, cj, others);  // sets next_due; handle() lowers it when it adds an earlier event
-                const int m2 = select_model(g);
+                const uint32_t d = take_event(ti, cj, others);  // sets next_due; handle() lowers it when it adds an earlier event
+                const int m2 = select_model(desc_group(d));
                 if (m2 < 0) break;  // the popped event is dropped, later due events stay (:742-743)
-                handle(ti, m2, g);
+                handle(ti, m2, d);
                 if (dead || !(next_due <= tstamp)) break;
             }
         }
@@ -802,11 +825,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 good_out[(size_t)i * kWave] = 0;
             }
         } else if (gsel == none) {
-            dead = MMSIM_E_UNSUPPORTED;  // every replica's clock is infinite; the reference indexes out of range here
+            // every replica's clock is infinite (only after a batch with infinite latency was accepted under an
+            // infinite SLO): the reference's g_id stays -1 here, which its arrays take as "the last group"
+            // (controller.py:760-778); that accident is not reproduced
+            dead = MMSIM_E_UNSUPPORTED;
         } else {
             const uint32_t d = ginfo[gsel * LS];
             const double idle_since = clk[(desc_last_slot(d) - desc_stages_m1(d)) * LS];
-            if (tstamp >= idle_since) handle(tstamp, m, gsel);  // :776-778
+            if (tstamp >= idle_since) handle(tstamp, m, d);  // :776-778
         }
     }
     // ---- drain (:781-787)
@@ -814,10 +840,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         double ti, others;
         int cj;
         chunk_scan(ti, cj, others);
-        const uint32_t g = take_event(ti, cj, others);
-        const int m2 = select_model(g);
+        const uint32_t d = take_event(ti, cj, others);
+        const int m2 = select_model(desc_group(d));
         if (m2 < 0) continue;
-        handle(ti, m2, g);
+        handle(ti, m2, d);
     }
 
     if constexpr (COOP) lat_sum = oct_sum(lat_sum);  // each lane summed the batch members it had fetched
