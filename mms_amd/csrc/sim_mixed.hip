@@ -451,7 +451,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 constexpr int j = decltype(J)::value;
                 k[j].d = pick_desc<j>(da, db);
                 k[j].c = lds_f64(rep_addr(k[j].d) + rel_base);
-                k[j].l = lrow_m[rep_lat_last(k[j].d)];
+                // (loop over runs: the winner's latency is read after the tournament instead, one read for eight)
+                k[j].l = RUNS ? 0.0f : lrow_m[rep_lat_last(k[j].d)];
                 return true;
             });
             const Cand a01 = first_min(k[0], k[1]), a23 = first_min(k[2], k[3]);
@@ -478,6 +479,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     win = first_min(win, Cand{lds_f64(rep_addr(d) + rel_base), d, lrow_m[rep_lat_last(d)]});
                 }
             }
+            if constexpr (RUNS) win.l = lrow_m[rep_lat_last(win.d)];
             // a clock that is infinite (a group that served a request with infinite latency) is never
             // chosen (:590-598: "tmp < min_device_clock" with min_device_clock starting at inf)
             ch_model = m;
