@@ -48,6 +48,11 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.Placements) == 40
     assert ctypes.sizeof(_lib.Result) == 10 * 8
     assert ctypes.sizeof(_lib.BatchInfo) == 8 * 4 + 3 * 8 + 4 * 4
+    assert ctypes.sizeof(_lib.ModelStats) == 9 * 8
+    # field order of mmsim_model_stats as the header declares it
+    header = open(os.path.join(ROOT, "include", "mmsim.h")).read()
+    body = re.search(r"typedef struct \{([^}]*)\} mmsim_model_stats;", header).group(1)
+    assert re.findall(r"\*(\w+);", body) == [f[0] for f in _lib.ModelStats._fields_]
 
 
 # ---- table build (controller.py:412-476) --------------------------------------------------
