@@ -10,12 +10,15 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <chrono>
 #include <cstring>
 #include <functional>
 #include <limits>
 #include <memory>
 #include <mutex>
+#include <atomic>
 #include <new>
+#include <thread>
 
 #include "mmsim_internal.h"
 
@@ -211,6 +214,23 @@ int check_tables(const mmsim_tables *t) {
 }
 
 // group -> models CSR of the C ABI into ordered per-(placement, model) replica lists
+// Runs fn(lo, hi) on slices of [0, n) on up to 16 host threads (one slice per thread; the caller's
+// slices write disjoint memory).  Small ranges run on the calling thread.
+template <class F>
+void parallel_slices(int64_t n, int64_t min_per_thread, F &&fn) {
+    int64_t threads = std::min<int64_t>(16, std::max(1u, std::thread::hardware_concurrency()));
+    threads = std::min<int64_t>(threads, n / std::max<int64_t>(1, min_per_thread));
+    if (threads <= 1) {
+        fn((int64_t)0, n);
+        return;
+    }
+    const int64_t per = (n + threads - 1) / threads;
+    std::vector<std::thread> pool;
+    for (int64_t lo = per; lo < n; lo += per) pool.emplace_back([&fn, lo, per, n] { fn(lo, std::min(n, lo + per)); });
+    fn((int64_t)0, std::min(n, per));
+    for (std::thread &th : pool) th.join();
+}
+
 int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLists *out) {
     if (!p || !p->num_groups || !p->group_cfg || !p->gm_off) return fail(MMSIM_E_INVALID, "placements: null pointer");
     if (p->B < 1 || p->Gmax < 1) return fail(MMSIM_E_INVALID, "placements: B and Gmax must be >= 1");
@@ -251,6 +271,16 @@ int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLi
 // Builds every device table of a batch from replica lists and launches nothing.
 int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seeds, const mmsim_tables *t,
                 const RepLists &rl, uint32_t flags, mmsim_batch **out, const int32_t *stream_of = nullptr) {
+    // MMSIM_TIMING=1 prints the host time of each phase of the packing (diagnostics)
+    const bool timing = std::getenv("MMSIM_TIMING") != nullptr;
+    auto t_last = std::chrono::steady_clock::now();
+    auto phase = [&](const char *name) {
+        if (!timing) return;
+        const auto now = std::chrono::steady_clock::now();
+        std::fprintf(stderr, "[mmsim] build_batch %-28s %8.3f ms\n", name, std::chrono::duration<double, std::milli>(now - t_last).count());
+        t_last = now;
+    };
+
     const bool batching = (flags & MMSIM_BATCHING) != 0;
     if (batching && (flags & MMSIM_WANT_OP_COUNT)) return fail(MMSIM_E_UNSUPPORTED, "operation counts are only available for the plain simulator");
     if (batching) {
@@ -318,6 +348,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     if (b->smax_bucket < 0) return fail(MMSIM_E_UNSUPPORTED, "no kernel bucket for this many pipeline stages");
     b->nslots = nslots;
 
+    phase("slots and replica counts");
     // ---- compact batch-size-1 latency table.  General form: row of model m = its stage
     //      latencies for configuration 0, then configuration 1, ... (the cfg_pp[c] real
     //      stages only).  When every (model, config) has one latency for all its stages the
@@ -355,6 +386,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (const char *env = std::getenv("MMSIM_RUNS")) runs = std::atoi(env) != 0;  // tuning knob
     }
 
+    phase("latency table, loop choice");
     // ---- LDS budget
     const int32_t rmax_lds_bytes = (M + 15) & ~15;
     size_t wave_bytes = 0, lat_bytes = 0, lds_tail = 0, sched_bytes = 0;
@@ -477,6 +509,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
 
     std::vector<int32_t> tile_nslots;  // most clock slots of a placement of each tile
     std::vector<int32_t> tile_stream;  // paired batches: the stream of each tile
+    phase("LDS budget");
     // ---- lane assignment.  A wavefront walks as many pipeline stages as its deepest
     //      lane needs, so placements are ordered by depth before they are cut into
     //      tiles of 64: first by their deepest group, then by the expected depth of a
@@ -487,20 +520,27 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             for (int32_t m = 0; m < M; ++m) weight[m] += (double)wls[s]->model_num_requests[m];
         std::vector<int32_t> deepest(B, 0);
         std::vector<double> expected(B, 0.0);
-        std::vector<int32_t> depth_of(M);
-        for (int32_t p = 0; p < B; ++p) {
-            std::fill(depth_of.begin(), depth_of.end(), 0);
-            for (int32_t m = 0; m < M; ++m)
-                for (int64_t x = rl.off[(size_t)p * M + m]; x < rl.off[(size_t)p * M + m + 1]; ++x) {
-                    const int32_t g = rl.grp[(size_t)x];
-                    if (g < 0 || g >= rl.num_groups[p]) return fail(MMSIM_E_INVALID, "replica list names a group that does not exist");
-                    depth_of[m] = std::max(depth_of[m], t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]]);
+        std::atomic<bool> bad_group{false};
+        parallel_slices(B, 512, [&](int64_t p0, int64_t p1) {
+            std::vector<int32_t> depth_of(M);
+            for (int64_t p = p0; p < p1; ++p) {
+                std::fill(depth_of.begin(), depth_of.end(), 0);
+                for (int32_t m = 0; m < M; ++m)
+                    for (int64_t x = rl.off[(size_t)p * M + m]; x < rl.off[(size_t)p * M + m + 1]; ++x) {
+                        const int32_t g = rl.grp[(size_t)x];
+                        if (g < 0 || g >= rl.num_groups[p]) {
+                            bad_group = true;
+                            return;
+                        }
+                        depth_of[m] = std::max(depth_of[m], t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]]);
+                    }
+                for (int32_t m = 0; m < M; ++m) {
+                    deepest[p] = std::max(deepest[p], depth_of[m]);
+                    expected[p] += weight[m] * depth_of[m];
                 }
-            for (int32_t m = 0; m < M; ++m) {
-                deepest[p] = std::max(deepest[p], depth_of[m]);
-                expected[p] += weight[m] * depth_of[m];
             }
-        }
+        });
+        if (bad_group) return fail(MMSIM_E_INVALID, "replica list names a group that does not exist");
         // Deepest first: their wavefronts take longest.  The loop over runs sizes a wavefront's LDS region by the
         // clock slots of its own tile, so there placements with similar slot counts share a tile
         // (MMSIM_TILE_ORDER=0: by expected depth only, tuning knob).
@@ -545,6 +585,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
     }
 
+    phase("lane assignment");
     // ---- loop over runs: the schedule.  An item is one (tile, stream) pair; it needs an LDS region as large as its
     //      tile's clock slots ask for.  Items are dealt to at most one workgroup per CU, tiles staying on one XCD (a
     //      workgroup goes to XCD blockIdx % 8; the tile's descriptor rows then live in one L2), largest first in
@@ -645,6 +686,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         b->lds_bytes = lat_bytes + sched_bytes + lds_used + lds_tail;
     }
 
+    phase("schedule");
     // ---- per lane group descriptors [tiles][Gmax+1][64]; row Gmax stays empty
     std::vector<uint32_t> ginfo((size_t)b->tiles * (Gmax + 1) * kWave, kEmpty);
     for (int32_t p = 0; p < B; ++p) {
@@ -683,14 +725,16 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     };
     if (!batching) {  // missing replicas: the +inf clock and the +inf latency, flagged empty
         const uint32_t inf_lat = (uint32_t)lat_off[C] << 18;
-        for (int32_t tile = 0; tile < b->tiles; ++tile) {
-            uint32_t lane_word[kWave];
-            for (int lane = 0; lane < kWave; ++lane) lane_word[lane] = kEmpty | clock_addr(tile * kWave + lane, -1) | inf_lat;
-            uint32_t *dst = rep32.data() + (size_t)tile * M * 2 * kWave * 4;
-            for (size_t i = 0; i < (size_t)M * 2 * kWave * 4; ++i) dst[i] = lane_word[(i / 4) % kWave];
-            uint32_t *dx = repx32.data() + (size_t)tile * M * RX * kWave;
-            for (size_t i = 0; i < (size_t)M * RX * kWave; ++i) dx[i] = lane_word[i % kWave];
-        }
+        parallel_slices(b->tiles, 8, [&](int64_t t0, int64_t t1) {
+            for (int64_t tile = t0; tile < t1; ++tile) {
+                uint32_t lane_word[kWave];
+                for (int lane = 0; lane < kWave; ++lane) lane_word[lane] = kEmpty | clock_addr((int)tile * kWave + lane, -1) | inf_lat;
+                uint32_t *dst = rep32.data() + (size_t)tile * M * 2 * kWave * 4;
+                for (size_t i = 0; i < (size_t)M * 2 * kWave * 4; ++i) dst[i] = lane_word[(i / 4) % kWave];
+                uint32_t *dx = repx32.data() + (size_t)tile * M * RX * kWave;
+                for (size_t i = 0; i < (size_t)M * RX * kWave; ++i) dx[i] = lane_word[i % kWave];
+            }
+        });
     }
     std::vector<uint8_t> slot_group;
     if (!batching && (flags & MMSIM_WANT_GROUP_COUNTS)) {
@@ -704,8 +748,21 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             }
         }
     }
+    std::vector<int32_t> tile_begin;
     std::vector<uint8_t> rmax((size_t)b->tiles * M, 0);
-    for (int32_t p = 0; p < B; ++p) {
+    // (by tile: the placements of a tile write that tile's rows only)
+    std::vector<int32_t> by_tile(B);
+    {
+        std::vector<int32_t> at((size_t)b->tiles + 1, 0);
+        for (int32_t p = 0; p < B; ++p) at[(size_t)(b->pos[p] / kWave) + 1] += 1;
+        for (int32_t k = 0; k < b->tiles; ++k) at[(size_t)k + 1] += at[(size_t)k];
+        std::vector<int32_t> fill(at.begin(), at.end() - 1);
+        for (int32_t p = 0; p < B; ++p) by_tile[(size_t)fill[(size_t)(b->pos[p] / kWave)]++] = p;
+        tile_begin = std::move(at);
+    }
+    parallel_slices(b->tiles, 8, [&](int64_t t0, int64_t t1) {
+    for (int64_t k = tile_begin[(size_t)t0]; k < tile_begin[(size_t)t1]; ++k) {
+        const int32_t p = by_tile[(size_t)k];
         const int tile = b->pos[p] / kWave, lane = b->pos[p] % kWave;
         for (int32_t m = 0; m < M; ++m) {
             const int64_t lo = rl.off[(size_t)p * M + m], hi = rl.off[(size_t)p * M + m + 1];
@@ -734,7 +791,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             if (batching) rep8[((size_t)tile * M + m) * kWave + lane] = word;
         }
     }
+    });
 
+    phase("descriptors");
     // ---- batching simulator: models of each group, full latency table, which models a lane hosts
     std::vector<uint16_t> g2m_off, g2m_idx;
     std::vector<float> lat_nb;
@@ -834,6 +893,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         b->lds_bytes = batching_lat_lds + (size_t)b->waves_per_block * wave_bytes;
     }
 
+    phase("batching tables");
     // ---- request streams back to back
     std::vector<int64_t> soff(n_seeds + 1, 0);
     for (int s = 0; s < n_seeds; ++s) {
@@ -944,6 +1004,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
     HIP_TRY(hipStreamSynchronize(st));  // host staging vectors go out of scope below
 
+    phase("streams + uploads");
     // ---- loop over runs: the schedule's tables, and room to park clocks between segments
     if (!plan.empty()) {
         HIP_TRY(b->plan.alloc(plan.size()));
@@ -1056,6 +1117,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         q.finish = b->finish.p;
         q.good = b->good.p;
     }
+    phase("schedule tables, kernel args");
     *out = b.release();
     return MMSIM_OK;
 }
