@@ -70,6 +70,60 @@ def cpu_baseline(cfg, table, stream, sols, n_threads):
     return ref, packed, evals / t1, evals / tm, t1
 
 
+def model_stats_bench(args, cfg, streams):
+    """One step = one mmsim_batch_model_stats call on the per-request outputs of B placements x the given
+    streams (uploads of the window, kernel, copy of the [L][M] results).  Prints one JSON line."""
+    from mms_amd import _lib, engine as E
+    eng = E.Engine.default()
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    dws = [E.DeviceWorkload(eng, s.tstamps, s.model_ids, s.slos, cfg.num_models) for s in streams]
+    flags = _lib.WANT_PER_REQUEST | (_lib.BATCHING if cfg.batching else 0)
+    batch = E.Batch(eng, dws, table, E.pack_placements(cfg.placements, table), flags)
+    batch.run()
+    batch.sync()
+    skip = [len(s.tstamps) // 50 for s in streams]
+    for _ in range(args.warmup):
+        batch.model_stats(skip)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        got = batch.model_stats(skip)
+    sec = (time.perf_counter() - t0) / args.steps
+    B, L = len(cfg.placements), len(cfg.placements) * len(streams)
+    pairs = B * sum(len(s.tstamps) for s in streams)
+    result = {
+        "metric": "per-request outputs reduced to serving statistics, (simulation x request) pairs/sec",
+        "value": pairs / sec, "unit": "pairs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
+        "data": "synthetic",
+        "config": {"workload": f"config {cfg.index} ({cfg.name}): statistics of {B} placements x {len(streams)} seeds, "
+                               f"{len(streams[0].tstamps)} requests/seed, {cfg.num_models} models",
+                   "kernel": "model_stats_kernel", "lanes": L},
+        # finish (8 B) and good (1 B) of every (simulation, request) once: what one pass over the outputs reads;
+        # the radix selection reads them eight times
+        "roofline": {"bound": "hbm", "achieved": 9.0 * pairs / sec / 1e9, "peak": 8000.0, "unit": "GB/s",
+                     "frac": 9.0 * pairs / sec / 8e12, "traffic": None,
+                     "note": "achieved = 9 algorithmic bytes per (simulation, request) over the whole call"},
+    }
+    if not args.no_cpu:     # the same statistics with numpy on the fetched outputs, first placement of the first stream
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        from oracle_backend import model_stats_numpy
+        out = batch.fetch()
+        st = streams[0]
+        R = len(st.tstamps)
+        t0 = time.perf_counter()
+        want = model_stats_numpy(st.tstamps, st.model_ids, out["finish"][0, 0, :R], out["good"][0, 0, :R], skip[0],
+                                 cfg.num_models)
+        t1 = time.perf_counter() - t0
+        same = all(np.array_equal(got[k][0, 0], want[k]) for k in
+                   ("model_num_requests", "model_num_good", "first_start", "last_start", "latency_p90", "latency_p99"))
+        close = all(np.allclose(got[k][0, 0], want[k], rtol=1e-12, atol=0) for k in ("latency_sum", "latency_mean", "latency_std"))
+        result["cpu_baseline"] = {"value": R / t1, "unit": "pairs/s", "cores": 1, "kind": "port",
+                                  "sample": f"placement 0 x seed 0 ({R} requests, {t1:.2f}s), numpy sort per model on the copied outputs",
+                                  "gpu_equals_cpu_on_sample": bool(same and close)}
+    batch.close()
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -86,6 +140,9 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters of a profiled run can be scaled")
     ap.add_argument("--flags", type=str, default="scores", choices=["scores", "model", "stats"],
                     help="scores: goodput+latency only; model: + per-model counts; stats: + per-group counts")
+    ap.add_argument("--model-stats", action="store_true",
+                    help="time mmsim_batch_model_stats (serving statistics of the per-request outputs, on the device) "
+                         "instead of the simulation: use with --placements 64 --seeds 1")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -114,6 +171,9 @@ def main():
         torch.cuda.synchronize()
         log(f"[bench] copy calibration: one device copy of {args.copy_calibration} bytes")
         del src, dst
+
+    if args.model_stats:
+        return model_stats_bench(args, cfg, streams)
 
     eng = E.Engine.default()
     dev = eng.device_info()

@@ -1460,61 +1460,71 @@ int mmsim_batch_model_stats(mmsim_batch *b, const mmsim_workload *const *workloa
     }
     HIP_TRY(hipSetDevice(b->ctx->device));
     hipStream_t st = b->ctx->stream;
-    const size_t cells = (size_t)b->waves * (size_t)M * kWave;
-    DevBuf<const MqEntry *> d_mq;
-    DevBuf<int64_t> d_i64;   // mq_off | lo | hi
-    DevBuf<int32_t> d_i32;   // model_req | model_good
-    DevBuf<double> d_f64;    // the seven double results
-    HIP_TRY(d_mq.alloc(mq.size()));
-    HIP_TRY(d_i64.alloc(mqo.size() + 2 * (size_t)n_streams));
-    HIP_TRY(d_i32.alloc(2 * cells));
-    HIP_TRY(d_f64.alloc(7 * cells));
-    HIP_TRY(hipMemcpyAsync(d_mq.p, mq.data(), sizeof(mq[0]) * mq.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(hipMemcpyAsync(d_i64.p, mqo.data(), sizeof(int64_t) * mqo.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(hipMemcpyAsync(d_i64.p + mqo.size(), lo.data(), sizeof(int64_t) * lo.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(hipMemcpyAsync(d_i64.p + mqo.size() + lo.size(), hi.data(), sizeof(int64_t) * hi.size(), hipMemcpyHostToDevice, st));
-    StatsArgs a{};
-    a.finish = b->finish.p;
-    a.good = b->good.p;
-    a.mq = d_mq.p;
-    a.mq_off = d_i64.p;
-    a.lo = d_i64.p + mqo.size();
-    a.hi = a.lo + n_streams;
-    a.tile_seed = b->tile_seed.p;
-    a.paired = b->paired ? 1 : 0;
-    a.tiles = tiles;
-    a.M = M;
-    a.Rmax = b->Rmax;
-    a.model_req = d_i32.p;
-    a.model_good = d_i32.p + cells;
-    double *f = d_f64.p;
-    a.first_start = f;
-    a.last_start = f + cells;
-    a.latency_sum = f + 2 * cells;
-    a.latency_mean = f + 3 * cells;
-    a.latency_std = f + 4 * cells;
-    a.latency_p90 = f + 5 * cells;
-    a.latency_p99 = f + 6 * cells;
-    std::string err;
-    hipError_t e = launch_model_stats(a, b->waves, st, &err);
-    if (e != hipSuccess) return fail(MMSIM_E_HIP, err.empty() ? std::string("model_stats launch: ") + hipGetErrorString(e) : err);
-    std::vector<int32_t> h32(2 * cells);
-    std::vector<double> h64(7 * cells);
-    HIP_TRY(hipMemcpyAsync(h32.data(), d_i32.p, sizeof(int32_t) * h32.size(), hipMemcpyDeviceToHost, st));
-    HIP_TRY(hipMemcpyAsync(h64.data(), d_f64.p, sizeof(double) * h64.size(), hipMemcpyDeviceToHost, st));
-    HIP_TRY(hipStreamSynchronize(st));
-    int32_t *const o32[2] = {out->model_num_requests, out->model_num_good};
-    double *const o64[7] = {out->first_start, out->last_start, out->latency_sum, out->latency_mean,
-                            out->latency_std, out->latency_p90, out->latency_p99};
+    // one workgroup per (simulation, model), results already in the caller's layout; a launch needs a scratch row
+    // of 8 bytes per request for each of its simulations, so many simulations take several launches
+    const int64_t n_sims = (int64_t)b->out_seeds * B;
+    int64_t pitch = 1;
+    for (int s = 0; s < n_streams; ++s) pitch = std::max<int64_t>(pitch, workloads[s]->mq_off[(size_t)M]);
+    int64_t scratch_bytes = kStatsScratchBytes;
+    if (const char *env = std::getenv("MMSIM_STATS_SCRATCH_BYTES")) scratch_bytes = std::max<int64_t>(0, std::atoll(env));  // tuning knob
+    const int64_t rows = std::max<int64_t>(1, std::min<int64_t>(n_sims, scratch_bytes / (pitch * (int64_t)sizeof(uint64_t))));
+    std::vector<int32_t> sim_stream((size_t)n_sims);
+    std::vector<int64_t> sim_base((size_t)n_sims);
     for (int s = 0; s < b->out_seeds; ++s)
         for (int32_t p = 0; p < B; ++p) {
-            const size_t wave = (size_t)s * tiles + b->pos[p] / kWave, lane = (size_t)(b->pos[p] % kWave);
-            for (int32_t m = 0; m < M; ++m) {
-                const size_t src = (wave * M + m) * kWave + lane, dst = ((size_t)s * B + p) * M + m;
-                for (int k = 0; k < 2; ++k) o32[k][dst] = h32[(size_t)k * cells + src];
-                for (int k = 0; k < 7; ++k) o64[k][dst] = h64[(size_t)k * cells + src];
-            }
+            const size_t sim = (size_t)s * B + p;
+            const int64_t wave = (int64_t)s * tiles + b->pos[p] / kWave;
+            sim_stream[sim] = b->paired ? b->stream_of[p] : s;
+            sim_base[sim] = wave * b->Rmax * kWave + b->pos[p] % kWave;
         }
+    const size_t cells = (size_t)n_sims * (size_t)M;
+    DevBuf<const MqEntry *> d_mq;
+    DevBuf<int64_t> d_i64;   // mq_off | lo | hi | sim_base
+    DevBuf<int32_t> d_i32;   // sim_stream | model_req | model_good
+    DevBuf<double> d_f64;    // the seven double results
+    DevBuf<uint64_t> d_scratch;
+    HIP_TRY(d_mq.alloc(mq.size()));
+    HIP_TRY(d_i64.alloc(mqo.size() + 2 * (size_t)n_streams + (size_t)n_sims));
+    HIP_TRY(d_i32.alloc((size_t)n_sims + 2 * cells));
+    HIP_TRY(d_f64.alloc(7 * cells));
+    HIP_TRY(d_scratch.alloc((size_t)rows * (size_t)pitch));
+    HIP_TRY(hipMemcpyAsync(d_mq.p, mq.data(), sizeof(mq[0]) * mq.size(), hipMemcpyHostToDevice, st));
+    int64_t *i64 = d_i64.p;
+    HIP_TRY(hipMemcpyAsync(i64, mqo.data(), sizeof(int64_t) * mqo.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(i64 + mqo.size(), lo.data(), sizeof(int64_t) * lo.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(i64 + mqo.size() + lo.size(), hi.data(), sizeof(int64_t) * hi.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(i64 + mqo.size() + 2 * lo.size(), sim_base.data(), sizeof(int64_t) * sim_base.size(), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipMemcpyAsync(d_i32.p, sim_stream.data(), sizeof(int32_t) * sim_stream.size(), hipMemcpyHostToDevice, st));
+    StatsArgs f{};
+    f.finish = b->finish.p;
+    f.good = b->good.p;
+    f.mq = d_mq.p;
+    f.mq_off = i64;
+    f.lo = i64 + mqo.size();
+    f.hi = f.lo + n_streams;
+    f.sim_base = f.hi + n_streams;
+    f.sim_stream = d_i32.p;
+    f.scratch = d_scratch.p;
+    f.scratch_pitch = pitch;
+    f.M = M;
+    f.model_req = d_i32.p + n_sims;
+    f.model_good = f.model_req + cells;
+    double *d = d_f64.p;
+    double **slots[7] = {&f.first_start, &f.last_start, &f.latency_sum, &f.latency_mean, &f.latency_std, &f.latency_p90, &f.latency_p99};
+    for (int k = 0; k < 7; ++k) *slots[k] = d + (size_t)k * cells;
+    for (int64_t sim0 = 0; sim0 < n_sims; sim0 += rows) {  // launches on one stream: the scratch rows are reused in order
+        f.sim0 = (int32_t)sim0;
+        std::string err;
+        hipError_t e = launch_model_stats(f, (int)std::min<int64_t>(rows, n_sims - sim0), st, &err);
+        if (e != hipSuccess) return fail(MMSIM_E_HIP, err.empty() ? std::string("model_stats launch: ") + hipGetErrorString(e) : err);
+    }
+    HIP_TRY(hipMemcpyAsync(out->model_num_requests, f.model_req, sizeof(int32_t) * cells, hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipMemcpyAsync(out->model_num_good, f.model_good, sizeof(int32_t) * cells, hipMemcpyDeviceToHost, st));
+    double *const o64[7] = {out->first_start, out->last_start, out->latency_sum, out->latency_mean,
+                            out->latency_std, out->latency_p90, out->latency_p99};
+    for (int k = 0; k < 7; ++k)
+        HIP_TRY(hipMemcpyAsync(o64[k], d + (size_t)k * cells, sizeof(double) * cells, hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
     return MMSIM_OK;
 }
 

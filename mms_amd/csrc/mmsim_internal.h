@@ -214,21 +214,25 @@ struct ScalarArgs {
     int32_t *group_req, *group_good;  // [G], zeroed by the caller
 };
 // Arguments of the statistics kernel: the per-request outputs of a batch and, per stream, its arrivals
-// regrouped by model and the window of request indices that the warm-up trimming leaves.
+// regrouped by model and the window of request indices that the warm-up trimming leaves.  One launch
+// handles the simulations sim0 .. sim0 + n - 1, one scratch row each.
 struct StatsArgs {
     const double *finish;           // [waves][Rmax][64]
     const uint8_t *good;            // [waves][Rmax][64]
     const MqEntry *const *mq;       // [n_streams] model-ordered arrivals of each stream
     const int64_t *mq_off;          // [n_streams][M+1]
     const int64_t *lo, *hi;         // [n_streams] window [lo, hi) of request indices
-    const int32_t *tile_seed;       // as in MixedArgs
-    int32_t paired, tiles, M;
-    int64_t Rmax;
-    // outputs, [waves][M][64]
+    const int32_t *sim_stream;      // [n_sims] stream of each simulation
+    const int64_t *sim_base;        // [n_sims] wave * Rmax * 64 + lane: where its column of finish / good starts
+    uint64_t *scratch;              // [rows][scratch_pitch] latencies of a stream's requests in model order (all ones: not accepted)
+    int64_t scratch_pitch;
+    int32_t M, sim0;
+    // outputs, [n_sims][M]
     int32_t *model_req, *model_good;
     double *first_start, *last_start, *latency_sum, *latency_mean, *latency_std, *latency_p90, *latency_p99;
 };
-hipError_t launch_model_stats(const StatsArgs &args, int waves, hipStream_t stream, std::string *err);
+hipError_t launch_model_stats(const StatsArgs &args, int n, hipStream_t stream, std::string *err);
+constexpr int64_t kStatsScratchBytes = (int64_t)1 << 30;  // scratch rows of one launch (more simulations take several launches)
 
 hipError_t launch_sim_scalar(const ScalarArgs &args, hipStream_t stream, std::string *err);
 

@@ -3,27 +3,26 @@
 // requests inside the window that the warm-up trimming leaves, the arrival times of the first and
 // the last of them, and the mean, standard deviation, 90th and 99th percentile of their latencies.
 //
-// One workgroup per (wavefront of simulations, model): lane = simulation, as in the simulators, so
-// finish[wave][request][64] is read a coalesced row at a time.  The requests of a model are the same
-// for every lane (the per-model lists of the stream), only `good` differs.  The workgroup's eight
-// wavefronts take contiguous slices of the model's requests and count into the same histograms.
+// One workgroup of 1024 threads per (simulation, model); its threads share the model's requests, which
+// the per-model lists of the stream name (index and arrival time).  The first pass gathers the model's
+// latencies out of the simulation's column of finish[wave][request][64] / good (one 8-byte element per
+// 512-byte row: read once; simulations of one wavefront run side by side, so the rows are shared in L2)
+// into a contiguous scratch row, all ones for requests that were not accepted, and counts, sums and bins
+// the top byte on the way; every thread later reads back only what it wrote itself.
 //
 // Percentiles are order statistics: sorted[int(q * n)] (workload.py:344-346), found exactly with a
 // radix selection on the bit pattern of the latency (positive doubles order as their bits do): eight
-// passes of eight bits, most significant first, each lane counting into its own 256 bins in LDS the
-// elements that match the digits it has fixed so far.  Both percentiles are selected in the same
-// passes (two histograms).  The first pass also counts and sums (n decides the two ranks), the
-// second one sums the squared deviations.  Sums are compensated (Neumaier), so mean and deviation
-// are within a few ulp of the exact value, as numpy's pairwise sums are; they are not bit-equal to
-// numpy's.
+// passes of eight bits, most significant first, counting into 256 bins in LDS the elements that match
+// the digits fixed so far; both percentiles in the same passes (two histograms).  The first pass also
+// counts and sums (n decides the two ranks), the second one sums the squared deviations.  Sums are
+// compensated (Neumaier) per thread and added up in a fixed order, so mean and deviation are within a
+// few ulp of the exact value, as numpy's pairwise sums are; they are not bit-equal to numpy's.
 #include "mmsim_internal.h"
 
 namespace mmsim {
 namespace {
 
 constexpr int kBins = 256;
-constexpr int kUnroll = 8;
-constexpr int kStatsWaves = 8;  // wavefronts of a workgroup; they share one pair of histograms
 
 struct Accum {
     double sum = 0.0, comp = 0.0;
@@ -35,41 +34,31 @@ struct Accum {
     __device__ double value() const { return sum + comp; }
 };
 
-// Finds the bin that holds rank k of a lane's histogram column (read only: every wavefront of the
-// workgroup does the same search and must find the same bin).
-__device__ inline void pick_bin(const uint32_t *col, uint32_t &k, uint64_t &prefix, int shift) {
-    uint32_t cum = 0, before = 0, sel = 0;
-    bool found = false;
-#pragma unroll 8
-    for (int bin = 0; bin < kBins; ++bin) {
-        const uint32_t c = col[bin * kWave];
-        if (!found && cum + c > k) {
-            found = true;
-            sel = (uint32_t)bin;
-            before = cum;
-        }
-        cum += c;
+constexpr int kStatsThreads = 1024;
+constexpr uint64_t kNotAccepted = ~0ull;
+
+__device__ inline Accum wave_sum(Accum v) {  // lanes of a wavefront, fixed order
+    for (int d = 32; d > 0; d >>= 1) {
+        const double s2 = __shfl_down(v.sum, d), c2 = __shfl_down(v.comp, d);
+        v.add(s2);
+        v.add(c2);
     }
-    prefix |= (uint64_t)sel << shift;
-    k -= before;
+    return v;
 }
 
-// What a wavefront found in its slice of a model's requests, handed to the others through LDS.
-struct Partial {
-    double sum[kStatsWaves][kWave], comp[kStatsWaves][kWave], first[kStatsWaves][kWave], last[kStatsWaves][kWave];
-    int32_t n[kStatsWaves][kWave];
-};
-
-__global__ __launch_bounds__(kStatsWaves *kWave) void model_stats_kernel(StatsArgs a) {
-    extern __shared__ uint32_t hist[];  // [2][kBins][64], then Partial
-    Partial &part = *reinterpret_cast<Partial *>(hist + 2 * kBins * kWave);
-    const int lane = threadIdx.x % kWave, wv = threadIdx.x / kWave;
-    const int wave = blockIdx.x;
-    const int m = blockIdx.y;
-    const int stream = a.paired ? a.tile_seed[wave] : wave / a.tiles;
+__global__ __launch_bounds__(kStatsThreads) void model_stats_kernel(StatsArgs a) {
+    __shared__ uint32_t hist[2][kBins];
+    __shared__ double part_sum[kStatsThreads / kWave], part_comp[kStatsThreads / kWave];
+    __shared__ int32_t part_n[kStatsThreads / kWave];
+    __shared__ long long part_first[kStatsThreads / kWave], part_last[kStatsThreads / kWave];
+    __shared__ uint64_t sh_pre[2];
+    __shared__ uint32_t sh_k[2];
+    __shared__ double sh_total;
+    const int tid = threadIdx.x, wv = tid / kWave, ln = tid % kWave;
+    const int row = blockIdx.x, sim = a.sim0 + row, m = blockIdx.y;  // row: the simulation's scratch row in this launch
+    const int stream = a.sim_stream[sim];
     const MqEntry *__restrict__ q = a.mq[stream];
     const int64_t lo = a.lo[stream], hi = a.hi[stream];
-    // a model's entries are in stream order: cut [e0, e1) down to the requests of the window [lo, hi)
     auto first_at_least = [&](int64_t b0, int64_t b1, int64_t v) {
         while (b0 < b1) {
             const int64_t mid = b0 + (b1 - b0) / 2;
@@ -79,142 +68,142 @@ __global__ __launch_bounds__(kStatsWaves *kWave) void model_stats_kernel(StatsAr
     };
     const int64_t m0 = a.mq_off[(size_t)stream * (a.M + 1) + m], m1 = a.mq_off[(size_t)stream * (a.M + 1) + m + 1];
     const int64_t e0 = first_at_least(m0, m1, lo), e1 = first_at_least(e0, m1, hi);
-    // the wavefronts of the workgroup share the model's requests in contiguous slices, in order
-    const int64_t per = (e1 - e0 + kStatsWaves - 1) / kStatsWaves;
-    const int64_t s0 = std::min(e1, e0 + wv * per), s1 = std::min(e1, s0 + per);
+    const double *__restrict__ fin = a.finish + a.sim_base[sim];
+    const uint8_t *__restrict__ gd = a.good + a.sim_base[sim];
+    uint64_t *__restrict__ scr = a.scratch + (size_t)row * (size_t)a.scratch_pitch;
 
-    uint32_t *col0 = hist + lane, *col1 = hist + kBins * kWave + lane;
-    auto clear = [&]() {  // each wavefront clears its share of the bins
-        for (int bin = wv; bin < kBins; bin += kStatsWaves) col0[bin * kWave] = col1[bin * kWave] = 0;
-    };
-    clear();
+    for (int b = tid; b < 2 * kBins; b += kStatsThreads) (&hist[0][0])[b] = 0;
     __syncthreads();
 
-    const size_t base = (size_t)wave * (size_t)a.Rmax * kWave + lane;
-    const double *__restrict__ fin = a.finish + base;
-    const uint8_t *__restrict__ gd = a.good + base;
-
+    // pass 0: gather, count, sum, first and last accepted request, top byte
     int32_t n = 0;
-    double first = 0.0, last = 0.0, mean = 0.0, lat_sum = 0.0, dev_sum = 0.0;
+    long long first_e = 0x7FFFFFFFFFFFFFFFll, last_e = -1;
     Accum acc;
-    uint64_t pre0 = 0, pre1 = 0;
-    uint32_t k0 = 0, k1 = 0;
-
-    for (int pass = 0; pass < 8; ++pass) {
-        const int shift = 56 - 8 * pass;
-        const uint64_t fixed = pass == 0 ? 0ull : ~0ull << (shift + 8);  // digits the earlier passes have fixed
-        auto take = [&](bool ok, double lat, double t) {
-            if (!ok) return;
-            const uint64_t bits = (uint64_t)__double_as_longlong(lat);
-            if (pass == 0) {
-                if (n == 0) first = t;
-                last = t;
-                n += 1;
-                acc.add(lat);
-            } else if (pass == 1) {
-                const double d = lat - mean;
-                acc.add(d * d);
-            }
-            const uint32_t bin = (uint32_t)(bits >> shift) & (kBins - 1);
-            if ((bits & fixed) == pre0) atomicAdd(&col0[bin * kWave], 1u);
-            if ((bits & fixed) == pre1) atomicAdd(&col1[bin * kWave], 1u);
-        };
-        // A block's rows are fetched together, and the entries of the next block (clamped to the slice) while
-        // this one is counted: the loop is bound by memory latency.
-        int32_t idx[kUnroll];
-        double t[kUnroll];
-        auto entries = [&](int64_t e) {
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const int64_t at = std::min(e + u, s1 - 1);
-                idx[u] = q[at].idx;
-                t[u] = q[at].t;
-            }
-        };
-        if (s0 < s1) entries(s0);
-        for (int64_t e = s0; e < s1; e += kUnroll) {
-            double f[kUnroll], at_t[kUnroll];
-            uint8_t g[kUnroll];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const size_t row = (size_t)idx[u] * kWave;
-                f[u] = fin[row];
-                g[u] = gd[row];
-                at_t[u] = t[u];
-            }
-            entries(e + kUnroll);
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) take(e + u < s1 && g[u] != 0, f[u] - at_t[u], at_t[u]);
+    for (int64_t e = e0 + tid; e < e1; e += kStatsThreads) {
+        const size_t row = (size_t)q[e].idx * kWave;
+        const bool ok = gd[row] != 0;
+        const double lat = fin[row] - q[e].t;
+        const uint64_t bits = ok ? (uint64_t)__double_as_longlong(lat) : kNotAccepted;
+        scr[e] = bits;
+        if (ok) {
+            n += 1;
+            acc.add(lat);
+            first_e = e < first_e ? e : first_e;
+            last_e = e > last_e ? e : last_e;
+            atomicAdd(&hist[0][(uint32_t)(bits >> 56)], 1u);
         }
-        if (pass <= 1) {  // the slices' counts and compensated sums, added up in slice order by every wavefront
-            part.sum[wv][lane] = acc.sum;
-            part.comp[wv][lane] = acc.comp;
-            if (pass == 0) {
-                part.n[wv][lane] = n;
-                part.first[wv][lane] = first;
-                part.last[wv][lane] = last;
-            }
+    }
+    auto block_sum = [&](Accum v) -> double {  // the workgroup's compensated sum, added up in a fixed order; in every thread
+        v = wave_sum(v);
+        if (ln == 0) {
+            part_sum[wv] = v.sum;
+            part_comp[wv] = v.comp;
         }
         __syncthreads();
-        if (pass <= 1) {
+        if (tid == 0) {
             Accum all;
-            int32_t count = 0;
-            for (int w = 0; w < kStatsWaves; ++w) {
-                all.add(part.sum[w][lane]);
-                all.add(part.comp[w][lane]);
-                if (pass == 0 && part.n[w][lane] > 0) {
-                    if (count == 0) first = part.first[w][lane];
-                    last = part.last[w][lane];
-                    count += part.n[w][lane];
-                }
+            for (int w = 0; w < kStatsThreads / kWave; ++w) {
+                all.add(part_sum[w]);
+                all.add(part_comp[w]);
             }
-            if (pass == 0) {
-                n = count;
-                lat_sum = all.value();
-                mean = n > 0 ? lat_sum / (double)n : 0.0;
-                k0 = (uint32_t)(int32_t)(0.90 * (double)n);  // int(0.90 * len(sorted_latency)), workload.py:345
-                k1 = (uint32_t)(int32_t)(0.99 * (double)n);
-            } else {
-                dev_sum = all.value();
-            }
-            acc = Accum();
+            sh_total = all.value();
         }
-        pick_bin(col0, k0, pre0, shift);
-        pick_bin(col1, k1, pre1, shift);
-        __syncthreads();  // everyone has read the bins (and the partial sums)
-        clear();
+        __syncthreads();
+        return sh_total;
+    };
+    const double lat_sum = block_sum(acc);
+    for (int d = 32; d > 0; d >>= 1) {
+        n += __shfl_down(n, d);
+        const long long f2 = __shfl_down(first_e, d), l2 = __shfl_down(last_e, d);
+        first_e = f2 < first_e ? f2 : first_e;
+        last_e = l2 > last_e ? l2 : last_e;
+    }
+    if (ln == 0) {
+        part_n[wv] = n;
+        part_first[wv] = first_e;
+        part_last[wv] = last_e;
+    }
+    __syncthreads();
+    n = 0;
+    first_e = 0x7FFFFFFFFFFFFFFFll;
+    last_e = -1;
+    for (int w = 0; w < kStatsThreads / kWave; ++w) {
+        n += part_n[w];
+        first_e = part_first[w] < first_e ? part_first[w] : first_e;
+        last_e = part_last[w] > last_e ? part_last[w] : last_e;
+    }
+    const double mean = n > 0 ? lat_sum / (double)n : 0.0;
+    double dev_sum = 0.0;
+
+    if (tid == 0) {
+        sh_pre[0] = sh_pre[1] = 0;
+        sh_k[0] = (uint32_t)(int32_t)(0.90 * (double)n);  // int(0.90 * len(sorted_latency)), workload.py:345
+        sh_k[1] = (uint32_t)(int32_t)(0.99 * (double)n);
+    }
+    __syncthreads();
+    for (int pass = 0; pass < 8; ++pass) {
+        const int shift = 56 - 8 * pass;
+        if (pass > 0) {
+            const uint64_t fixed = ~0ull << (shift + 8);
+            const uint64_t pre0 = sh_pre[0], pre1 = sh_pre[1];
+            Accum dev;
+            for (int64_t e = e0 + tid; e < e1; e += kStatsThreads) {
+                const uint64_t bits = scr[e];
+                if (bits == kNotAccepted) continue;
+                if (pass == 1) {
+                    const double d = __longlong_as_double((long long)bits) - mean;
+                    dev.add(d * d);
+                }
+                const uint32_t bin = (uint32_t)(bits >> shift) & (kBins - 1);
+                if ((bits & fixed) == pre0) atomicAdd(&hist[0][bin], 1u);
+                if ((bits & fixed) == pre1) atomicAdd(&hist[1][bin], 1u);
+            }
+            if (pass == 1) dev_sum = block_sum(dev);
+        }
+        __syncthreads();
+        if (tid < 2) {  // thread h finds the bin that holds rank k of histogram h (pass 0: both ranks in histogram 0)
+            const uint32_t *hh = hist[pass == 0 ? 0 : tid];
+            uint32_t k = sh_k[tid], cum = 0, sel = 0, before = 0;
+            bool found = false;
+            for (int bin = 0; bin < kBins; ++bin) {
+                const uint32_t c = hh[bin];
+                if (!found && cum + c > k) {
+                    found = true;
+                    sel = (uint32_t)bin;
+                    before = cum;
+                }
+                cum += c;
+            }
+            sh_pre[tid] |= (uint64_t)sel << shift;
+            sh_k[tid] = k - before;
+        }
+        __syncthreads();
+        for (int b = tid; b < 2 * kBins; b += kStatsThreads) (&hist[0][0])[b] = 0;
         __syncthreads();
     }
 
-    if (wv != 0) return;
-    const size_t o = ((size_t)wave * a.M + m) * kWave + lane;
+    if (tid != 0) return;
+    const size_t o = (size_t)sim * a.M + m;
     a.model_req[o] = (int32_t)(e1 - e0);
     a.model_good[o] = n;
-    a.first_start[o] = first;
-    a.last_start[o] = last;
+    a.first_start[o] = n > 0 ? q[first_e].t : 0.0;
+    a.last_start[o] = n > 0 ? q[last_e].t : 0.0;
     a.latency_sum[o] = n > 0 ? lat_sum : 0.0;
-    a.latency_mean[o] = mean;  // a model without accepted requests reports the latencies [0] (workload.py:340-342)
+    a.latency_mean[o] = mean;
     a.latency_std[o] = n > 0 ? sqrt(dev_sum / (double)n) : 0.0;
-    a.latency_p90[o] = n > 0 ? __longlong_as_double((long long)pre0) : 0.0;
-    a.latency_p99[o] = n > 0 ? __longlong_as_double((long long)pre1) : 0.0;
+    a.latency_p90[o] = n > 0 ? __longlong_as_double((long long)sh_pre[0]) : 0.0;
+    a.latency_p99[o] = n > 0 ? __longlong_as_double((long long)sh_pre[1]) : 0.0;
 }
 
 }  // namespace
 
-hipError_t launch_model_stats(const StatsArgs &args, int waves, hipStream_t stream, std::string *err) {
-    constexpr size_t lds = 2 * kBins * kWave * sizeof(uint32_t) + sizeof(Partial);
-    if (waves <= 0 || args.M <= 0) return hipSuccess;
+hipError_t launch_model_stats(const StatsArgs &args, int n_sims, hipStream_t stream, std::string *err) {
+    if (n_sims <= 0 || args.M <= 0) return hipSuccess;
     if (args.M > 65535) {
         if (err) *err = "model_stats_kernel: more than 65535 models";
         return hipErrorInvalidValue;
     }
-    hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(model_stats_kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (rc != hipSuccess) {
-        if (err) *err = "model_stats_kernel: cannot raise the LDS limit";
-        return rc;
-    }
-    hipLaunchKernelGGL(model_stats_kernel, dim3((unsigned)waves, (unsigned)args.M), dim3(kStatsWaves * kWave), lds, stream, args);
+    hipLaunchKernelGGL(model_stats_kernel, dim3((unsigned)n_sims, (unsigned)args.M), dim3(kStatsThreads), 0, stream, args);
     return hipGetLastError();
 }
 

@@ -1,8 +1,8 @@
 """GPU parity of the statistics kernel (mmsim_batch_model_stats) with
 Workload.compute_stats' conventions (workload.py:308-354).
 
-The kernel reduces the per-request outputs that the simulation kernels left in
-device memory; the check fetches those same outputs and reduces them with
+The kernel (one workgroup per simulation and model) reduces the per-request
+outputs that the simulation kernels left in device memory; the check fetches those same outputs and reduces them with
 numpy (``model_stats_numpy``: sort, ``sorted[int(q * n)]``, ``np.mean``,
 ``np.std``).  Bars: counts, first / last accepted arrival and both percentiles
 bit-exact; sum, mean and deviation within 1e-12 relative (compensated sums on
@@ -57,6 +57,13 @@ def test_plain_simulator_two_streams_every_window(eng):
     assert 0 < out["good"].mean() < 1       # both accepted and rejected requests took part
 
 
+def test_more_simulations_than_scratch_rows_take_several_launches(eng, monkeypatch):
+    cfg = make_config(2, 11)
+    R = len(cfg.stream(0).tstamps)
+    monkeypatch.setenv("MMSIM_STATS_SCRATCH_BYTES", str(3 * 8 * R + 100))   # three simulations per launch, 22 in all
+    _check(eng, cfg, cfg.placements, (0, 1), [(0, 0), (R // 9, R // 8)])
+
+
 def test_more_placements_than_one_wavefront_and_deep_pipelines(eng):
     cfg = make_config(4, 96)
     cfg.duration *= 0.02        # about 20000 requests
@@ -69,6 +76,18 @@ def test_batching_simulator(eng):
     cfg.duration *= 0.05
     R = len(cfg.stream(0).tstamps)
     _check(eng, cfg, cfg.placements, (0,), [(0,), (R // 9,)], flags=_lib.BATCHING)
+
+
+@pytest.mark.parametrize("config, placements, seeds, shrink, flags", [
+    (2, 5, (0, 1), 1.0, 0), (4, 1, (2,), 0.05, 0), (4, 16, (1,), 0.02, 0), (5, 3, (0,), 0.05, _lib.BATCHING)],
+    ids=["cfg2-5x2", "cfg4-1", "cfg4-16", "cfg5-3-batching"])
+def test_a_handful_of_simulations(eng, config, placements, seeds, shrink, flags):
+    """One placement on one stream is what approximate_one_case(fast_stats=False) sends."""
+    cfg = make_config(config, placements)
+    cfg.duration *= shrink
+    R = min(len(cfg.stream(s).tstamps) for s in seeds)
+    _check(eng, cfg, cfg.placements, seeds, [tuple(0 for _ in seeds), tuple(R // 11 for _ in seeds),
+                                             tuple(R // 2 + 3 for _ in seeds)], flags=flags)
 
 
 def test_requires_per_request_outputs_and_the_same_streams(eng):
