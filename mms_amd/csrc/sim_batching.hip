@@ -525,8 +525,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             const int col = ilog2i(bs);
             int32_t next_rank;
             if constexpr (COOP) {
-                const int kb = kfirst + bs;
-                next_rank = (int32_t)oct_get((uint32_t)(kb < 8 ? ir.y : rank8), kb & 7);
+                const int kb = kfirst + bs;  // batches of sixteen and more reach past what was fetched
+                next_rank = kb < 16 ? (int32_t)oct_get((uint32_t)(kb < 8 ? ir.y : rank8), kb & 7) : a.mq[first + bs].rank;
             } else {
                 next_rank = a.mq[first + bs].rank;
             }

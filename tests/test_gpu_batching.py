@@ -64,6 +64,53 @@ def test_random_cases_match_oracle(eng):
             assert np.array_equal(a, b), seed
 
 
+def test_batches_of_sixteen_and_more(eng):
+    """Batches larger than the sixteen queue entries that an octet fetches at once: the arrival behind the batch
+    and the members past the fetched ones come from memory.  (Seeds found by a randomized comparison.)"""
+    biggest = 0
+    for seed in (137, 160, 179, 215, 226, 304, 311, 412, 497, 592, 593, 647, 664, 773, 857, 1000, 1006, 1091):
+        nb = 1 + seed % 6
+        assert nb >= 5
+        c = random_case(9_000_000 + seed, max_m=2 + seed % 12, max_g=1 + seed % 14, max_s=1 + seed % 8, max_r=300,
+                        nb=nb, load=0.5 + (seed % 23), inf_slo=False, tie_prob=0.05 * (seed % 8),
+                        p_member=0.2 + 0.1 * (seed % 7))
+        bss = [1 << k for k in range(nb)]
+        f0, g0, c0, _ = oracle_c.simulate_requests_mixed_batching(
+            c["tstamps"], c["model_ids"], c["slos"], c["m2g"], c["g2m"], c["num_stages"], c["lat"], bss)
+        fin, good, cnt = _single(eng, c, bss)
+        assert np.array_equal(good, g0), seed
+        assert np.array_equal(fin.view(np.uint64), f0.view(np.uint64)), seed
+        for a, b in zip(cnt, c0):
+            assert np.array_equal(a, b), seed
+        if g0.any():
+            biggest = max(biggest, int(np.unique(f0[g0], return_counts=True)[1].max()))
+    assert biggest >= 16
+
+
+@pytest.mark.parametrize("lanes", [8, 64])
+def test_batch_sizes_that_are_not_powers_of_two(eng, monkeypatch, lanes):
+    """The latency column of a batch size is floor(log2(size)) (controller.py:668, :716), so sizes such as 3 and 5
+    share columns with 2 and 4; the kernel's shortcut for sizes 1, 2, 4, ... must not be taken then."""
+    monkeypatch.setenv("MMSIM_BATCHING_LANES", str(lanes))
+    odd = [1, 2, 3, 5, 8, 9, 17]        # floor(log2) = 0, 1, 1, 2, 3, 3, 4
+    grown = 0
+    for seed in range(60):
+        nb = 2 + seed % 6
+        c = random_case(5_000_000 + 1000 * lanes + seed, max_m=6, max_g=4, max_s=5, max_r=250, nb=nb,
+                        load=3.0 + seed % 9, inf_slo=False)
+        bss = odd[:nb]
+        f0, g0, c0, _ = oracle_c.simulate_requests_mixed_batching(
+            c["tstamps"], c["model_ids"], c["slos"], c["m2g"], c["g2m"], c["num_stages"], c["lat"], bss)
+        fin, good, cnt = _single(eng, c, bss)
+        assert np.array_equal(good, g0), seed
+        assert np.array_equal(fin.view(np.uint64), f0.view(np.uint64)), seed
+        for a, b in zip(cnt, c0):
+            assert np.array_equal(a, b), seed
+        served = f0[g0]
+        grown += int(len(served) - len(np.unique(served)))     # requests that shared a batch finish together
+    assert grown > 100
+
+
 @pytest.mark.parametrize("lanes", [8, 16, 32, 64])
 @pytest.mark.parametrize("lds_tables", [0, 1, 2, 3])
 def test_every_kernel_variant(eng, monkeypatch, lanes, lds_tables):
