@@ -187,8 +187,10 @@ int mmsim_batch_fetch(mmsim_batch *batch, mmsim_result *out);
  * the reference's latency = [0] does (:340-342).
  *
  * Counts, times and the two percentiles are exact.  Sum, mean and deviation
- * are compensated sums: within 1e-14 relative of the exact value, hence within
- * 1e-12 of numpy's pairwise sums, but not bit-equal to them.
+ * are compensated sums: sum and mean within 1e-14 relative of the exact value,
+ * hence within 1e-12 of numpy's pairwise sums, but not bit-equal to them; a
+ * deviation far below the mean (nearly equal latencies) is exact to 1e-12 of
+ * the mean, not of itself -- in numpy as well.
  *
  * The batch must have been created with MMSIM_WANT_PER_REQUEST and run;
  * `workloads` are the n_streams streams it was created with (their per-model

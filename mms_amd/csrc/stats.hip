@@ -11,7 +11,7 @@
 // the top byte on the way; every thread later reads back only what it wrote itself.
 //
 // Percentiles are order statistics: sorted[int(q * n)] (workload.py:344-346), found exactly with a
-// radix selection on the bit pattern of the latency (positive doubles order as their bits do): eight
+// radix selection on a 64-bit key that orders like the latency (its bit pattern with the sign handled): eight
 // passes of eight bits, most significant first, counting into 256 bins in LDS the elements that match
 // the digits fixed so far; both percentiles in the same passes (two histograms).  The first pass also
 // counts and sums (n decides the two ranks), the second one sums the squared deviations.  Sums are
@@ -35,7 +35,19 @@ struct Accum {
 };
 
 constexpr int kStatsThreads = 1024;
+// Latencies are selected by a 64-bit key that orders like the double (sign flipped for positive values, all bits
+// for negative ones: the batching simulator can finish a request before it arrived, when a group that became idle
+// earlier picks it up with its old idle time, controller.py:739-744, :715-720).  All ones is the key of a NaN
+// pattern and marks requests that were not accepted.
 constexpr uint64_t kNotAccepted = ~0ull;
+__device__ inline uint64_t key_of(double v) {
+    const uint64_t bits = (uint64_t)__double_as_longlong(v);
+    return bits ^ ((uint64_t)((long long)bits >> 63) | 0x8000000000000000ull);
+}
+__device__ inline double value_of(uint64_t key) {
+    const uint64_t bits = (key >> 63) ? key ^ 0x8000000000000000ull : ~key;
+    return __longlong_as_double((long long)bits);
+}
 
 __device__ inline Accum wave_sum(Accum v) {  // lanes of a wavefront, fixed order
     for (int d = 32; d > 0; d >>= 1) {
@@ -83,7 +95,7 @@ __global__ __launch_bounds__(kStatsThreads) void model_stats_kernel(StatsArgs a)
         const size_t row = (size_t)q[e].idx * kWave;
         const bool ok = gd[row] != 0;
         const double lat = fin[row] - q[e].t;
-        const uint64_t bits = ok ? (uint64_t)__double_as_longlong(lat) : kNotAccepted;
+        const uint64_t bits = ok ? key_of(lat) : kNotAccepted;
         scr[e] = bits;
         if (ok) {
             n += 1;
@@ -151,7 +163,7 @@ __global__ __launch_bounds__(kStatsThreads) void model_stats_kernel(StatsArgs a)
                 const uint64_t bits = scr[e];
                 if (bits == kNotAccepted) continue;
                 if (pass == 1) {
-                    const double d = __longlong_as_double((long long)bits) - mean;
+                    const double d = value_of(bits) - mean;
                     dev.add(d * d);
                 }
                 const uint32_t bin = (uint32_t)(bits >> shift) & (kBins - 1);
@@ -191,8 +203,8 @@ __global__ __launch_bounds__(kStatsThreads) void model_stats_kernel(StatsArgs a)
     a.latency_sum[o] = n > 0 ? lat_sum : 0.0;
     a.latency_mean[o] = mean;
     a.latency_std[o] = n > 0 ? sqrt(dev_sum / (double)n) : 0.0;
-    a.latency_p90[o] = n > 0 ? __longlong_as_double((long long)sh_pre[0]) : 0.0;
-    a.latency_p99[o] = n > 0 ? __longlong_as_double((long long)sh_pre[1]) : 0.0;
+    a.latency_p90[o] = n > 0 ? value_of(sh_pre[0]) : 0.0;
+    a.latency_p99[o] = n > 0 ? value_of(sh_pre[1]) : 0.0;
 }
 
 }  // namespace
