@@ -216,13 +216,17 @@ COUNTS_IN_LDS = -2          # the same counts, per-group counters in LDS
 
 
 @pytest.mark.parametrize("flags", [0, COUNTS_IN_REGISTERS, COUNTS_IN_LDS, ALL])
-@pytest.mark.parametrize("groups,regions,segment", [(1, 1, 64), (3, 2, 256), (5, 8, 512), (64, 8, 16384)])
-def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, groups, regions, segment):
+@pytest.mark.parametrize("groups,regions,segment,spin", [(1, 1, 64, None), (3, 2, 256, None), (5, 8, 512, None),
+                                                        (64, 8, 16384, None), (1, 8, 64, 0), (2, 5, 128, 1)])
+def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, groups, regions, segment, spin):
     """The loop over runs is launched as a schedule: a workgroup owns several (tile, stream) items, its
     LDS is cut into regions sized by the items' clock slots, and its wavefronts simulate the items a
     segment at a time, clocks parked in device memory in between.  Forced here on a small batch with
     few workgroups, few regions and short segments: 420 placements using 4..56 devices (7 tiles of
-    different sizes x 2 streams of odd, unequal lengths), every output level."""
+    different sizes x 2 streams of odd, unequal lengths), every output level.  With ``spin`` 0 or 1 a
+    wavefront that finds all the items it could take in other wavefronts' hands leaves at once instead
+    of waiting (normally it would look again for about 70 ms): the holders then finish the items alone,
+    and every item must still be completed."""
     from types import SimpleNamespace
     from mms_amd.profiling import ParallelConfig
     from mms_amd.placement_policy.base_policy import ModelPlacement
@@ -231,6 +235,8 @@ def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, group
     monkeypatch.setenv("MMSIM_SCHED_GROUPS", str(groups))
     monkeypatch.setenv("MMSIM_WAVES_PER_CU", str(regions))
     monkeypatch.setenv("MMSIM_SEGMENT_REQUESTS", str(segment))
+    if spin is not None:
+        monkeypatch.setenv("MMSIM_SCHED_SPIN_LIMIT", str(spin))
     if flags in (COUNTS_IN_REGISTERS, COUNTS_IN_LDS):
         monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", "0" if flags == COUNTS_IN_REGISTERS else "1")
         flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
