@@ -814,9 +814,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         }
         if (m >= 0) {
             // every lane sees the same arrival count; lanes that do not host m never read it
+            // (all lanes read the same count and write the same count + 1: no lane needs to be singled out, and
+            // a wavefront's LDS accesses are carried out in program order)
             __builtin_amdgcn_wave_barrier();
-            if (lane == 0) arrived[m] += 1u;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            const uint32_t seen = arrived[m];
+            arrived[m] = seen + 1u;
             __builtin_amdgcn_wave_barrier();
         }
         if (!queued) {
