@@ -150,7 +150,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const bool want_group = (a.flags & MMSIM_WANT_GROUP_COUNTS) != 0;
     const bool want_req = (a.flags & MMSIM_WANT_PER_REQUEST) != 0;
     const int M = a.M, Gmax = a.Gmax, NB = a.NB;
-    const int LS = a.lane_stride;  // simulations per wavefront (64, 32, 16 or 8): pitch of the per-simulation LDS arrays
+    // simulations per wavefront (64, 32, 16 or 8): pitch of the per-simulation LDS arrays.  Octets mean 8: a constant
+    // there, so that the index arithmetic is shifts, not multiplications
+    const int LS = OCT ? 8 : a.lane_stride;
     const int sl = OCT ? lane >> 3 : lane;  // this lane's simulation within the tile
     const int oj = OCT ? lane & 7 : 0;      // this lane's place in its octet
     const int fill = OCT ? kWave : LS;      // lanes that fill the wavefront's shared LDS arrays
