@@ -163,16 +163,17 @@ struct mmsim_batch {
     DevBuf<uint32_t> rep32, repx32;
     DevBuf<uint64_t> rep8;
     DevBuf<uint8_t> repx;
-    DevBuf<uint8_t> rmax, slot_group;
+    DevBuf<uint8_t> rmax;
     DevBuf<int32_t> kerr;
     DevBuf<uint32_t> ginfo;
     DevBuf<float> lat;
     DevBuf<int32_t> n_good;
     DevBuf<double> lat_sum;
     DevBuf<int32_t> model_good, group_req, group_good;
-    DevBuf<unsigned long long> slot_cnt;      // per-group counts by last clock slot [waves][nslots][64] (group_global)
-    std::vector<int16_t> group_last_slot;     // [B][Gmax] last clock slot of each group, -1: no such group (group_global)
-    int32_t group_global = 0, slot_rows = 0;
+    DevBuf<unsigned long long> slot_cnt;      // plain simulator: per-group counts by last clock slot [waves][nslots][64]
+    std::vector<int16_t> group_last_slot;     // [B][Gmax] last clock slot of each group, -1: no such group
+    int32_t group_by_slot = 0, slot_rows = 0; // group_by_slot: the group counts are in slot_cnt (else in group_req / group_good)
+    int32_t group_lds = 0;                    // the kernel keeps the slot counters in LDS while it runs
     DevBuf<double> finish;
     DevBuf<uint8_t> good;
     DevBuf<int64_t> fp_ops;
@@ -406,14 +407,12 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     }
     if (const char *env = std::getenv("MMSIM_WAVES_PER_CU")) wpb_cap = std::max(1, std::min(kMaxWavesPerBlock, std::atoi(env)));
     // plain simulator, per wavefront: request block | replica bounds | clocks (one extra row that stays +inf)
-    // | slot owners | group counters | model counters; the latency table is shared by the workgroup
+    // | slot counters | model counters; the latency table is shared by the workgroup
     size_t model_lds_bytes = 0;  // per-model counters [M][64] in LDS (decided below)
-    bool group_in_lds = (flags & MMSIM_WANT_GROUP_COUNTS) != 0;  // slot owners and group counters in LDS (decided below)
+    bool group_in_lds = false;   // a 64-bit counter per (clock slot, lane) in LDS (decided below)
     auto mixed_wave_bytes = [&](int ns) {
         return ((size_t)mixed_clock_offset(rmax_lds_bytes, runs) + (size_t)(ns + 1) * kSlotBytes +
-                (group_in_lds
-                     ? (((size_t)ns * kWave + 15) & ~(size_t)15) + (size_t)2 * Gmax * kWave * sizeof(uint32_t)
-                     : 0) + model_lds_bytes + 15) & ~(size_t)15;
+                (group_in_lds ? (size_t)ns * kSlotBytes : 0) + model_lds_bytes + 15) & ~(size_t)15;
     };
     if (!batching) {
         wave_bytes = mixed_wave_bytes(nslots);  // of the largest placement
@@ -433,30 +432,42 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             lds_tail = 0;
             pow2_depths = false;
         }
-        // Per-group counters: slot owners and counters in LDS can cost a CU a wavefront (configuration 4: three
-        // instead of four, i.e. three rounds of wavefronts instead of two).  The counts-only kernel can keep them in
-        // registers per lane instead and add them to global rows when the lane's group changes; that is used when
-        // it gives a CU more wavefronts.  MMSIM_GROUP_COUNTS_LDS=0/1 forces the choice (tuning knob).
-        if (group_in_lds && !(flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT))) {
-            const size_t room = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail;
-            const size_t with = std::min<size_t>(wpb_cap, room / wave_bytes);
-            group_in_lds = false;
-            const size_t without = std::min<size_t>(wpb_cap, room / mixed_wave_bytes(nslots));
-            group_in_lds = without <= with;
-            if (const char *env = std::getenv("MMSIM_GROUP_COUNTS_LDS")) group_in_lds = std::atoi(env) != 0;
+        // Per-model and per-group counters.  In LDS (a row of 64-bit counters per clock slot, a row of 32-bit counters
+        // per model) they cost one LDS add each per request, but the rows can cost a CU wavefronts (configuration 4:
+        // 32 KB more per wavefront).  Without LDS the group counts are kept per lane in registers and added to global
+        // rows when the lane's group changes, and accepted requests are added to global per-model rows, which a lone
+        // wavefront has to wait behind (small batches: about 300 cycles per request).  So the counters go to LDS, both
+        // kinds together, when that does not lower the wavefronts a CU gets.  MMSIM_COUNTS_LDS=0/1 forces the choice
+        // (tuning knob).  With per-request outputs or operation counts (the general kernel) each kind goes to LDS if
+        // it fits at all.
+        const size_t room = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail;
+        const size_t model_rows = (size_t)M * kWave * sizeof(uint32_t);
+        if (flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT)) {
+            group_in_lds = (flags & MMSIM_WANT_GROUP_COUNTS) != 0;
             wave_bytes = mixed_wave_bytes(nslots);
-        }
-        // Per-model counters: one relaxed add to a global row per accepted (lane, request) costs a small
-        // batch (one wavefront per CU, nothing to hide behind) about 300 cycles per request, because later
-        // loads wait behind it; counters in LDS do not.  They take M * 256 bytes per wavefront, so they are
-        // used when that does not lower the wavefronts a CU gets.
-        if (flags & MMSIM_WANT_MODEL_COUNTS) {
-            const size_t room = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail, extra = (size_t)M * kWave * sizeof(uint32_t);
-            const size_t used_now = std::min<size_t>(wpb_cap, room / wave_bytes);
-            if (wave_bytes + extra <= room && std::min<size_t>(wpb_cap, room / (wave_bytes + extra)) >= used_now) {
-                model_lds_bytes = extra;
+            if (group_in_lds && wave_bytes > room) {
+                group_in_lds = false;
                 wave_bytes = mixed_wave_bytes(nslots);
             }
+            if ((flags & MMSIM_WANT_MODEL_COUNTS) && wave_bytes + model_rows <= room) {
+                model_lds_bytes = model_rows;
+                wave_bytes = mixed_wave_bytes(nslots);
+            }
+        } else if (flags & (MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) {
+            group_in_lds = false;
+            const size_t without = std::min<size_t>(wpb_cap, room / mixed_wave_bytes(nslots));
+            group_in_lds = true;
+            model_lds_bytes = model_rows;
+            const size_t with = std::min<size_t>(wpb_cap, room / mixed_wave_bytes(nslots));
+            bool in_lds = with >= 1 && with >= without;
+            if (const char *env = std::getenv("MMSIM_COUNTS_LDS")) in_lds = with >= 1 && std::atoi(env) != 0;
+            if (!in_lds) {
+                group_in_lds = false;
+                model_lds_bytes = 0;
+            }
+            wave_bytes = mixed_wave_bytes(nslots);
+        } else {
+            group_in_lds = false;
         }
     } else {
         // per wavefront: descriptors | clocks | event times | chunk minima | queue heads | head ranks | event
@@ -736,18 +747,6 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             }
         });
     }
-    std::vector<uint8_t> slot_group;
-    if (!batching && (flags & MMSIM_WANT_GROUP_COUNTS)) {
-        slot_group.assign((size_t)b->tiles * nslots * kWave, 0);
-        for (int32_t p = 0; p < B; ++p) {
-            const int tile = b->pos[p] / kWave, lane = b->pos[p] % kWave;
-            for (int32_t g = 0; g < rl.num_groups[p]; ++g) {
-                const int pp = t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]];
-                for (int k = 0; k < pp; ++k)
-                    slot_group[((size_t)tile * nslots + slot0[(size_t)p * Gmax + g] + k) * kWave + lane] = (uint8_t)g;
-            }
-        }
-    }
     std::vector<int32_t> tile_begin;
     std::vector<uint8_t> rmax((size_t)b->tiles * M, 0);
     // (by tile: the placements of a tile write that tile's rows only)
@@ -925,10 +924,6 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (!repx32.empty())
             HIP_TRY(hipMemcpyAsync(b->repx32.p, repx32.data(), sizeof(uint32_t) * repx32.size(), hipMemcpyHostToDevice, st));
     }
-    if (!slot_group.empty()) {
-        HIP_TRY(b->slot_group.alloc(slot_group.size()));
-        HIP_TRY(hipMemcpyAsync(b->slot_group.p, slot_group.data(), slot_group.size(), hipMemcpyHostToDevice, st));
-    }
     if (b->paired) {
         HIP_TRY(b->tile_seed.alloc(tile_stream.size()));
         HIP_TRY(hipMemcpyAsync(b->tile_seed.p, tile_stream.data(), sizeof(int32_t) * tile_stream.size(), hipMemcpyHostToDevice, st));
@@ -975,12 +970,13 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     HIP_TRY(b->n_good.alloc(lanes_padded));
     HIP_TRY(b->lat_sum.alloc(lanes_padded));
     if (flags & MMSIM_WANT_MODEL_COUNTS) HIP_TRY(b->model_good.alloc(lanes_padded * M));
-    if (flags & MMSIM_WANT_GROUP_COUNTS) {
+    if (batching && (flags & MMSIM_WANT_GROUP_COUNTS)) {
         HIP_TRY(b->group_req.alloc(lanes_padded * Gmax));
         HIP_TRY(b->group_good.alloc(lanes_padded * Gmax));
     }
-    if (!batching && (flags & MMSIM_WANT_GROUP_COUNTS) && !group_in_lds) {
-        b->group_global = 1;
+    if (!batching && (flags & MMSIM_WANT_GROUP_COUNTS)) {
+        b->group_by_slot = 1;
+        b->group_lds = group_in_lds ? 1 : 0;
         b->slot_rows = nslots;
         HIP_TRY(b->slot_cnt.alloc(lanes_padded * (size_t)nslots));
         b->group_last_slot.assign((size_t)B * Gmax, -1);
@@ -1039,7 +1035,6 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.rep32 = reinterpret_cast<const uint4 *>(b->rep32.p);
     a.repx32 = b->repx32.p;
     a.rmax = b->rmax.p;
-    a.slot_group = b->slot_group.p;
     a.lat_lds_bytes = (int32_t)lat_bytes;
     a.error = b->kerr.p;
     a.lat = b->lat.p;
@@ -1063,15 +1058,13 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.lat_sum = b->lat_sum.p;
     a.model_good = b->model_good.p;
     a.model_lds = model_lds_bytes ? 1 : 0;
-    a.group_global = b->group_global;
+    a.group_lds = b->group_lds;
     a.slot_cnt = b->slot_cnt.p;
     a.xcd_map = 1;
     a.runs = runs ? 1 : 0;
     a.skip_ahead = 1;
     if (const char *env = std::getenv("MMSIM_SKIP_AHEAD")) a.skip_ahead = std::atoi(env) ? 1 : 0;  // tuning knob
     if (const char *env = std::getenv("MMSIM_XCD_MAP")) a.xcd_map = std::atoi(env) ? 1 : 0;  // tuning knob
-    a.group_req = b->group_req.p;
-    a.group_good = b->group_good.p;
     a.finish = b->finish.p;
     a.good = b->good.p;
     a.fp_ops = b->fp_ops.p;
@@ -1286,7 +1279,7 @@ int mmsim_batch_run(mmsim_batch *b) {
     HIP_TRY(hipSetDevice(ctx->device));
     if (b->flags & MMSIM_WANT_MODEL_COUNTS)
         HIP_TRY(hipMemsetAsync(b->model_good.p, 0, b->model_good.bytes(), ctx->stream));
-    if (b->group_global) {
+    if (b->group_by_slot) {
         HIP_TRY(hipMemsetAsync(b->slot_cnt.p, 0, b->slot_cnt.bytes(), ctx->stream));
     }
     if ((b->flags & MMSIM_BATCHING) && (b->flags & MMSIM_WANT_GROUP_COUNTS)) {
@@ -1385,7 +1378,7 @@ int mmsim_batch_fetch(mmsim_batch *b, mmsim_result *out) {
                     out->model_num_requests[((size_t)s * B + p) * M + m] =
                         (b->hosted.empty() || b->hosted[(size_t)p * M + m]) ? b->wl_model_requests[(size_t)(b->paired ? b->stream_of[p] : s)][m] : 0;
     }
-    if (wg && b->group_global) {  // counted per last clock slot of the group: map slots back to groups
+    if (wg && b->group_by_slot) {  // counted per last clock slot of the group: map slots back to groups
         std::vector<unsigned long long> h(b->slot_cnt.n);
         HIP_TRY(hipMemcpy(h.data(), b->slot_cnt.p, b->slot_cnt.bytes(), hipMemcpyDeviceToHost));
         const size_t rows = (size_t)b->slot_rows;

@@ -91,14 +91,13 @@ struct MixedArgs {
     const uint4 *rep32;          // [tiles][M][2][64] descriptors of the first 8 replicas, four to a 16-byte word
     const uint32_t *repx32;      // [tiles][M][rep_extra][64] descriptors of replicas 8, 9, ...
     const uint8_t *rmax;         // [tiles][M] most replicas of model m over the tile's lanes
-    const uint8_t *slot_group;   // [tiles][nslots][64] group that owns each clock slot (only with group counters)
     const float *lat;            // [M][lat_row] compact stage latencies (batch size 1)
     int32_t M, lat_row, rep_extra;
     int32_t n_seeds, B, tiles, nslots, Gmax;
     const int32_t *tile_seed;    // paired batches: the one stream each tile is simulated on (see `paired`)
     int32_t paired;              // 1: every tile has its own stream and results are laid out as for one seed;
                                  // 0: every tile is simulated on every stream
-    int32_t slot_rows;           // row pitch of slot_group (most slots of any tile)
+    int32_t slot_rows;           // row pitch of slot_cnt (most slots of any tile)
     int32_t state_rows;          // row pitch of state
     double *state;               // [waves][state_rows][64] clocks parked between segments (scheduled launch)
     // Scheduled launch (loop over runs): workgroup w owns the items wg_off[w] .. wg_off[w+1]-1, an item being one
@@ -129,18 +128,18 @@ struct MixedArgs {
     int32_t *n_good;             // [n_seeds][tiles*64]
     double *lat_sum;             // [n_seeds][tiles*64]
     int32_t *model_good;         // [waves][M][64]
-    int32_t *group_req;          // [waves][Gmax][64]
-    int32_t *group_good;         // [waves][Gmax][64]
     double *finish;              // [waves][Rmax][64]
     uint8_t *good;               // [waves][Rmax][64]
     int64_t *fp_ops;             // [n_seeds][tiles*64]
     int32_t *error;              // set to 1 if the kernel finds its LDS layout assumption broken
-    int32_t model_lds;           // 1: per-model counters [M][64] live in LDS behind the group counters (small batches,
+    int32_t model_lds;           // 1: per-model counters [M][64] live in LDS behind the slot counters (small batches,
                                  // where LDS is not what limits the wavefronts per CU); 0: relaxed adds to model_good
-    int32_t group_global;        // 1: per-group counts are kept per lane in registers and added to slot_cnt when
-                                 // the lane's group changes (no group counters or slot owners in LDS); 0: counters in LDS
-    unsigned long long *slot_cnt;  // [waves][slot_rows][64] requests (low half) and accepted requests (high half) of the group
-                                 // whose last clock slot this is (group_global; zeroed by the host before the first segment)
+    // Per-group counts are kept per clock slot: the row of a group's last stage holds, per lane, its requests (low half)
+    // and accepted requests (high half); the host knows which slot is which group's last.
+    int32_t group_lds;           // 1: a row of 64-bit counters per clock slot in LDS behind the clocks, one add per request,
+                                 // added to slot_cnt when the turn ends (small batches); 0: counts per lane in registers,
+                                 // added to slot_cnt when the lane's group changes
+    unsigned long long *slot_cnt;  // [waves][slot_rows][64], zeroed by the host before the launch
     int32_t runs;                // 1: the request loop walks runs of equal models (streams whose requests mostly repeat the
                                  // model of the one before); 0: fixed chunks of four requests
     int32_t skip_ahead;          // 1: requests that every lane must reject are found a block at a time and not simulated (scores only)
@@ -151,7 +150,7 @@ struct MixedArgs {
 // that bakes LDS addresses into the replica descriptors:
 //   [latency table][wavefront 0][wavefront 1]...
 //   wavefront: [64 staged requests (chunked loop only)][replica bounds u8[M]]
-//              [clocks: nslots+1 rows of 64 f64][slot owners][group counters]
+//              [clocks: nslots+1 rows of 64 f64][slot counters: nslots rows of 64 u64][model counters]
 // Row nslots of the clocks is the +inf row that empty descriptors point at.
 // rmax_lds_bytes is M rounded up to 16.
 __host__ __device__ inline uint32_t mixed_clock_offset(int32_t rmax_lds_bytes, bool runs) {

@@ -133,6 +133,11 @@ __device__ __forceinline__ void lds_set_f64(uint32_t addr, double v) {
     *reinterpret_cast<__attribute__((address_space(3))) double *>(addr) = v;
 }
 
+// 64-bit LDS add that returns nothing (the wavefront does not wait for it; LDS operations of a wavefront stay in order)
+__device__ __forceinline__ void lds_add_u64(uint32_t addr, unsigned long long v) {
+    asm volatile("ds_add_u64 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+
 // 32-bit LDS byte address of a pointer into shared memory (for ds_* in inline asm).
 __device__ __forceinline__ uint32_t lds_addr(const void *p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
@@ -234,7 +239,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     constexpr bool SCHED = RUNS;
 
     // ---- LDS: [latency table][schedule state (SCHED)][per wavefront: request block (chunked loop) | replica
-    //            bounds | clocks (+inf row last) | slot owners | group counters | model counters].
+    //            bounds | clocks (+inf row last) | slot counters | model counters].
     if (lds_addr(lds_raw) != 0u) {  // the descriptors assume the dynamic LDS starts at address 0
         if (threadIdx.x == 0) *a.error = 1;
         return;
@@ -271,9 +276,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     double *clk = reinterpret_cast<double *>(lds_raw + clk_off) + lane;
     const uint32_t rel_base = SCHED ? clk_off : 0u;  // what turns a descriptor's clock address into an LDS address
     // Counter homes: output level 1 keeps no counters in LDS (its request loop carries no code for them)
-    const bool group_regs = want_group && (OUT == 1 || a.group_global != 0);  // counts per lane in registers, flushed to global rows
-    const bool group_lds = OUT >= 2 && want_group && !group_regs;
-    const bool model_lds = OUT >= 2 && want_model && a.model_lds != 0;
+    // Level 2 is compiled for counters in LDS and keeps both kinds, wanted or not (the host provides the room), so
+    // that its request loop tests no flag; level 3 looks at the arguments.
+    const bool group_lds = OUT == 2 || (OUT == 3 && want_group && a.group_lds != 0);  // a 64-bit counter per (clock slot, lane) in LDS
+    const bool group_regs = want_group && !group_lds;  // counts per lane in registers, added to global rows when the group changes
+    const bool model_lds = OUT == 2 || (OUT == 3 && want_model && a.model_lds != 0);
     if constexpr (!SCHED) {
         if (live)
             for (int i = lane; i < a.M; i += kWave) rmax_lds[i] = a.rmax[(size_t)tile * a.M + i];
@@ -344,10 +351,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         for (int i = lane; i < a.M; i += kWave) rmax_lds[i] = a.rmax[(size_t)tile * a.M + i];
     }
     const int nslots = SCHED ? a.item_nslots[item0 + item_k] : a.nslots;
-    const int own_bytes = group_lds ? ((nslots * kWave + 15) & ~15) : 0;
-    uint8_t *owner = lds_raw + clk_off + (nslots + 1) * kSlotBytes;  // owner[slot * 64 + lane]
-    uint32_t *gcnt = reinterpret_cast<uint32_t *>(owner + own_bytes) + lane;
-    uint32_t *mcnt = gcnt + (group_lds ? 2 * a.Gmax * kWave : 0);  // [M][64] accepted requests per model
+    // Slot counters (group_lds): one row per clock row, behind the clocks.  The counter of the group whose last-stage
+    // clock is at LDS address x is at x + cnt_rel: requests in the low half, accepted requests in the high half.
+    const uint32_t cnt_rel = (uint32_t)(nslots + 1) * kSlotBytes;
+    unsigned long long *scnt = reinterpret_cast<unsigned long long *>(lds_raw + clk_off + cnt_rel) + lane;  // [nslots][64]
+    uint32_t *mcnt = reinterpret_cast<uint32_t *>(lds_raw + clk_off + cnt_rel + (group_lds ? nslots * kSlotBytes : 0)) + lane;  // [M][64] accepted requests per model
 
     const int wave = a.paired ? tile : seed * a.tiles + tile;  // where this (tile, stream) pair's results go
     const size_t out = (size_t)wave * kWave + lane;
@@ -360,8 +368,6 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const bool resume = seg > 0;
     const bool last_seg = r1 >= R;
     double *saved = a.state + (size_t)wave * a.state_rows * kWave + lane;
-    int32_t *greq = a.group_req + (size_t)wave * a.Gmax * kWave + lane;
-    int32_t *ggood = a.group_good + (size_t)wave * a.Gmax * kWave + lane;
 
     int32_t n_good = 0;
     double lat_sum = 0.0;
@@ -375,17 +381,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         for (int s = 0; s < nslots; ++s) clk[s * kWave] = 0.0;
     }
     clk[nslots * kWave] = __builtin_inf();
-    if (group_lds) {
-        for (int s = 0; s < nslots; ++s) owner[s * kWave + lane] = a.slot_group[((size_t)tile * a.slot_rows + s) * kWave + lane];
-        for (int g = 0; g < a.Gmax; ++g) {
-            gcnt[g * kWave] = resume ? (uint32_t)greq[g * kWave] : 0u;
-            gcnt[(a.Gmax + g) * kWave] = resume ? (uint32_t)ggood[g * kWave] : 0u;
-        }
-    }
+    if (group_lds)
+        for (int s = 0; s < nslots; ++s) scnt[s * kWave] = 0ull;  // of this turn; added to slot_cnt when it ends
 
     int32_t *model_good = a.model_good + (size_t)wave * a.M * kWave + lane;
     if (model_lds)
-        for (int m = 0; m < a.M; ++m) mcnt[m * kWave] = resume ? (uint32_t)model_good[(size_t)m * kWave] : 0u;
+        for (int m = 0; m < a.M; ++m) mcnt[m * kWave] = resume && want_model ? (uint32_t)model_good[(size_t)m * kWave] : 0u;
 
     const int4 *__restrict__ reqs4 = reinterpret_cast<const int4 *>(a.streams + off);
     const uint4 *__restrict__ rep_tile = a.rep32 + (size_t)tile * a.M * 2 * kWave + lane;
@@ -625,12 +626,8 @@ asm volatile(NAME##_TEXT                                                        
         }
         if (group_regs) {
             // counted when the lane's group changes (above)
-        } else if (want_group && has) {  // :611, :618
-            const uint32_t g = owner[(last_addr - clk_off) >> 3];  // (slot * 512 + lane * 8) / 8
-            // LDS adds that return nothing: the wavefront does not wait for them
-            __hip_atomic_fetch_add(&gcnt[g * kWave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-            __hip_atomic_fetch_add(&gcnt[(a.Gmax + g) * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_WAVEFRONT);
+        } else if (group_lds && has) {  // :611, :618
+            lds_add_u64(last_addr + cnt_rel, acc ? 0x100000001ull : 1ull);
         }
         if (want_ops) {
             asm volatile("" ::: "memory");  // keep this a wave-uniform branch, off the common path
@@ -646,9 +643,8 @@ asm volatile(NAME##_TEXT                                                        
             }
             if (has) fp_ops += 2 * (sm1 + 1) + nvalid + 3;
         }
-        if (model_lds) {  // an LDS add that returns nothing
-            if (m >= 0)
-                __hip_atomic_fetch_add(&mcnt[m * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        if (model_lds) {  // an LDS add that returns nothing (a request of an unknown model is accepted by nobody: adds 0 to row 0)
+            __hip_atomic_fetch_add(&mcnt[(m < 0 ? 0 : m) * kWave], acc ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
         } else if (want_model && !model_per_run && m >= 0 && acc) {  // one owner per counter: a relaxed add that nobody waits for
             __hip_atomic_fetch_add(&model_good[(size_t)m * kWave], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -757,11 +753,8 @@ asm volatile(NAME##_TEXT                                                        
                         if constexpr (OUT == 2) {
                             // requests of the run that are passed over for good
                             const int passed = __builtin_popcountll(next < 64 ? later & ~(~0ull << next) : later);
-                            if (group_lds && passed > 0 && ch_sm1 >= 0) {
-                                const uint32_t g = owner[(ch_last - clk_off) >> 3];
-                                __hip_atomic_fetch_add(&gcnt[g * kWave], (uint32_t)passed, __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_WAVEFRONT);
-                            }
+                            if (group_lds && passed > 0 && ch_sm1 >= 0)
+                                lds_add_u64(ch_last + cnt_rel, (unsigned long long)passed);
                         }
                         if (!todo) break;
                         later &= ~1ull << next;
@@ -840,13 +833,13 @@ asm volatile(NAME##_TEXT                                                        
     if (want_ops) a.fp_ops[out] = fp_ops;
     if (!last_seg)
         for (int s = 0; s < nslots; ++s) saved[(size_t)s * kWave] = clk[s * kWave];
-    if (model_lds)
+    if (model_lds && want_model)
         for (int m = 0; m < a.M; ++m) model_good[(size_t)m * kWave] = (int32_t)mcnt[m * kWave];
     if (group_regs) flush_group((uint32_t)(r1 - r0));
-    if (group_lds) {
-        for (int g = 0; g < a.Gmax; ++g) {
-            greq[g * kWave] = (int32_t)gcnt[g * kWave];
-            ggood[g * kWave] = (int32_t)gcnt[(a.Gmax + g) * kWave];
+    if (group_lds && want_group) {  // one owner per counter at a time (segments of an item follow one another)
+        for (int s = 0; s < nslots; ++s) {
+            const unsigned long long v = scnt[s * kWave];
+            if (v != 0ull) __hip_atomic_fetch_add(&slot_cnt[s * kWave + lane], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     if constexpr (SCHED) {
@@ -894,8 +887,7 @@ template <int SMAX, bool UNIFORM>
 hipError_t launch_u(const MixedArgs &args, int wpb, size_t lds_bytes, hipStream_t stream) {
     // what the request loop has to produce: 0 scores only, 1 also per-model / per-group counts without counters in
     // LDS, 2 counts with counters in LDS (small batches), 3 anything
-    const bool lds_counters = ((args.flags & MMSIM_WANT_GROUP_COUNTS) && !args.group_global) ||
-                              ((args.flags & MMSIM_WANT_MODEL_COUNTS) && args.model_lds);
+    const bool lds_counters = args.group_lds && args.model_lds;  // both or neither, unless per-request outputs are asked for
     const int out = (args.flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT)) ? 3
                     : (args.flags & (MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) ? (lds_counters ? 2 : 1) : 0;
     if (!args.lat_in_lds) return launch_one<SMAX, false, UNIFORM, false, 3>(args, wpb, lds_bytes, stream);
@@ -929,8 +921,7 @@ int smax_bucket_for(int smax) {
 // The template instance launch_sim_mixed picks for these arguments, as profilers print it (same choices as
 // launch_u / launch_s above).
 std::string sim_mixed_kernel_name(const MixedArgs &args, int sb) {
-    const bool lds_counters = ((args.flags & MMSIM_WANT_GROUP_COUNTS) && !args.group_global) ||
-                              ((args.flags & MMSIM_WANT_MODEL_COUNTS) && args.model_lds);
+    const bool lds_counters = args.group_lds && args.model_lds;  // both or neither, unless per-request outputs are asked for
     int out = (args.flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT)) ? 3
               : (args.flags & (MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) ? (lds_counters ? 2 : 1) : 0;
     bool latlds = args.lat_in_lds != 0, pow2 = latlds && (sb == 4 || sb == 16) && args.pow2_depths;

@@ -238,7 +238,7 @@ def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, group
     if spin is not None:
         monkeypatch.setenv("MMSIM_SCHED_SPIN_LIMIT", str(spin))
     if flags in (COUNTS_IN_REGISTERS, COUNTS_IN_LDS):
-        monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", "0" if flags == COUNTS_IN_REGISTERS else "1")
+        monkeypatch.setenv("MMSIM_COUNTS_LDS", "0" if flags == COUNTS_IN_REGISTERS else "1")
         flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
     traces = bool(flags & _lib.WANT_PER_REQUEST)
     rng = np.random.default_rng(77)
@@ -361,7 +361,7 @@ def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placem
     # (group counters in LDS, or in registers with adds to global rows when a lane's group changes)
     for runs, lds in (("1", "1"), ("1", "0"), ("0", "0")):
         monkeypatch.setenv("MMSIM_RUNS", runs)
-        monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", lds)
+        monkeypatch.setenv("MMSIM_COUNTS_LDS", lds)
         batch = E.Batch(eng, [dw], table, packed, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
         for _ in range(2):      # a second run starts from zeroed counters again
             batch.run()
@@ -381,7 +381,7 @@ def test_runs_of_one_model_with_odd_requests(eng, monkeypatch, loop, flags):
     monkeypatch.setenv("MMSIM_RUNS", "1" if loop == "runs" else "0")
     if flags >= 1000:       # per-group counts alone, kept in registers and added to global rows
         flags -= 1000
-        monkeypatch.setenv("MMSIM_GROUP_COUNTS_LDS", "0")
+        monkeypatch.setenv("MMSIM_COUNTS_LDS", "0")
     cfg = make_config(2)
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
     packed = E.pack_placements(cfg.placements, table)
