@@ -469,16 +469,18 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         // repeat the model of the one before, and most of a burst is rejected).
         if (!RUNS || m != ch_model || ch_stale) {  // the chunked loop always scans
             Cand win{__builtin_inf(), kEmpty, 0.0f};
-            if (n > 4)
+            // (one to four listed replicas is the usual case: it is the straight path, the others branch off it)
+            if (__builtin_expect(n > 4, 0)) {
                 scan(win, Idx<8>{});
-            else if (n > 0)
-                scan(win, Idx<4>{});
-            if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
-                const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
-                for (int j = RREG; j < n; ++j) {
-                    const uint32_t d = row[(size_t)(j - RREG) * kWave];
-                    win = first_min(win, Cand{lds_f64(rep_addr(d) + rel_base), d, lrow_m[rep_lat_last(d)]});
+                if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
+                    const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
+                    for (int j = RREG; j < n; ++j) {
+                        const uint32_t d = row[(size_t)(j - RREG) * kWave];
+                        win = first_min(win, Cand{lds_f64(rep_addr(d) + rel_base), d, lrow_m[rep_lat_last(d)]});
+                    }
                 }
+            } else if (__builtin_expect(n > 0, 1)) {
+                scan(win, Idx<4>{});
             }
             if constexpr (RUNS) win.l = lrow_m[rep_lat_last(win.d)];
             // a clock that is infinite (a group that served a request with infinite latency) is never
