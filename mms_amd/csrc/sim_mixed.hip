@@ -445,12 +445,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             const bool right = y.c < x.c;
             return Cand{vmin(x.c, y.c), right ? y.d : x.d, right ? y.l : x.l};
         };
-        auto scan = [&](Cand &win, auto NJ) {
-            constexpr int nj = decltype(NJ)::value;
+        auto scan = [&](Cand &win, auto J0) {  // entries J0 .. J0 + 3
+            constexpr int j0 = decltype(J0)::value, nj = 4;
             Cand k[nj];
             static_while<0, nj>([&](auto J) {
                 constexpr int j = decltype(J)::value;
-                k[j].d = pick_desc<j>(da, db);
+                k[j].d = pick_desc<j0 + j>(da, db);
                 k[j].c = lds_f64(rep_addr(k[j].d) + rel_base);
                 // (loop over runs: the winner's latency is read after the tournament instead, one read for eight)
                 k[j].l = RUNS ? 0.0f : lrow_m[rep_lat_last(k[j].d)];
@@ -458,10 +458,6 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             });
             const Cand a01 = first_min(k[0], k[1]), a23 = first_min(k[2], k[3]);
             win = first_min(a01, a23);
-            if constexpr (nj == 8) {
-                const Cand a45 = first_min(k[4], k[5]), a67 = first_min(k[6], k[7]);
-                win = first_min(win, first_min(a45, a67));
-            }
         };
         // Clocks change only when a request is accepted, so while no lane of the wavefront has
         // accepted anything since the last scan, a request for the same model finds the same group
@@ -469,18 +465,34 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         // repeat the model of the one before, and most of a burst is rejected).
         if (!RUNS || m != ch_model || ch_stale) {  // the chunked loop always scans
             Cand win{__builtin_inf(), kEmpty, 0.0f};
-            // (one to four listed replicas is the usual case: it is the straight path, the others branch off it)
-            if (__builtin_expect(n > 4, 0)) {
-                scan(win, Idx<8>{});
-                if (n > RREG) {  // rare: more than 8 replicas, read the rest on demand
-                    const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
-                    for (int j = RREG; j < n; ++j) {
-                        const uint32_t d = row[(size_t)(j - RREG) * kWave];
-                        win = first_min(win, Cand{lds_f64(rep_addr(d) + rel_base), d, lrow_m[rep_lat_last(d)]});
-                    }
+            // The loop over runs serves bursty streams of well-replicated models: it fetches eight entries at once
+            // when the tile lists more than four.  The chunked loop serves streams of many models with few replicas
+            // each: one to four listed replicas are its straight path, entries 4-7 a second step off that path.
+            auto beyond_eight = [&]() {  // rare: more than 8 replicas, read the rest on demand
+                const uint32_t *row = repx_tile + (size_t)m * a.rep_extra * kWave;
+                for (int j = RREG; j < n; ++j) {
+                    const uint32_t d = row[(size_t)(j - RREG) * kWave];
+                    win = first_min(win, Cand{lds_f64(rep_addr(d) + rel_base), d, lrow_m[rep_lat_last(d)]});
                 }
-            } else if (__builtin_expect(n > 0, 1)) {
-                scan(win, Idx<4>{});
+            };
+            if constexpr (RUNS) {
+                if (__builtin_expect(n > 4, 0)) {
+                    Cand more;
+                    scan(win, Idx<0>{});
+                    scan(more, Idx<4>{});
+                    win = first_min(win, more);  // the final of the tournament of eight: entries 0-3 against 4-7
+                    if (n > RREG) beyond_eight();
+                } else if (__builtin_expect(n > 0, 1)) {
+                    scan(win, Idx<0>{});
+                }
+            } else {
+                if (__builtin_expect(n > 0, 1)) scan(win, Idx<0>{});
+                if (__builtin_expect(n > 4, 0)) {
+                    Cand more;
+                    scan(more, Idx<4>{});
+                    win = first_min(win, more);
+                    if (n > RREG) beyond_eight();
+                }
             }
             if constexpr (RUNS) win.l = lrow_m[rep_lat_last(win.d)];
             // a clock that is infinite (a group that served a request with infinite latency) is never
