@@ -142,8 +142,12 @@ def main():
                     help="scores: goodput+latency only; model: + per-model counts; stats: + per-group counts")
     ap.add_argument("--model-stats", action="store_true",
                     help="time mmsim_batch_model_stats (serving statistics of the per-request outputs, on the device) "
-                         "instead of the simulation: use with --placements 64 --seeds 1")
+                         "instead of the simulation; the per-request outputs of every simulation stay on the device, so "
+                         "it defaults to --placements 64 --seeds 1")
     args = ap.parse_args()
+    if args.model_stats:    # 9 bytes per (simulation, request): the full batch would not fit
+        args.placements = 64 if args.placements is None else args.placements
+        args.seeds = 1 if args.seeds is None else args.seeds
 
     if args.gpus != 1:
         print("bench.py: this build evaluates placements on ONE GPU; --gpus must be 1 "

@@ -30,7 +30,9 @@ FLAGS = [
 # One wavefront per SIMD is the rule for the plain simulator's kernel (LDS-bound occupancy), so
 # instruction-level parallelism inside a wavefront is what hides latency: schedule for it (measured
 # -7 % kernel time).  The batching kernel is built with the default scheduler (this one fails on it).
-SOURCE_FLAGS = {"sim_mixed.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"]}
+# Blocks that are only reached by a branch start on a 64-byte boundary: a taken branch costs a lone wavefront
+# tens of cycles, less when its target starts an instruction cache line (measured: -1 % in the counts mode).
+SOURCE_FLAGS = {"sim_mixed.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp", "-mllvm", "-align-all-nofallthru-blocks=6"]}
 
 
 def _compile(src, extra, src_dir=HERE, obj_dir=OBJ_DIR):
