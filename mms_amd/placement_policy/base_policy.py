@@ -45,8 +45,23 @@ class ModelPlacement:
         the sort must be the stable sort on the model tuples (:29-35)."""
         rows = [tuple(sorted(ms)) for ms in self.group_models]
         order = sorted(range(len(self.group_configs)), key=rows.__getitem__)
-        return ModelPlacement(tuple(self.group_configs[i] for i in order),
-                              tuple(rows[i] for i in order))
+        out = ModelPlacement(tuple(self.group_configs[i] for i in order),
+                             tuple(rows[i] for i in order))
+        out._canonical = True  # not a field: lets add_model_normalized skip the sorts that change nothing
+        return out
+
+    def add_model_normalized(self, group_id: int, model_id: int):
+        """``add_model(group_id, model_id).normalize()``; cheaper when this placement is already in
+        canonical form (only the touched row is re-sorted)."""
+        if not getattr(self, "_canonical", False):
+            return self.add_model(group_id, model_id).normalize()
+        rows = list(self.group_models)
+        rows[group_id] = tuple(sorted(rows[group_id] + (model_id,)))
+        order = sorted(range(len(rows)), key=rows.__getitem__)
+        cfgs = self.group_configs
+        out = ModelPlacement(tuple([cfgs[i] for i in order]), tuple([rows[i] for i in order]))
+        out._canonical = True
+        return out
 
     def copy(self):
         return ModelPlacement(list(self.group_configs), [list(ms) for ms in self.group_models])
@@ -273,12 +288,22 @@ class PlacementEvaluator:
         if not self._is_plain(sols):
             return [(st.goodput, [x.goodput for x in st.per_model_stats], st.group_num_requests, st)
                     for st in self._mixed_stats(sols)]
+        stats_of = self.get_stats_lazy(sols)
+        return [stats_of(b) for b in range(len(sols))]
+
+    def get_stats_lazy(self, sols: List[ModelPlacement]):
+        """One batch for all of ``sols`` like ``get_stats``; returns a function
+        that builds the ``get_stats`` entry of placement ``b`` when asked.  For
+        callers that evaluate more placements than they will read (the look-ahead
+        of the greedy search).  Plain placements and the fast simulator only."""
+        assert self.method == "fast_simulator" and self._is_plain(sols)
         out = self._run(sols, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
         arrivals = self.workload.arrivals
         R = len(arrivals)
         interval = arrivals[-1] - arrivals[0]
-        ret = []
-        for b, sol in enumerate(sols):
+
+        def stats_of(b):
+            sol = sols[b]
             mreq = out["model_num_requests"][0, b]
             mgood = out["model_num_good"][0, b]
             greq = out["group_num_requests"][0, b, :len(sol.group_configs)]
@@ -288,8 +313,8 @@ class PlacementEvaluator:
             goodput = np.float64(out["n_good"][0, b]) / R
             latency_mean = out["latency_sum"][0, b] / R
             stats = StatsResult(per_model, tuple(greq), goodput, latency_mean, R, R / interval)
-            ret.append((stats.goodput, [x.goodput for x in per_model], stats.group_num_requests, stats))
-        return ret
+            return (stats.goodput, [x.goodput for x in per_model], stats.group_num_requests, stats)
+        return stats_of
 
     # -- one placement at a time, same signatures as the reference's static methods -----
     @staticmethod
@@ -409,9 +434,27 @@ def replica_placement_fast_greedy(init_sol: ModelPlacement, model_datas: List[Mo
                                                   evaluator, verbose)[0]
 
 
+def _fast_greedy_successors(sol, weight_mem, cluster_env):
+    """Every (group, model) that ``_fast_greedy_step`` could return for ``sol``, whatever the statistics:
+    the model is not on the group yet and fits beside what the group holds (the same sum as there)."""
+    group_mem = _group_memory(sol, weight_mem)
+    out = []
+    for g_id, (cfg, hosted) in enumerate(zip(sol.group_configs, sol.group_models)):
+        need = weight_mem[cfg]
+        for m_id in range(len(need)):
+            if m_id not in hosted and need[m_id] + group_mem[g_id] <= cluster_env.mem_budget:
+                out.append((g_id, m_id))
+    return out
+
+
+# Most placements one evaluator call of the greedy search may hold when it looks ahead: up to this many,
+# every placement is a lane of a wavefront that has a CU to itself, so the call takes as long as for one.
+FAST_GREEDY_LOOKAHEAD_LANES = 16384
+
+
 def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], model_datas: List[ModelData],
                                            cluster_env: ClusterEnv, workload: Workload,
-                                           evaluator: PlacementEvaluator, verbose: int):
+                                           evaluator: PlacementEvaluator, verbose: int, lookahead: bool = True):
     """``replica_placement_fast_greedy`` for several initial placements at once.
 
     The reference runs one greedy search per enumerated group layout, each
@@ -419,27 +462,65 @@ def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], mode
     :533-541).  The searches do not depend on each other, so they are advanced
     together: every iteration evaluates the current placement of every search
     that is still running in one evaluator call (one lane each on the GPU), and
-    each search takes exactly the step it would take alone.  Returns the final
-    placements in the order of ``init_sols``."""
+    each search takes exactly the step it would take alone.
+
+    A step needs the statistics of one placement, and a call for one placement
+    takes the GPU as long as a call for thousands.  So with ``lookahead`` a
+    call also evaluates every placement the step could lead to (current
+    placement + one replica that fits); when the step is known, the statistics
+    of the placement it leads to are already there and the next step is taken
+    at once: two steps per call, each the step the search would take alone.
+    Used while the call stays within ``FAST_GREEDY_LOOKAHEAD_LANES`` placements
+    and the evaluator is the batched one.  Returns the final placements in the
+    order of ``init_sols``."""
     tic = time.time()
     if evaluator is None:
         evaluator = PlacementEvaluator(model_datas, cluster_env, workload, "fast_simulator", False)
     sols = list(init_sols)
     weight_mems = [weight_mem_table(sol.group_configs, model_datas) for sol in sols]
     running = list(range(len(sols)))
+    can_look = (lookahead and getattr(evaluator, "method", None) == "fast_simulator"
+                and hasattr(evaluator, "get_stats_lazy"))
     it = 0
     while running:
-        all_stats = evaluator.get_stats([sols[i] for i in running])
+        batch, first, kids_of = [], {}, {}
+        look = can_look and all(isinstance(sols[i], ModelPlacement) for i in running)
+        if look:
+            for i in running:
+                kids_of[i] = _fast_greedy_successors(sols[i], weight_mems[i], cluster_env)
+            look = len(running) + sum(len(k) for k in kids_of.values()) <= FAST_GREEDY_LOOKAHEAD_LANES
+        for i in running:
+            first[i] = len(batch)
+            batch.append(sols[i])
+            if look:
+                batch.extend([sols[i].add_model_normalized(g, m) for g, m in kids_of[i]])
+        if look:
+            stats_of = evaluator.get_stats_lazy(batch)
+        else:
+            all_stats = evaluator.get_stats(batch)
+            stats_of = all_stats.__getitem__
         still = []
-        for i, stats in zip(running, all_stats):
+        for i in running:
+            stats = stats_of(first[i])
             choice = _fast_greedy_step(sols[i], stats, weight_mems[i], cluster_env)
             if choice is None:
                 continue
             sols[i] = sols[i].add_model(*choice).normalize()
-            still.append(i)
             if verbose >= 2:
                 print(f"iter: {it}, search: {i}, score: {stats[0]:.4f}, elapsed: {time.time() - tic:.2f}, "
                       f"best placement: {sols[i]}, ")
+            if look and choice in kids_of[i]:
+                at = first[i] + 1 + kids_of[i].index(choice)
+                assert batch[at] == sols[i]
+                stats = stats_of(at)
+                choice = _fast_greedy_step(sols[i], stats, weight_mems[i], cluster_env)
+                if choice is None:
+                    continue
+                sols[i] = sols[i].add_model(*choice).normalize()
+                if verbose >= 2:
+                    print(f"iter: {it}+, search: {i}, score: {stats[0]:.4f}, elapsed: {time.time() - tic:.2f}, "
+                          f"best placement: {sols[i]}, ")
+            still.append(i)
         running = still
         it += 1
     return sols

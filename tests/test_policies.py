@@ -316,16 +316,24 @@ def test_greedy_searches_in_lockstep_take_the_steps_they_take_alone(backend):
     class Counting(PlacementEvaluator):
         calls = 0
 
-        def get_stats(self, sols):
+        def _run(self, sols, flags):
             Counting.calls += 1
-            return super().get_stats(sols)
+            return super()._run(sols, flags)
 
     ev = Counting(model_datas, cluster_env, wl, "fast_simulator", False)
-    alone = [replica_placement_fast_greedy(s, model_datas, cluster_env, wl, ev, 0) for s in starts]
+    alone = [replica_placement_fast_greedy_lockstep([s], model_datas, cluster_env, wl, ev, 0, lookahead=False)[0]
+             for s in starts]
     calls_alone, Counting.calls = Counting.calls, 0
-    together = replica_placement_fast_greedy_lockstep(starts, model_datas, cluster_env, wl, ev, 0)
+    together = replica_placement_fast_greedy_lockstep(starts, model_datas, cluster_env, wl, ev, 0, lookahead=False)
+    calls_together, Counting.calls = Counting.calls, 0
     assert [str(a) for a in alone] == [str(t) for t in together]
-    assert Counting.calls < calls_alone / 2
+    assert calls_together < calls_alone / 2
+    # with the look-ahead a call also evaluates every placement a step can lead to: two steps per call, same steps
+    ahead = replica_placement_fast_greedy_lockstep(starts, model_datas, cluster_env, wl, ev, 0)
+    assert [str(a) for a in alone] == [str(t) for t in ahead]
+    assert Counting.calls <= calls_together // 2 + 1
+    assert [str(a) for a in alone] == [str(replica_placement_fast_greedy(s, model_datas, cluster_env, wl, ev, 0))
+                                       for s in starts]
 
 
 def test_separations_solved_together_equal_separations_solved_one_by_one(backend):
