@@ -135,20 +135,14 @@ def pack_placements(sols: Sequence, table: LatencyTable):
     B = len(sols)
     num_groups = np.fromiter((len(s.group_configs) for s in sols), np.int32, B)
     Gmax = max(int(num_groups.max()) if B else 1, 1)
-    cid = table.config_id
-    if B and int(num_groups.min()) == Gmax:  # every placement has Gmax groups (the usual case): two flat passes
-        group_cfg = np.fromiter(map(cid, chain.from_iterable(s.group_configs for s in sols)),
-                                np.int32, B * Gmax).reshape(B, Gmax)
-        sizes = np.fromiter(map(len, chain.from_iterable(s.group_models for s in sols)),
-                            np.int64, B * Gmax).reshape(B, Gmax)
-    else:
-        group_cfg = np.zeros((B, Gmax), np.int32)
-        sizes = np.zeros((B, Gmax), np.int64)
-        for b, s in enumerate(sols):
-            g = num_groups[b]
-            if g:
-                group_cfg[b, :g] = [cid(c) for c in s.group_configs]
-                sizes[b, :g] = [len(ms) for ms in s.group_models]
+    # two flat passes over all groups of all placements, scattered into the padded [B][Gmax] arrays row by row
+    total_groups = int(num_groups.sum()) if B else 0
+    has = np.arange(Gmax)[None, :] < num_groups[:, None]
+    group_cfg = np.zeros((B, Gmax), np.int32)
+    sizes = np.zeros((B, Gmax), np.int64)
+    group_cfg[has] = np.fromiter(map(table.config_id, chain.from_iterable(s.group_configs for s in sols)),
+                                 np.int32, total_groups)
+    sizes[has] = np.fromiter(map(len, chain.from_iterable(s.group_models for s in sols)), np.int64, total_groups)
     gm_off = np.zeros((B, Gmax + 1), np.int64)
     np.cumsum(sizes, axis=1, out=gm_off[:, 1:])
     per_sol = gm_off[:, -1].copy()
