@@ -488,7 +488,9 @@ def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], mode
         if look:
             for i in running:
                 kids_of[i] = _fast_greedy_successors(sols[i], weight_mems[i], cluster_env)
-            look = len(running) + sum(len(k) for k in kids_of.values()) <= FAST_GREEDY_LOOKAHEAD_LANES
+            # (the batching simulator runs eight placements per wavefront instead of sixty-four)
+            cap = FAST_GREEDY_LOOKAHEAD_LANES // (8 if getattr(evaluator, "enable_batching", False) else 1)
+            look = len(running) + sum(len(k) for k in kids_of.values()) <= cap
         for i in running:
             first[i] = len(batch)
             batch.append(sols[i])
