@@ -263,3 +263,27 @@ def test_alpa_serve_import_names_resolve_to_this_package():
     finally:
         for k in [k for k in sys.modules if k == "alpa_serve" or k.startswith("alpa_serve.")]:
             del sys.modules[k]
+
+
+def test_add_model_normalized_is_add_model_then_normalize():
+    """The greedy look-ahead builds its successor placements with add_model_normalized; it must give what
+    add_model followed by normalize gives (base_policy.py:19-35 of the reference), ties between equal groups
+    included, whether the placement it starts from is in canonical form or not."""
+    import random
+    from mms_amd.placement_policy.base_policy import ModelPlacement
+    from mms_amd.profiling import ParallelConfig
+    rnd = random.Random(5)
+    for _ in range(1500):
+        G = rnd.randint(1, 8)
+        cfgs = [ParallelConfig(1, 1, rnd.choice([1, 2, 4])) for _ in range(G)]
+        rows = [rnd.sample(range(10), rnd.randint(0, 4)) for _ in range(G)]
+        sol = ModelPlacement(cfgs, rows)
+        if rnd.random() < 0.7:
+            sol = sol.normalize()
+        g = rnd.randrange(G)
+        m = rnd.choice([x for x in range(12) if x not in sol.group_models[g]])
+        want = sol.add_model(g, m).normalize()
+        got = sol.add_model_normalized(g, m)
+        assert got == want
+        assert type(got.group_models) is tuple and all(type(r) is tuple for r in got.group_models)
+        assert got.add_model_normalized(0, 99) == got.add_model(0, 99).normalize()
