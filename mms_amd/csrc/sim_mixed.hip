@@ -427,7 +427,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
 
     // One request for the whole wavefront: `at` is its place in the stream, m / n the model and the tile's
     // replica bound for it (wave-uniform), da / db this lane's descriptors of the model's replicas.
-    auto simulate = [&](int64_t at, int m, int n, const uint4 &da, const uint4 &db, double tstamp, double slo) -> uint64_t {
+    // (PLAIN: the caller has seen that the tile lists one to four replicas for the model: the scan has no case to tell)
+    auto simulate = [&](int64_t at, int m, int n, const uint4 &da, const uint4 &db, double tstamp, double slo,
+                        auto PLAIN) -> uint64_t {
+        constexpr bool plain_scan = decltype(PLAIN)::value != 0;
         const float *lrow_m = lat_base + (size_t)(m < 0 ? 0 : m) * a.lat_row;
 
         // ---- choose the replica group: strictly smallest last-stage clock (:590-598).
@@ -485,6 +488,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 } else if (__builtin_expect(n > 0, 1)) {
                     scan(win, Idx<0>{});
                 }
+            } else if constexpr (plain_scan) {
+                scan(win, Idx<0>{});
             } else {
                 if (__builtin_expect(n > 0, 1)) scan(win, Idx<0>{});
                 if (__builtin_expect(n > 4, 0)) {
@@ -730,7 +735,7 @@ asm volatile(NAME##_TEXT                                                        
                 auto request = [&](int i) {
                     return simulate(blk + i, m, n, da, db,
                                     __hiloint2double(__builtin_amdgcn_readlane(r.y, i), __builtin_amdgcn_readlane(r.x, i)),
-                                    (double)__int_as_float(__builtin_amdgcn_readlane(r.w, i)));
+                                    (double)__int_as_float(__builtin_amdgcn_readlane(r.w, i)), Idx<0>{});
                 };
 
                 if constexpr (SKIP) {
@@ -831,12 +836,31 @@ asm volatile(NAME##_TEXT                                                        
             for (int cb = 0; cb < nblk; cb += kChunk) {
                 const bool more = cb + kChunk < nblk;
                 load_chunk(nxt, more ? cb + kChunk : cb);
+                // Single-stage groups: the usual chunk -- four requests, each of a model with one to four listed
+                // replicas -- is simulated as straight-line code (no test between its requests, so that the fetches
+                // of the next chunk and the address arithmetic of the next request fill the waits of the dependent
+                // chain); any other chunk goes the general way.  (With the walk blocks of the deeper buckets, which
+                // branch inside, the second copy of the loop body costs more than it gains: measured.)
+                bool usual = SMAX == 1 && cb + kChunk <= nblk;
                 static_while<0, kChunk>([&](auto U) {
                     constexpr int u = decltype(U)::value;
-                    if (cb + u >= nblk) return false;
-                    simulate(blk + cb + u, cur.m[u], cur.nrep[u], cur.da[u], cur.db[u], cur.t[u], (double)cur.slo[u]);
+                    usual = usual && (unsigned)(cur.nrep[u] - 1) < 4u;
                     return true;
                 });
+                if (__builtin_expect(usual, 1)) {
+                    static_while<0, kChunk>([&](auto U) {
+                        constexpr int u = decltype(U)::value;
+                        simulate(blk + cb + u, cur.m[u], cur.nrep[u], cur.da[u], cur.db[u], cur.t[u], (double)cur.slo[u], Idx<1>{});
+                        return true;
+                    });
+                } else {
+                    static_while<0, kChunk>([&](auto U) {
+                        constexpr int u = decltype(U)::value;
+                        if (cb + u >= nblk) return false;
+                        simulate(blk + cb + u, cur.m[u], cur.nrep[u], cur.da[u], cur.db[u], cur.t[u], (double)cur.slo[u], Idx<0>{});
+                        return true;
+                    });
+                }
                 cur = nxt;
             }
         }
