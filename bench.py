@@ -124,6 +124,69 @@ def model_stats_bench(args, cfg, streams):
     print(json.dumps(result), flush=True)
 
 
+def search_bench(args):
+    """Wall clock of whole placement searches (the callers of the hot path): the three greedy policies on a
+    synthetic problem of 32 models, 32 devices and a training workload of about 1.1e5 requests, with and without
+    the one-step look-ahead of the greedy search.  Prints one JSON line; `value` is greedy steps per second of
+    `ModelParallelismSearch` with the look-ahead."""
+    from mms_amd.placement_policy import (ClusterEnv, ModelData, ModelParallelismGreedy, ModelParallelismSearch,
+                                          SelectiveReplicationGreedy)
+    from mms_amd.placement_policy import base_policy
+    from mms_amd.profiling import ParallelConfig, synthetic_profile
+    from mms_amd.simulator.workload import GammaProcess, Workload
+    from mms_amd.synthetic import power_law_rates
+    GB = 1 << 30
+    num_models, num_devices, total_rate, duration = 32, 32, 60.0, 1800.0
+    configs = [ParallelConfig(1, 1, pp) for pp in (1, 2, 4, 8)]
+    rates = power_law_rates(num_models, total_rate, 0.6)
+    model_datas = []
+    for i in range(num_models):
+        base = [0.15, 0.25, 0.5][i % 3]
+        prof = synthetic_profile(f"p{i % 3}", base, configs, weight_bytes=[2.6, 5.2, 13.4][i % 3] * GB)
+        model_datas.append(ModelData(f"m{i}", base * 5, float(rates[i]), 4.0, prof))
+    workload = Workload.merge(*[GammaProcess(md.rate, md.cv).generate_workload(md.name, 0, duration, slo=md.slo, seed=100 + i)
+                                for i, md in enumerate(model_datas)])
+    cluster_env = ClusterEnv(num_devices, 13 * GB)
+    log(f"[bench] search problem: {num_models} models, {num_devices} devices, {len(workload)} requests")
+
+    calls = [0]
+    run = base_policy.PlacementEvaluator._run
+
+    def counted(self, sols, flags):
+        calls[0] += 1
+        return run(self, sols, flags)
+    base_policy.PlacementEvaluator._run = counted
+    policies = [("ModelParallelismSearch", lambda: ModelParallelismSearch(verbose=0)),
+                ("SelectiveReplicationGreedy", lambda: SelectiveReplicationGreedy(verbose=0)),
+                ("ModelParallelismGreedy(group_size=4)", lambda: ModelParallelismGreedy(group_size=4))]
+    ModelParallelismSearch(verbose=0).solve_placement(model_datas[:4], ClusterEnv(4, 13 * GB), workload)  # warm-up: library, context
+    rows, same = {}, True
+    for name, make in policies:
+        out = {}
+        for mode in ("lookahead", "plain"):
+            base_policy.FAST_GREEDY_LOOKAHEAD = mode == "lookahead"
+            calls[0] = 0
+            t0 = time.perf_counter()
+            sol, _ = make().solve_placement(model_datas, cluster_env, workload)
+            out[mode] = {"seconds": time.perf_counter() - t0, "evaluator_calls": calls[0], "placement": str(sol)}
+        same = same and out["lookahead"]["placement"] == out["plain"]["placement"]
+        rows[name] = {m: {k: v for k, v in r.items() if k != "placement"} for m, r in out.items()}
+        log(f"[bench] {name}: look-ahead {out['lookahead']['seconds']:.2f} s / {out['lookahead']['evaluator_calls']} calls, "
+            f"plain {out['plain']['seconds']:.2f} s / {out['plain']['evaluator_calls']} calls")
+    base_policy.FAST_GREEDY_LOOKAHEAD = True
+    base_policy.PlacementEvaluator._run = run
+    head = rows["ModelParallelismSearch"]
+    steps = head["plain"]["evaluator_calls"]   # one greedy step of every layout per call of the plain loop
+    print(json.dumps({
+        "metric": "greedy placement search, steps of all layouts per second (ModelParallelismSearch, look-ahead)",
+        "value": steps / head["lookahead"]["seconds"], "unit": "steps/s", "n_gpus": 1, "steps": 1, "warmup": 1,
+        "ms_per_step": head["lookahead"]["seconds"] * 1e3 / steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": f"placement search: {num_models} models, {num_devices} devices, {len(workload)} requests in the "
+                               f"training workload, 13 GB per device"},
+        "searches": rows, "same_placements_with_and_without_lookahead": bool(same)}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -144,6 +207,9 @@ def main():
                     help="time mmsim_batch_model_stats (serving statistics of the per-request outputs, on the device) "
                          "instead of the simulation; the per-request outputs of every simulation stay on the device, so "
                          "it defaults to --placements 64 --seeds 1")
+    ap.add_argument("--search", action="store_true",
+                    help="time whole greedy placement searches (the callers of the hot path) with and without the "
+                         "one-step look-ahead instead of the simulation")
     args = ap.parse_args()
     if args.model_stats:    # 9 bytes per (simulation, request): the full batch would not fit
         args.placements = 64 if args.placements is None else args.placements
@@ -153,6 +219,9 @@ def main():
         print("bench.py: this build evaluates placements on ONE GPU; --gpus must be 1 "
               "(lanes are independent, a multi-GPU run would only split the batch).", file=sys.stderr)
         sys.exit(2)
+
+    if args.search:
+        return search_bench(args)
 
     from mms_amd import _lib, engine as E
     from mms_amd.synthetic import make_config

@@ -12,7 +12,7 @@ hands the whole list to the GPU as one batch (one placement per lane).
 import dataclasses
 import time
 from functools import partial
-from typing import List
+from typing import List, Optional
 
 import numpy as np
 
@@ -450,11 +450,12 @@ def _fast_greedy_successors(sol, weight_mem, cluster_env):
 # Most placements one evaluator call of the greedy search may hold when it looks ahead: up to this many,
 # every placement is a lane of a wavefront that has a CU to itself, so the call takes as long as for one.
 FAST_GREEDY_LOOKAHEAD_LANES = 16384
+FAST_GREEDY_LOOKAHEAD = True  # what ``lookahead=None`` means (module switch for measurements)
 
 
 def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], model_datas: List[ModelData],
                                            cluster_env: ClusterEnv, workload: Workload,
-                                           evaluator: PlacementEvaluator, verbose: int, lookahead: bool = True):
+                                           evaluator: PlacementEvaluator, verbose: int, lookahead: Optional[bool] = None):
     """``replica_placement_fast_greedy`` for several initial placements at once.
 
     The reference runs one greedy search per enumerated group layout, each
@@ -479,6 +480,8 @@ def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], mode
     sols = list(init_sols)
     weight_mems = [weight_mem_table(sol.group_configs, model_datas) for sol in sols]
     running = list(range(len(sols)))
+    if lookahead is None:
+        lookahead = FAST_GREEDY_LOOKAHEAD
     can_look = (lookahead and getattr(evaluator, "method", None) == "fast_simulator"
                 and hasattr(evaluator, "get_stats_lazy"))
     it = 0
