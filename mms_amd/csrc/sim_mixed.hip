@@ -129,6 +129,9 @@ __device__ __forceinline__ void wave_min2_u32(uint32_t &x, uint32_t &y) {
 __device__ __forceinline__ double lds_f64(uint32_t addr) {
     return *reinterpret_cast<const __attribute__((address_space(3))) double *>(addr);
 }
+__device__ __forceinline__ float lds_f32(uint32_t addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) float *>(addr);
+}
 __device__ __forceinline__ void lds_set_f64(uint32_t addr, double v) {
     *reinterpret_cast<__attribute__((address_space(3))) double *>(addr) = v;
 }
@@ -427,9 +430,33 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
 
     // One request for the whole wavefront: `at` is its place in the stream, m / n the model and the tile's
     // replica bound for it (wave-uniform), da / db this lane's descriptors of the model's replicas.
-    // (PLAIN: the caller has seen that the tile lists one to four replicas for the model: the scan has no case to tell)
+    // Where the scan of a request's first four replicas reads: the last-stage clocks and the last-stage latencies.
+    // Worked out ahead of the request (it depends on the descriptors only), while the request before waits for LDS.
+    // (LDS byte addresses; used with the latency table in LDS only.)  The empty statement at the end keeps the
+    // compiler from moving the arithmetic to where the addresses are used, which is after the wait.
+    struct ScanAddr {
+        uint32_t c[4];
+        uint32_t l[4];
+    };
+    auto scan_addr = [&](ScanAddr &sa, const uint4 &da, int m) {
+        const uint32_t lrow_m = lds_addr(lat_lds) + (uint32_t)(m < 0 ? 0 : m) * (uint32_t)a.lat_row * 4u;
+        static_while<0, 4>([&](auto J) {
+            constexpr int j = decltype(J)::value;
+            const uint32_t d = pick_desc<j>(da, da);
+            sa.c[j] = rep_addr(d) + rel_base;
+            sa.l[j] = lrow_m + rep_lat_last(d) * 4u;
+            return true;
+        });
+        asm volatile("" : "+v"(sa.c[0]), "+v"(sa.c[1]), "+v"(sa.c[2]), "+v"(sa.c[3]), "+v"(sa.l[0]), "+v"(sa.l[1]),
+                          "+v"(sa.l[2]), "+v"(sa.l[3]));
+    };
+    const ScanAddr no_addr{};
+    auto nothing = []() {};
+
+    // (PLAIN: the caller has seen that the tile lists one to four replicas for the model: the scan has no case to
+    // tell, reads where `sa` says, and calls `meanwhile` once its reads are under way)
     auto simulate = [&](int64_t at, int m, int n, const uint4 &da, const uint4 &db, double tstamp, double slo,
-                        auto PLAIN) -> uint64_t {
+                        auto PLAIN, const ScanAddr &sa, auto &&meanwhile) -> uint64_t {
         constexpr bool plain_scan = decltype(PLAIN)::value != 0;
         const float *lrow_m = lat_base + (size_t)(m < 0 ? 0 : m) * a.lat_row;
 
@@ -454,11 +481,17 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             static_while<0, nj>([&](auto J) {
                 constexpr int j = decltype(J)::value;
                 k[j].d = pick_desc<j0 + j>(da, db);
-                k[j].c = lds_f64(rep_addr(k[j].d) + rel_base);
-                // (loop over runs: the winner's latency is read after the tournament instead, one read for eight)
-                k[j].l = RUNS ? 0.0f : lrow_m[rep_lat_last(k[j].d)];
+                if constexpr (plain_scan) {
+                    k[j].c = lds_f64(sa.c[j]);
+                    k[j].l = lds_f32(sa.l[j]);
+                } else {
+                    k[j].c = lds_f64(rep_addr(k[j].d) + rel_base);
+                    // (loop over runs: the winner's latency is read after the tournament instead, one read for eight)
+                    k[j].l = RUNS ? 0.0f : lrow_m[rep_lat_last(k[j].d)];
+                }
                 return true;
             });
+            if constexpr (plain_scan) meanwhile();
             const Cand a01 = first_min(k[0], k[1]), a23 = first_min(k[2], k[3]);
             win = first_min(a01, a23);
         };
@@ -735,7 +768,7 @@ asm volatile(NAME##_TEXT                                                        
                 auto request = [&](int i) {
                     return simulate(blk + i, m, n, da, db,
                                     __hiloint2double(__builtin_amdgcn_readlane(r.y, i), __builtin_amdgcn_readlane(r.x, i)),
-                                    (double)__int_as_float(__builtin_amdgcn_readlane(r.w, i)), Idx<0>{});
+                                    (double)__int_as_float(__builtin_amdgcn_readlane(r.w, i)), Idx<0>{}, no_addr, nothing);
                 };
 
                 if constexpr (SKIP) {
@@ -841,23 +874,29 @@ asm volatile(NAME##_TEXT                                                        
                 // of the next chunk and the address arithmetic of the next request fill the waits of the dependent
                 // chain); any other chunk goes the general way.  (With the walk blocks of the deeper buckets, which
                 // branch inside, the second copy of the loop body costs more than it gains: measured.)
-                bool usual = SMAX == 1 && cb + kChunk <= nblk;
+                bool usual = SMAX == 1 && LATLDS && cb + kChunk <= nblk;
                 static_while<0, kChunk>([&](auto U) {
                     constexpr int u = decltype(U)::value;
                     usual = usual && (unsigned)(cur.nrep[u] - 1) < 4u;
                     return true;
                 });
                 if (__builtin_expect(usual, 1)) {
+                    ScanAddr sa[2];
+                    scan_addr(sa[0], cur.da[0], cur.m[0]);
                     static_while<0, kChunk>([&](auto U) {
                         constexpr int u = decltype(U)::value;
-                        simulate(blk + cb + u, cur.m[u], cur.nrep[u], cur.da[u], cur.db[u], cur.t[u], (double)cur.slo[u], Idx<1>{});
+                        simulate(blk + cb + u, cur.m[u], cur.nrep[u], cur.da[u], cur.db[u], cur.t[u], (double)cur.slo[u], Idx<1>{},
+                                 sa[u & 1], [&]() {
+                                     if constexpr (u + 1 < kChunk) scan_addr(sa[(u + 1) & 1], cur.da[u + 1], cur.m[u + 1]);
+                                 });
                         return true;
                     });
                 } else {
                     static_while<0, kChunk>([&](auto U) {
                         constexpr int u = decltype(U)::value;
                         if (cb + u >= nblk) return false;
-                        simulate(blk + cb + u, cur.m[u], cur.nrep[u], cur.da[u], cur.db[u], cur.t[u], (double)cur.slo[u], Idx<0>{});
+                        simulate(blk + cb + u, cur.m[u], cur.nrep[u], cur.da[u], cur.db[u], cur.t[u], (double)cur.slo[u], Idx<0>{},
+                                 no_addr, nothing);
                         return true;
                     });
                 }
