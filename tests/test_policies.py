@@ -336,6 +336,39 @@ def test_greedy_searches_in_lockstep_take_the_steps_they_take_alone(backend):
                                        for s in starts]
 
 
+def test_greedy_searches_with_and_without_lookahead_on_random_problems(backend, monkeypatch):
+    """The greedy policies return the same placement whether the search looks a step ahead or not: random small
+    problems (2-9 models, 2-8 devices, pipelines up to 8 stages, memory budgets that bind or do not)."""
+    import random
+    from mms_amd.placement_policy import base_policy
+    from mms_amd.profiling import ParallelConfig, synthetic_profile
+    rnd = random.Random(20)
+    for case in range(16):
+        M, D, budget = rnd.randint(2, 9), rnd.choice([2, 4, 4, 8]), rnd.choice([3.0, 6.0, 13.0]) * GB
+        configs = [ParallelConfig(1, 1, pp) for pp in (1, 2, 4, 8) if pp <= D]
+        model_datas = []
+        for i in range(M):
+            base = rnd.choice([0.05, 0.1, 0.2, 0.4])
+            prof = synthetic_profile(f"p{i}", base, configs, weight_bytes=rnd.choice([1.0, 2.6, 5.2]) * GB)
+            model_datas.append(ModelData(f"m{i}", base * rnd.choice([2, 5, 10]), rnd.choice([0.5, 2.0, 6.0]),
+                                         rnd.choice([1.0, 4.0]), prof))
+        wl = Workload.merge(*[GammaProcess(md.rate, md.cv).generate_workload(md.name, 0, rnd.choice([30.0, 120.0]),
+                                                                             slo=md.slo, seed=rnd.randint(0, 10 ** 6))
+                              for md in model_datas])
+        env = ClusterEnv(D, budget)
+        group_size = rnd.choice([g for g in (1, 2, 4) if D % g == 0])
+        for make in (lambda: ModelParallelismSearch(verbose=0), lambda: SelectiveReplicationGreedy(verbose=0),
+                     lambda: ModelParallelismGreedy(group_size=group_size)):
+            got = []
+            for ahead in (True, False):
+                monkeypatch.setattr(base_policy, "FAST_GREEDY_LOOKAHEAD", ahead)
+                try:
+                    got.append(str(make().solve_placement(model_datas, env, wl)[0]))
+                except AssertionError as e:     # a problem the policy refuses (nothing fits): refused either way
+                    got.append("refused: " + str(e)[:40])
+            assert got[0] == got[1], f"case {case}: {got}"
+
+
 def test_separations_solved_together_equal_separations_solved_one_by_one(backend):
     """model_parallelism.py:432-434 solves every separation on its own; here all their greedy searches
     share one evaluator and advance together.  Same stitched placements."""
