@@ -34,19 +34,40 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def kernel_sources_sha16():
+    """First 16 hex digits of the SHA-256 over the library's kernel and host sources (mms_amd/csrc/*.hip, *.h,
+    *.inc, in name order): what a recorded counter figure is tied to."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "mms_amd", "csrc")
+    for path in sorted(p for ext in ("*.hip", "*.h", "*.inc") for p in glob.glob(os.path.join(src, ext))):
+        h.update(os.path.basename(path).encode() + b"\0")
+        h.update(open(path, "rb").read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(kernel, workload):
     """HBM bytes per launch of `kernel` on `workload` from the committed counter summary
     (profiles/traffic.json: FETCH_SIZE / WRITE_SIZE of a rocprofv3 --pmc run, scaled by the same
-    counters of a device copy of known size), or None when the summary is for another kernel or workload."""
+    counters of a device copy of known size), and where the figure comes from.  The figure is a RECORDED one,
+    not measured in this run (the counters need a profiler run of their own), so it is only given when the
+    record is for this kernel instance, this workload and these very sources; otherwise None."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     if not os.path.exists(path):
-        return None
+        return None, {"status": "no record"}
+    sha = kernel_sources_sha16()
     for e in json.load(open(path)):
         if e["kernel"] == kernel and e["workload"] == workload:
+            about = {"status": "recorded", "source": e.get("source"), "kernel_sources_sha16": e.get("kernel_sources_sha16"),
+                     "measured_in_this_run": False}
+            if e.get("kernel_sources_sha16") != sha:
+                about["status"] = f"stale: the record is for other kernel sources (now {sha}); profile again"
+                return None, about
             fetch = e["fetch_size_kib"] * e["copy_bytes"] / 1024.0 / e["copy_fetch_size_kib"]
             write = e["write_size_kib"] * e["copy_bytes"] / 1024.0 / e["copy_write_size_kib"]
-            return (fetch + write) * 1024.0
-    return None
+            return (fetch + write) * 1024.0, about
+    return None, {"status": "no record for this kernel and workload"}
 
 
 def cpu_baseline(cfg, table, stream, sols, n_threads):
@@ -311,7 +332,7 @@ def main():
         ops_note = "achieved counts 2*stages+2 per check_slo call (+1 per head deadline) and 2*stages+1 per committed " \
                    "batch of the reference loop, counted by the oracle on the CPU sample and scaled to the batch"
 
-    traffic = measured_traffic(kernel, workload) if args.flags == "scores" else None
+    traffic, traffic_record = measured_traffic(kernel, workload) if args.flags == "scores" else (None, {"status": "not recorded for this output level"})
 
     hbm_bytes = info["stream_bytes"] + info["table_bytes"] + 12 * lanes
     # dispatched requests = evaluations whose model has a replica: every one costs 3 operations beyond clocks
@@ -358,6 +379,7 @@ def main():
             "ops_per_launch": total_ops,
             "ops_per_eval": None if total_ops is None else total_ops / evals_per_step,
             "traffic": traffic,
+            "traffic_record": traffic_record,
             "note": "fp64 add/max/compare only (no FMA): peak = published 78.6 TFLOP/s / 2; " + ops_note,
             # the two other ceilings of this path, for the record: compulsory HBM bytes (streams once per
             # wavefront group + tables + results) and algorithmic LDS bytes (8 per clock read or written:

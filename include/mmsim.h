@@ -75,6 +75,49 @@ const char *mmsim_last_error(void);
 int mmsim_ctx_create(int device, mmsim_ctx **out);
 void mmsim_ctx_destroy(mmsim_ctx *ctx);
 
+/*
+ * Tuning options of the launch plan.  The reference keeps its simulator knobs
+ * as module constants (alpa_serve/simulator/controller.py:432, 517, 575, 644;
+ * alpa_serve/util.py:11-13); here they are explicit, defaulted parameters.
+ * Fill the struct with mmsim_options_default() and change what is needed:
+ * -1 (switches) or 0 (numbers) means "let the library decide".  No option
+ * changes a result; they move work between kernels, wavefronts and memories,
+ * and exist for measurements and for tests that must reach every code path.
+ */
+typedef struct {
+    int32_t struct_size;          /* sizeof(mmsim_options), set by mmsim_options_default                      */
+    int32_t request_loop;         /* plain simulator: 1 = loop over runs of equal models (scheduled launch),
+                                     0 = chunks of four requests; -1: runs when at least four in five requests
+                                     of the batch's streams repeat the model of the request before            */
+    int32_t waves_per_cu;         /* 1..8: most wavefronts per workgroup of the plain simulator; 0: as many as fit */
+    int32_t counts_in_lds;        /* counts of the plain simulator: 1 = counters in LDS, 0 = in registers and
+                                     global rows; -1: LDS when that does not cost a CU wavefronts              */
+    int32_t tile_order_by_slots;  /* loop over runs: 0 = tiles composed by pipeline depth only; -1 / 1: by clock
+                                     slots as well                                                              */
+    int32_t sched_groups;         /* workgroups of the scheduled launch; 0: one per CU                          */
+    int32_t segment_requests;     /* requests per turn of an item in the scheduled launch; 0: 16384             */
+    int32_t sched_spin_limit;     /* looks in a row after which a wavefront that finds only busy items leaves;
+                                     -1: 20000                                                                  */
+    int32_t skip_ahead;           /* loop over runs: 0 = simulate every request; -1 / 1: requests that every lane
+                                     of a wavefront must reject are not simulated                              */
+    int32_t xcd_map;              /* chunked loop: 0 = seeds innermost in the workgroup numbering; -1 / 1: all
+                                     seeds of a tile group on one XCD                                           */
+    int32_t batching_lanes;       /* batching simulator: 8, 16, 32 or 64 simulations per wavefront; 0: the widest
+                                     that still gives a CU eight wavefronts                                    */
+    int32_t batching_event_slots; /* batching simulator: idle-event slots per simulation (a multiple of eight);
+                                     0: from the group count.  Too few makes a simulation stop with
+                                     MMSIM_E_OVERFLOW                                                           */
+    int32_t batching_lds_tables;  /* batching simulator: bit 0 latency table, bit 1 models of each group may be
+                                     copied to LDS; -1: both, subject to fit                                    */
+    int32_t reserved;
+    int64_t stats_scratch_bytes;  /* scratch of one launch of mmsim_batch_model_stats; 0: 1 GiB                 */
+} mmsim_options;
+void mmsim_options_default(mmsim_options *options);
+/* Options for every batch the context makes from now on without options of its own (mmsim_batch_create,
+ * mmsim_eval_batch, mmsim_eval_pairs, mmsim_eval_batch_static, the single-placement calls); NULL restores the
+ * defaults. */
+int mmsim_ctx_set_options(mmsim_ctx *ctx, const mmsim_options *options);
+
 typedef struct {
     char name[128];
     char arch[64];
@@ -90,6 +133,11 @@ int mmsim_ctx_device_info(mmsim_ctx *ctx, mmsim_device_info *out);
  *   tstamps   [R] arrival times in the order the requests are to be processed
  *   model_ids [R] model index in [0, M) or negative for "not registered"
  *   slos      [R] float32 seconds; +inf = never dropped, NaN = always dropped
+ * Streams are generated on the host by design: the reference draws them from
+ * numpy's legacy Mersenne-Twister / rejection-sampled gamma stream
+ * (alpa_serve/simulator/workload.py:135-155), which is sequential per model
+ * and goes through the host's libm; a device generator could not reproduce
+ * those arrivals bit for bit, and a stream is made once per search.
  */
 int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M,
                           const double *tstamps, const int32_t *model_ids,
@@ -158,10 +206,16 @@ typedef struct {
 } mmsim_result;
 
 /* Packs the placements, uploads them and allocates device result buffers.  The
- * batch copies what it needs of the workloads: they may be destroyed before it. */
+ * batch copies what it needs of the workloads for mmsim_batch_run / _fetch:
+ * they may be destroyed before it (mmsim_batch_model_stats is the exception,
+ * see there). */
 int mmsim_batch_create(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
                        const mmsim_tables *tables, const mmsim_placements *placements,
                        uint32_t flags, mmsim_batch **out);
+/* The same with options for this batch only (NULL: the context's). */
+int mmsim_batch_create_ex(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                          const mmsim_tables *tables, const mmsim_placements *placements,
+                          uint32_t flags, const mmsim_options *options, mmsim_batch **out);
 /* Enqueues the simulation kernels on the context's stream (asynchronous). */
 int mmsim_batch_run(mmsim_batch *batch);
 /* Waits for the last run.  kernel_ms (optional) receives the time between HIP
@@ -193,9 +247,12 @@ int mmsim_batch_fetch(mmsim_batch *batch, mmsim_result *out);
  * the mean, not of itself -- in numpy as well.
  *
  * The batch must have been created with MMSIM_WANT_PER_REQUEST and run;
- * `workloads` are the n_streams streams it was created with (their per-model
- * request lists are read; the batch keeps no copy of them).  Call
- * mmsim_batch_fetch as well to learn of simulations that failed. */
+ * `workloads` are the n_streams workload objects it was created with, in the
+ * same order and not destroyed in between (their per-model request lists are
+ * read; the batch keeps no copy of them, and it checks that these are the
+ * objects it was made from: any other stream, even one of the same length, is
+ * refused with MMSIM_E_INVALID).  Call mmsim_batch_fetch as well to learn of
+ * simulations that failed. */
 typedef struct {
     int32_t *model_num_requests; /* requests of the model inside the window     */
     int32_t *model_num_good;     /* accepted ones among them                     */
@@ -225,10 +282,12 @@ int mmsim_eval_pairs(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
                      const int32_t *stream_of, uint32_t flags, mmsim_result *out);
 
 /*
- * mmsim_eval_batch without any device allocation.  It has no counterpart in
- * the reference; it is for callers that cannot allocate device memory: code
- * under HIP graph capture, tight search or serving loops, harnesses that
- * forbid hipMalloc.  Same arguments, results and error codes as
+ * mmsim_eval_batch without any device allocation or free.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device
+ * memory: tight search or serving loops, harnesses that forbid hipMalloc.
+ * The call is synchronous and runs on the context's own stream (it copies,
+ * clears and waits like mmsim_eval_batch, so it cannot itself be recorded
+ * into a HIP graph).  Same arguments, results and error codes as
  * mmsim_eval_batch, bit for bit, but every device table and result buffer of
  * the batch lives in a static device array of MMSIM_STATIC_SCRATCH_BYTES that
  * the library holds on each GPU it runs on until the process ends: no

@@ -49,6 +49,15 @@ class Result(C.Structure):
                 ("finish", _p_f64), ("good", _p_u8), ("status", _p_i32), ("fp_ops", _p_i64)]
 
 
+class Options(C.Structure):
+    """mmsim_options: -1 (switches) / 0 (numbers) leave the choice to the library."""
+    _fields_ = [("struct_size", C.c_int32), ("request_loop", C.c_int32), ("waves_per_cu", C.c_int32),
+                ("counts_in_lds", C.c_int32), ("tile_order_by_slots", C.c_int32), ("sched_groups", C.c_int32),
+                ("segment_requests", C.c_int32), ("sched_spin_limit", C.c_int32), ("skip_ahead", C.c_int32),
+                ("xcd_map", C.c_int32), ("batching_lanes", C.c_int32), ("batching_event_slots", C.c_int32),
+                ("batching_lds_tables", C.c_int32), ("reserved", C.c_int32), ("stats_scratch_bytes", C.c_int64)]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
                 ("clock_khz", C.c_int32), ("lds_bytes_per_block", C.c_int32), ("hbm_bytes", C.c_int64)]
@@ -76,6 +85,11 @@ SIGNATURES = {
     "mmsim_ctx_create": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
     "mmsim_ctx_destroy": (None, [C.c_void_p]),
     "mmsim_ctx_device_info": (C.c_int, [C.c_void_p, C.POINTER(DeviceInfo)]),
+    "mmsim_options_default": (None, [C.POINTER(Options)]),
+    "mmsim_ctx_set_options": (C.c_int, [C.c_void_p, C.POINTER(Options)]),
+    "mmsim_batch_create_ex": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
+                                         C.POINTER(Placements), C.c_uint32, C.POINTER(Options),
+                                         C.POINTER(C.c_void_p)]),
     "mmsim_workload_create": (C.c_int, [C.c_void_p, C.c_int64, C.c_int32, _p_f64, _p_i32, _p_f32,
                                          C.POINTER(C.c_void_p)]),
     "mmsim_workload_destroy": (None, [C.c_void_p]),

@@ -27,7 +27,7 @@ FLAGS = [
 ]
 
 
-# One wavefront per SIMD is the rule for the plain simulator's kernel (LDS-bound occupancy), so
+# The plain simulator runs one or two wavefronts per SIMD (LDS decides how many), so
 # instruction-level parallelism inside a wavefront is what hides latency: schedule for it (measured
 # -7 % kernel time).  The batching kernel is built with the default scheduler (this one fails on it).
 # Blocks that are only reached by a branch start on a 64-byte boundary: a taken branch costs a lone wavefront

@@ -107,10 +107,14 @@ struct mmsim_ctx {
     int max_lds = 0;
     unsigned char *scratch = nullptr;     // this device's copy of the static scratch (mmsim_eval_batch_static)
     hipEvent_t ev_static[2] = {};         // timing events of batches that live in the static scratch
+    mmsim_options opt{};                  // what batches made without options of their own use (mmsim_ctx_set_options)
 };
+
+std::atomic<uint64_t> g_next_workload_id{1};
 
 struct mmsim_workload {
     mmsim_ctx *ctx = nullptr;
+    uint64_t id = 0;  // unique per mmsim_workload_create: a batch remembers which streams it was made from
     int64_t R = 0;
     int32_t M = 0;
     DevBuf<Req> reqs;
@@ -143,6 +147,7 @@ struct mmsim_batch {
     size_t lds_bytes = 0;
     int64_t Rmax = 0, Rtotal = 0;
     std::vector<int64_t> wl_R;                           // [n_seeds] stream lengths
+    std::vector<uint64_t> wl_id;                         // [n_seeds] ids of the workloads the batch was made from
     std::vector<std::vector<int32_t>> wl_model_requests;  // [n_seeds][M] requests per model of each stream
     std::vector<int32_t> pos;  // pos[placement] = tile * 64 + lane it is simulated on
     // Paired batch (mmsim_eval_pairs): placement p is simulated on stream stream_of[p] only; a tile holds
@@ -190,6 +195,7 @@ struct mmsim_batch {
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     bool own_events = true;  // false: the context's events (batch in the static scratch)
     bool ran = false;
+    mmsim_options opt{};     // the options the batch was built with
 
     ~mmsim_batch() {
         if (own_events && ev_start) (void)hipEventDestroy(ev_start);
@@ -214,7 +220,23 @@ int check_tables(const mmsim_tables *t) {
     return MMSIM_OK;
 }
 
-// group -> models CSR of the C ABI into ordered per-(placement, model) replica lists
+int check_options(const mmsim_options *o) {
+    if (!o) return MMSIM_OK;
+    if (o->struct_size != (int32_t)sizeof(mmsim_options))
+        return fail(MMSIM_E_INVALID, "options: struct_size is not sizeof(mmsim_options); start from mmsim_options_default");
+    auto tri = [](int32_t v) { return v >= -1 && v <= 1; };
+    if (!tri(o->request_loop) || !tri(o->counts_in_lds) || !tri(o->tile_order_by_slots) || !tri(o->skip_ahead) || !tri(o->xcd_map))
+        return fail(MMSIM_E_INVALID, "options: a -1 / 0 / 1 switch has another value");
+    if (o->waves_per_cu < 0 || o->waves_per_cu > kMaxWavesPerBlock) return fail(MMSIM_E_INVALID, "options: waves_per_cu outside 0..8");
+    if (o->sched_groups < 0 || o->segment_requests < 0 || o->sched_spin_limit < -1 || o->batching_event_slots < 0 ||
+        o->stats_scratch_bytes < 0)
+        return fail(MMSIM_E_INVALID, "options: negative value");
+    if (o->batching_lanes != 0 && o->batching_lanes != 8 && o->batching_lanes != 16 && o->batching_lanes != 32 && o->batching_lanes != 64)
+        return fail(MMSIM_E_INVALID, "options: batching_lanes must be 0, 8, 16, 32 or 64");
+    if (o->batching_lds_tables < -1 || o->batching_lds_tables > 3) return fail(MMSIM_E_INVALID, "options: batching_lds_tables outside -1..3");
+    return MMSIM_OK;
+}
+
 // Runs fn(lo, hi) on slices of [0, n) on up to 16 host threads (one slice per thread; the caller's
 // slices write disjoint memory).  Small ranges run on the calling thread.
 template <class F>
@@ -232,6 +254,7 @@ void parallel_slices(int64_t n, int64_t min_per_thread, F &&fn) {
     for (std::thread &th : pool) th.join();
 }
 
+// group -> models CSR of the C ABI into ordered per-(placement, model) replica lists
 int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLists *out) {
     if (!p || !p->num_groups || !p->group_cfg || !p->gm_off) return fail(MMSIM_E_INVALID, "placements: null pointer");
     if (p->B < 1 || p->Gmax < 1) return fail(MMSIM_E_INVALID, "placements: B and Gmax must be >= 1");
@@ -271,7 +294,9 @@ int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLi
 
 // Builds every device table of a batch from replica lists and launches nothing.
 int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seeds, const mmsim_tables *t,
-                const RepLists &rl, uint32_t flags, mmsim_batch **out, const int32_t *stream_of = nullptr) {
+                const RepLists &rl, uint32_t flags, mmsim_batch **out, const int32_t *stream_of = nullptr,
+                const mmsim_options *options = nullptr) {
+    const mmsim_options &o = options ? *options : ctx->opt;
     // MMSIM_TIMING=1 prints the host time of each phase of the packing (diagnostics)
     const bool timing = std::getenv("MMSIM_TIMING") != nullptr;
     auto t_last = std::chrono::steady_clock::now();
@@ -305,6 +330,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     std::unique_ptr<mmsim_batch> b(new (std::nothrow) mmsim_batch);
     if (!b) return fail(MMSIM_E_NOMEM, "host allocation failed");
     b->ctx = ctx;
+    b->opt = o;
     b->flags = flags;
     b->n_seeds = n_seeds;
     b->B = B;
@@ -312,6 +338,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     b->Gmax = Gmax;
     for (int s = 0; s < n_seeds; ++s) {  // copied: the batch does not depend on the workloads outliving it
         b->wl_R.push_back(wls[s]->R);
+        b->wl_id.push_back(wls[s]->id);
         b->wl_model_requests.push_back(wls[s]->model_num_requests);
     }
     b->paired = stream_of != nullptr;
@@ -384,7 +411,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             tot += wls[s]->R;
         }
         runs = 5 * rep > 4 * tot;  // four in five (measured: at three in four the chunked loop is still ahead)
-        if (const char *env = std::getenv("MMSIM_RUNS")) runs = std::atoi(env) != 0;  // tuning knob
+        if (o.request_loop >= 0) runs = o.request_loop != 0;
     }
 
     phase("latency table, loop choice");
@@ -398,14 +425,14 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     int blanes = kWave;  // batching simulator: lanes of a wavefront that simulate
     // Wavefronts per workgroup: no more than it takes to give every CU its share of the
     // batch (a small batch is spread over the CUs, one wavefront per workgroup), and
-    // no more than fit in LDS.  MMSIM_WAVES_PER_CU (1..8) sets the number instead (tuning knob).
+    // no more than fit in LDS.  Option waves_per_cu (1..8) sets the number instead.
     int wpb_cap = kMaxWavesPerBlock;
     {
         const int64_t waves_total = (int64_t)((B + kWave - 1) / kWave) * b->out_seeds;
         const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
         wpb_cap = (int)std::min<int64_t>(wpb_cap, std::max<int64_t>(1, (waves_total + cus - 1) / cus));
     }
-    if (const char *env = std::getenv("MMSIM_WAVES_PER_CU")) wpb_cap = std::max(1, std::min(kMaxWavesPerBlock, std::atoi(env)));
+    if (o.waves_per_cu > 0) wpb_cap = std::min(kMaxWavesPerBlock, o.waves_per_cu);
     // plain simulator, per wavefront: request block | replica bounds | clocks (one extra row that stays +inf)
     // | slot counters | model counters; the latency table is shared by the workgroup
     size_t model_lds_bytes = 0;  // per-model counters [M][64] in LDS (decided below)
@@ -437,8 +464,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         // 32 KB more per wavefront).  Without LDS the group counts are kept per lane in registers and added to global
         // rows when the lane's group changes, and accepted requests are added to global per-model rows, which a lone
         // wavefront has to wait behind (small batches: about 300 cycles per request).  So the counters go to LDS, both
-        // kinds together, when that does not lower the wavefronts a CU gets.  MMSIM_COUNTS_LDS=0/1 forces the choice
-        // (tuning knob).  With per-request outputs or operation counts (the general kernel) each kind goes to LDS if
+        // kinds together, when that does not lower the wavefronts a CU gets.  Option counts_in_lds = 0 / 1 forces the
+        // choice.  With per-request outputs or operation counts (the general kernel) each kind goes to LDS if
         // it fits at all.
         const size_t room = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail;
         const size_t model_rows = (size_t)M * kWave * sizeof(uint32_t);
@@ -460,7 +487,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             model_lds_bytes = model_rows;
             const size_t with = std::min<size_t>(wpb_cap, room / mixed_wave_bytes(nslots));
             bool in_lds = with >= 1 && with >= without;
-            if (const char *env = std::getenv("MMSIM_COUNTS_LDS")) in_lds = with >= 1 && std::atoi(env) != 0;
+            if (o.counts_in_lds >= 0) in_lds = with >= 1 && o.counts_in_lds != 0;
             if (!in_lds) {
                 group_in_lds = false;
                 model_lds_bytes = 0;
@@ -484,9 +511,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         };
         heap_min = (Gmax + 4 + 7) & ~7;
         heap_pref = std::max(heap_min, std::min(2 * Gmax + 8, Gmax + 16) & ~7);
-        // MMSIM_BATCHING_EVENT_SLOTS fixes the number of event slots per simulation (a multiple of eight; fewer than
+        // Option batching_event_slots fixes the number of event slots per simulation (a multiple of eight; fewer than
         // the simulation needs makes it stop with MMSIM_E_OVERFLOW: used to test that path)
-        if (const char *env = std::getenv("MMSIM_BATCHING_EVENT_SLOTS")) heap_pref = heap_min = std::max(8, std::atoi(env) & ~7);
+        if (o.batching_event_slots > 0) heap_pref = heap_min = std::max(8, o.batching_event_slots & ~7);
         auto size_for = [&](int lanes) {
             for (heap_cap = heap_pref; heap_cap >= heap_min; heap_cap -= 8) {
                 wave_bytes = bytes_for(lanes, heap_cap);
@@ -499,9 +526,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         // simulate, the others only help fetching requests) put more wavefronts on a CU, and that is
         // what hides the latency.  The widest tile that still gives every SIMD two wavefronts is used.
         blanes = kWave;
-        if (const char *env = std::getenv("MMSIM_BATCHING_LANES")) {
-            const int v = std::atoi(env);
-            if (v == 8 || v == 16 || v == 32 || v == 64) blanes = v;
+        if (o.batching_lanes > 0) {
+            blanes = o.batching_lanes;
         } else {
             const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
             for (;;) {
@@ -554,9 +580,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (bad_group) return fail(MMSIM_E_INVALID, "replica list names a group that does not exist");
         // Deepest first: their wavefronts take longest.  The loop over runs sizes a wavefront's LDS region by the
         // clock slots of its own tile, so there placements with similar slot counts share a tile
-        // (MMSIM_TILE_ORDER=0: by expected depth only, tuning knob).
+        // (option tile_order_by_slots = 0: by expected depth only).
         bool by_slots = runs;
-        if (const char *env = std::getenv("MMSIM_TILE_ORDER")) by_slots = runs && std::atoi(env) != 0;
+        if (o.tile_order_by_slots >= 0) by_slots = runs && o.tile_order_by_slots != 0;
         std::vector<int32_t> order(B);
         for (int32_t p = 0; p < B; ++p) order[p] = p;
         std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
@@ -611,7 +637,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         const int64_t n_items = (int64_t)b->waves;
         const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
         int64_t groups = std::min<int64_t>(cus, n_items);
-        if (const char *env = std::getenv("MMSIM_SCHED_GROUPS")) groups = std::max<int64_t>(1, std::min<int64_t>(n_items, std::atoi(env)));  // tuning knob
+        if (o.sched_groups > 0) groups = std::min<int64_t>(n_items, o.sched_groups);
         if (n_items > groups * kMaxGroupItems) return fail(MMSIM_E_UNSUPPORTED, "too many (tile, stream) pairs for one launch; split the batch");
         std::vector<int32_t> tile_bytes(b->tiles);
         for (int32_t t2 = 0; t2 < b->tiles; ++t2) tile_bytes[t2] = (int32_t)mixed_wave_bytes(tile_nslots[t2]);
@@ -639,9 +665,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             }
         }
         int max_regions = kMaxWavesPerBlock;
-        if (const char *env = std::getenv("MMSIM_WAVES_PER_CU")) max_regions = std::max(1, std::min(kMaxWavesPerBlock, std::atoi(env)));
+        if (o.waves_per_cu > 0) max_regions = std::min(kMaxWavesPerBlock, o.waves_per_cu);
         int64_t seg_requests = 16384;
-        if (const char *env = std::getenv("MMSIM_SEGMENT_REQUESTS")) seg_requests = std::max<int64_t>(kWave, std::atoll(env) & ~(int64_t)(kWave - 1));  // tuning knob
+        if (o.segment_requests > 0) seg_requests = std::max<int64_t>(kWave, (int64_t)o.segment_requests & ~(int64_t)(kWave - 1));
         std::vector<int32_t> wg_off(groups + 1, 0), part_off((size_t)groups * kMaxWavesPerBlock, -1), part_bytes((size_t)groups * kMaxWavesPerBlock, 0);
         bool shared = false;  // some workgroup has more items than regions: streams are cut into segments
         size_t lds_used = 0;
@@ -678,7 +704,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 const size_t at = (size_t)wg_off[w] + i;
                 const int64_t Rs = b->wl_R[(size_t)it.seed];
                 const int64_t ns = std::max<int64_t>(1, (Rs + seg_requests - 1) / seg_requests);
-                if (ns > 60000) return fail(MMSIM_E_INVALID, "MMSIM_SEGMENT_REQUESTS is too small for these streams");
+                if (ns > 60000) return fail(MMSIM_E_INVALID, "option segment_requests is too small for these streams");
                 p_tile[at] = it.tile;
                 p_seed[at] = it.seed;
                 p_ns[at] = tile_nslots[it.tile];
@@ -862,9 +888,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         const int wpb_max = kMaxWavesPerBlockBatching;
         const int heap_try_min = std::min(heap_cap, std::max(heap_min, (Gmax + 8 + 7) & ~7));
         int best_w = 0, best_total = 0, best_heap = heap_cap;
-        // MMSIM_BATCHING_LDS_TABLES (bit 0: latency table, bit 1: group lists) fixes which tables may go to LDS
-        int allowed = 3;
-        if (const char *env = std::getenv("MMSIM_BATCHING_LDS_TABLES")) allowed = std::atoi(env) & 3;
+        // option batching_lds_tables (bit 0: latency table, bit 1: group lists) fixes which tables may go to LDS
+        const int allowed = o.batching_lds_tables >= 0 ? (o.batching_lds_tables & 3) : 3;
         for (int hc = heap_cap; hc >= heap_try_min; hc -= 8) {
             const size_t wb = batching_bytes_for(blanes, hc);
             for (int per_cu = 1; per_cu <= 2; ++per_cu)  // workgroups meant to share a CU (each gets that share of LDS)
@@ -1029,7 +1054,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.seg_requests = b->seg_requests;
     a.sched_lds_bytes = (int32_t)sched_bytes;
     a.sched_spin_limit = 20000;  // waits of 127 x 64 cycles: about 70 ms, several segments
-    if (const char *env = std::getenv("MMSIM_SCHED_SPIN_LIMIT")) a.sched_spin_limit = std::max(0, std::atoi(env));  // tuning knob
+    if (o.sched_spin_limit >= 0) a.sched_spin_limit = o.sched_spin_limit;
     a.streams = b->streams.p;
     a.stream_off = b->stream_off.p;
     a.rep32 = reinterpret_cast<const uint4 *>(b->rep32.p);
@@ -1062,9 +1087,8 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     a.slot_cnt = b->slot_cnt.p;
     a.xcd_map = 1;
     a.runs = runs ? 1 : 0;
-    a.skip_ahead = 1;
-    if (const char *env = std::getenv("MMSIM_SKIP_AHEAD")) a.skip_ahead = std::atoi(env) ? 1 : 0;  // tuning knob
-    if (const char *env = std::getenv("MMSIM_XCD_MAP")) a.xcd_map = std::atoi(env) ? 1 : 0;  // tuning knob
+    a.skip_ahead = o.skip_ahead >= 0 ? (o.skip_ahead ? 1 : 0) : 1;
+    if (o.xcd_map >= 0) a.xcd_map = o.xcd_map ? 1 : 0;
     a.finish = b->finish.p;
     a.good = b->good.p;
     a.fp_ops = b->fp_ops.p;
@@ -1123,6 +1147,25 @@ int mmsim_abi_version(void) { return MMSIM_ABI_VERSION; }
 
 const char *mmsim_last_error(void) { return g_last_error.c_str(); }
 
+void mmsim_options_default(mmsim_options *o) {
+    if (!o) return;
+    std::memset(o, 0, sizeof(*o));
+    o->struct_size = (int32_t)sizeof(mmsim_options);
+    o->request_loop = o->counts_in_lds = o->tile_order_by_slots = o->sched_spin_limit = -1;
+    o->skip_ahead = o->xcd_map = o->batching_lds_tables = -1;
+}
+
+int mmsim_ctx_set_options(mmsim_ctx *ctx, const mmsim_options *options) {
+    if (!ctx) return fail(MMSIM_E_INVALID, "ctx_set_options: null context");
+    int rc = check_options(options);
+    if (rc) return rc;
+    if (options)
+        ctx->opt = *options;
+    else
+        mmsim_options_default(&ctx->opt);
+    return MMSIM_OK;
+}
+
 int mmsim_ctx_create(int device, mmsim_ctx **out) {
     if (!out) return fail(MMSIM_E_INVALID, "ctx_create: out is null");
     *out = nullptr;
@@ -1134,6 +1177,7 @@ int mmsim_ctx_create(int device, mmsim_ctx **out) {
     std::unique_ptr<mmsim_ctx> c(new (std::nothrow) mmsim_ctx);
     if (!c) return fail(MMSIM_E_NOMEM, "host allocation failed");
     c->device = device;
+    mmsim_options_default(&c->opt);
     HIP_TRY(hipSetDevice(device));
     HIP_TRY(hipGetDeviceProperties(&c->prop, device));
     if (std::strncmp(c->prop.gcnArchName, "gfx950", 6) != 0)
@@ -1195,6 +1239,7 @@ int mmsim_workload_create(mmsim_ctx *ctx, int64_t R, int32_t M, const double *ts
     std::unique_ptr<mmsim_workload> w(new (std::nothrow) mmsim_workload);
     if (!w) return fail(MMSIM_E_NOMEM, "host allocation failed");
     w->ctx = ctx;
+    w->id = g_next_workload_id.fetch_add(1);
     w->R = R;
     w->M = M;
     w->model_num_requests.assign(M, 0);
@@ -1260,17 +1305,25 @@ void mmsim_workload_destroy(mmsim_workload *wl) {
     delete wl;
 }
 
-int mmsim_batch_create(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
-                       const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
-                       mmsim_batch **out) {
+int mmsim_batch_create_ex(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                          const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
+                          const mmsim_options *options, mmsim_batch **out) {
     if (!ctx || !out) return fail(MMSIM_E_INVALID, "batch_create: null pointer");
     *out = nullptr;
     int rc = check_tables(tables);
     if (rc) return rc;
+    rc = check_options(options);
+    if (rc) return rc;
     RepLists rl;
     rc = lists_from_placements(placements, tables->M, tables->C, &rl);
     if (rc) return rc;
-    return build_batch(ctx, workloads, n_seeds, tables, rl, flags, out);
+    return build_batch(ctx, workloads, n_seeds, tables, rl, flags, out, nullptr, options);
+}
+
+int mmsim_batch_create(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                       const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
+                       mmsim_batch **out) {
+    return mmsim_batch_create_ex(ctx, workloads, n_seeds, tables, placements, flags, nullptr, out);
 }
 
 int mmsim_batch_run(mmsim_batch *b) {
@@ -1443,8 +1496,9 @@ int mmsim_batch_model_stats(mmsim_batch *b, const mmsim_workload *const *workloa
     std::vector<int64_t> mqo((size_t)n_streams * (M + 1)), lo((size_t)n_streams), hi((size_t)n_streams);
     for (int s = 0; s < n_streams; ++s) {
         const mmsim_workload *w = workloads[s];
-        if (!w || w->ctx != b->ctx || w->M != M || w->R != b->wl_R[(size_t)s])
-            return fail(MMSIM_E_INVALID, "batch_model_stats: pass the request streams the batch was created with");
+        if (!w || w->ctx != b->ctx || w->id != b->wl_id[(size_t)s] || w->M != M || w->R != b->wl_R[(size_t)s])
+            return fail(MMSIM_E_INVALID, "batch_model_stats: pass the request streams the batch was created with "
+                                         "(the same workload objects, in the same order, still alive)");
         if (skip[s] < 0) return fail(MMSIM_E_INVALID, "batch_model_stats: negative skip");
         mq[(size_t)s] = w->mq.p;
         for (int32_t m = 0; m <= M; ++m) mqo[(size_t)s * (M + 1) + m] = w->mq_off[(size_t)m];
@@ -1458,8 +1512,7 @@ int mmsim_batch_model_stats(mmsim_batch *b, const mmsim_workload *const *workloa
     const int64_t n_sims = (int64_t)b->out_seeds * B;
     int64_t pitch = 1;
     for (int s = 0; s < n_streams; ++s) pitch = std::max<int64_t>(pitch, workloads[s]->mq_off[(size_t)M]);
-    int64_t scratch_bytes = kStatsScratchBytes;
-    if (const char *env = std::getenv("MMSIM_STATS_SCRATCH_BYTES")) scratch_bytes = std::max<int64_t>(0, std::atoll(env));  // tuning knob
+    const int64_t scratch_bytes = b->opt.stats_scratch_bytes > 0 ? b->opt.stats_scratch_bytes : kStatsScratchBytes;
     const int64_t rows = std::max<int64_t>(1, std::min<int64_t>(n_sims, scratch_bytes / (pitch * (int64_t)sizeof(uint64_t))));
     std::vector<int32_t> sim_stream((size_t)n_sims);
     std::vector<int64_t> sim_base((size_t)n_sims);

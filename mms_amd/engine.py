@@ -10,6 +10,7 @@ placement is reduced to "which config does each group use, which models does
 it host".
 """
 import ctypes as C
+from contextlib import contextmanager
 from itertools import chain
 from typing import List, Sequence
 
@@ -42,6 +43,34 @@ class Engine:
         return {"name": info.name.decode(), "arch": info.arch.decode(),
                 "compute_units": info.compute_units, "clock_khz": info.clock_khz,
                 "lds_bytes_per_block": info.lds_bytes_per_block, "hbm_bytes": info.hbm_bytes}
+
+    def make_options(self, **fields):
+        """An ``mmsim_options`` with the library's defaults and ``fields`` changed."""
+        opt = _lib.Options()
+        self.lib.mmsim_options_default(C.byref(opt))
+        names = {f[0] for f in _lib.Options._fields_} - {"struct_size", "reserved"}
+        for k, v in fields.items():
+            if k not in names:
+                raise TypeError(f"mmsim_options has no field {k!r}")
+            setattr(opt, k, int(v))
+        return opt
+
+    def set_options(self, **fields):
+        """Options of every batch this context makes from now on (``mmsim_ctx_set_options``);
+        without arguments: the defaults."""
+        opt = self.make_options(**fields)
+        _lib.check(self.lib.mmsim_ctx_set_options(self._h, C.byref(opt)))
+        self._options = dict(fields)
+
+    @contextmanager
+    def options(self, **fields):
+        """``with engine.options(request_loop=1): ...`` -- the fields on top of what is set now, put back afterwards."""
+        before = dict(getattr(self, "_options", {}))
+        self.set_options(**{**before, **fields})
+        try:
+            yield self
+        finally:
+            self.set_options(**before)
 
     def close(self):
         if self._h:
@@ -185,13 +214,31 @@ def _result_arrays(flags, n_seeds, B, M, Gmax, Rmax):
     return out, r
 
 
-def _shape_results(out, n_seeds, B):
+def check_status(status, what="simulation"):
+    """Raises ``MmsimError`` when a simulation's ``status`` is not 0: such a simulation ran out of idle-event
+    slots (``E_OVERFLOW``) or met an input the batching simulator does not support (``E_UNSUPPORTED``), and its
+    counts and per-request outputs are partly unwritten."""
+    status = np.asarray(status)
+    bad = np.flatnonzero(status.reshape(-1) != 0)
+    if bad.size:
+        code = int(status.reshape(-1)[bad[0]])
+        names = ", ".join(str(tuple(int(x) for x in np.unravel_index(i, status.shape))) for i in bad[:8])
+        why = {_lib.E_OVERFLOW: "ran out of idle-event slots",
+               _lib.E_UNSUPPORTED: "met an input the batching simulator does not support (all replica clocks infinite)"
+               }.get(code, "failed")
+        raise _lib.MmsimError(code, f"{bad.size} {what}(s) {why}; their results are invalid: {names}"
+                                    f"{' ...' if bad.size > 8 else ''} (pass allow_failed=True to read status[] instead)")
+
+
+def _shape_results(out, n_seeds, B, allow_failed=False):
     L = n_seeds * B
     if "good" in out:
         out["good"] = out["good"].astype(bool)
     for k in list(out):
         if out[k].ndim >= 1 and out[k].shape[0] == L:
             out[k] = out[k].reshape((n_seeds, B) + out[k].shape[1:])
+    if not allow_failed:
+        check_status(out["status"], "simulation (seed, placement)")
     return out
 
 
@@ -217,7 +264,7 @@ def _abi_inputs(workloads, table, packed, fixed_overhead):
 
 
 def eval_batch(engine: "Engine", workloads, table: "LatencyTable", packed, flags: int = 0,
-               fixed_overhead: float = FIXED_OVERHEAD, static: bool = False):
+               fixed_overhead: float = FIXED_OVERHEAD, static: bool = False, allow_failed: bool = False):
     """One call of ``mmsim_eval_batch`` (create + run + sync + fetch + destroy inside the library), or of
     ``mmsim_eval_batch_static`` -- the same without any device allocation, for batches that fit the
     library's static device scratch.  Result arrays are [n_seeds][B][...]."""
@@ -228,13 +275,14 @@ def eval_batch(engine: "Engine", workloads, table: "LatencyTable", packed, flags
     fn = engine.lib.mmsim_eval_batch_static if static else engine.lib.mmsim_eval_batch
     _lib.check(fn(engine._h, wl, n_seeds, C.byref(t), C.byref(p), int(flags), C.byref(r)))
     del keep
-    return _shape_results(out, n_seeds, B)
+    return _shape_results(out, n_seeds, B, allow_failed)
 
 
 def eval_pairs(engine: "Engine", workloads, table: "LatencyTable", packed, stream_of, flags: int = 0,
-               fixed_overhead: float = FIXED_OVERHEAD):
+               fixed_overhead: float = FIXED_OVERHEAD, allow_failed: bool = False):
     """One call of ``mmsim_eval_pairs``: placement b on ``workloads[stream_of[b]]`` only.
-    Result arrays are [B][...]."""
+    Result arrays are [B][...].  A simulation that failed (``status[b] != 0``) raises unless
+    ``allow_failed``."""
     workloads = list(workloads)
     t, p, wl, keep = _abi_inputs(workloads, table, packed, fixed_overhead)
     so = _lib.carray(stream_of, np.int32)
@@ -243,6 +291,8 @@ def eval_pairs(engine: "Engine", workloads, table: "LatencyTable", packed, strea
     _lib.check(engine.lib.mmsim_eval_pairs(engine._h, wl, len(workloads), C.byref(t), C.byref(p),
                                            _lib.ptr(so, C.c_int32), int(flags), C.byref(r)))
     del keep
+    if not allow_failed:
+        check_status(out["status"])
     if "good" in out:
         out["good"] = out["good"].astype(bool)
     return out
@@ -252,7 +302,8 @@ class Batch:
     """Device-resident batch of placements x seeds; run() may be repeated."""
 
     def __init__(self, engine: Engine, workloads: Sequence[DeviceWorkload], table: LatencyTable,
-                 packed, flags: int, fixed_overhead: float = FIXED_OVERHEAD):
+                 packed, flags: int, fixed_overhead: float = FIXED_OVERHEAD, options=None):
+        """``options``: dict of ``mmsim_options`` fields for this batch only (default: the engine's)."""
         self.engine = engine
         self.workloads = list(workloads)
         self.flags = int(flags)
@@ -261,8 +312,9 @@ class Batch:
         self.n_seeds = len(self.workloads)
         self.Rmax = max(w.R for w in self.workloads)
         self._h = C.c_void_p()
-        _lib.check(engine.lib.mmsim_batch_create(engine._h, wl, self.n_seeds, C.byref(t), C.byref(p),
-                                                 self.flags, C.byref(self._h)))
+        opt = C.byref(engine.make_options(**options)) if options is not None else None
+        _lib.check(engine.lib.mmsim_batch_create_ex(engine._h, wl, self.n_seeds, C.byref(t), C.byref(p),
+                                                    self.flags, opt, C.byref(self._h)))
 
     def run(self):
         _lib.check(self.engine.lib.mmsim_batch_run(self._h))
@@ -284,13 +336,15 @@ class Batch:
         _lib.check(self.engine.lib.mmsim_batch_kernel_name(self._h, buf, len(buf)))
         return buf.value.decode()
 
-    def fetch(self, per_request=True):
+    def fetch(self, per_request=True, allow_failed=False):
         """Results of the last run.  ``per_request=False`` leaves finish / good of a
-        ``WANT_PER_REQUEST`` batch on the device (for ``model_stats``)."""
+        ``WANT_PER_REQUEST`` batch on the device (for ``model_stats``).  A simulation that
+        failed (``status != 0``: batching simulator only) raises ``MmsimError`` naming it,
+        unless ``allow_failed``, in which case the caller reads ``out["status"]``."""
         flags = self.flags if per_request else self.flags & ~_lib.WANT_PER_REQUEST
         out, r = _result_arrays(flags, self.n_seeds, self.B, self.M, self.Gmax, self.Rmax)
         _lib.check(self.engine.lib.mmsim_batch_fetch(self._h, C.byref(r)))
-        return _shape_results(out, self.n_seeds, self.B)
+        return _shape_results(out, self.n_seeds, self.B, allow_failed)
 
     def model_stats(self, skip):
         """Per (simulation, model) statistics of the last run's per-request outputs, computed on

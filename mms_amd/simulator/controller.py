@@ -156,6 +156,10 @@ def replacement_cuts(placement, arrivals):
     return list(zip(cuts[:-1], cuts[1:]))
 
 
+# Device copies of arrival slices a caller-provided cache of simulate_replacements may hold.
+SEGMENT_CACHE_ENTRIES = 64
+
+
 def simulate_replacements(sols, model_names, prof_ress, model_ids, slos, arrivals, flags=0,
                           enable_batching=False, table=None, workload_cache=None):
     """All segments of all ``ModelPlacementWithReplacement`` in ``sols`` as lanes of ONE GPU launch
@@ -166,6 +170,11 @@ def simulate_replacements(sols, model_names, prof_ress, model_ids, slos, arrival
     ``model_num_requests`` / ``model_num_good`` / ``group_num_requests`` / ``group_num_good`` summed
     over its segments (:385-391; the group axis is as wide as the candidate's widest placement), and
     with ``WANT_PER_REQUEST`` ``finish`` / ``good`` concatenated (:381-383).
+
+    ``workload_cache``: a dict that keeps the device copies of the arrival slices between calls (keyed by
+    slice; the oldest are closed beyond ``SEGMENT_CACHE_ENTRIES``).  Without one the copies made for this call
+    are closed before it returns.  A segment whose simulation failed (batching simulator: ``status != 0``)
+    raises ``MmsimError``.
     """
     eng = _engine.Engine.default()
     arrivals = np.asarray(arrivals, dtype=np.float64)
@@ -175,18 +184,29 @@ def simulate_replacements(sols, model_names, prof_ress, model_ids, slos, arrival
         flags |= _lib.BATCHING
     cache = {} if workload_cache is None else workload_cache
     streams, stream_index, lanes, stream_of, owner = [], {}, [], [], []
-    for n, sol in enumerate(sols):
-        for seg, (lo, hi) in enumerate(replacement_cuts(sol, arrivals)):
-            if (lo, hi) not in stream_index:
-                if (lo, hi) not in cache:
-                    cache[(lo, hi)] = _engine.DeviceWorkload(eng, arrivals[lo:hi], model_ids[lo:hi], slos[lo:hi],
-                                                             len(model_names))
-                stream_index[(lo, hi)] = len(streams)
-                streams.append(cache[(lo, hi)])
-            lanes.append(sol.placements[seg])
-            stream_of.append(stream_index[(lo, hi)])
-            owner.append((n, lo, hi))
-    out = _engine.eval_pairs(eng, streams, table, _engine.pack_placements(lanes, table), stream_of, flags)
+    try:
+        for n, sol in enumerate(sols):
+            for seg, (lo, hi) in enumerate(replacement_cuts(sol, arrivals)):
+                if (lo, hi) not in stream_index:
+                    if (lo, hi) in cache:
+                        cache[(lo, hi)] = cache.pop((lo, hi))      # most recently used last
+                    else:
+                        cache[(lo, hi)] = _engine.DeviceWorkload(eng, arrivals[lo:hi], model_ids[lo:hi],
+                                                                 slos[lo:hi], len(model_names))
+                    stream_index[(lo, hi)] = len(streams)
+                    streams.append(cache[(lo, hi)])
+                lanes.append(sol.placements[seg])
+                stream_of.append(stream_index[(lo, hi)])
+                owner.append((n, lo, hi))
+        out = _engine.eval_pairs(eng, streams, table, _engine.pack_placements(lanes, table), stream_of, flags)
+    finally:
+        if workload_cache is None:
+            for w in cache.values():
+                w.close()
+        else:                       # keep the slices used last, close the device copies of the others
+            for key in list(cache)[:max(0, len(cache) - max(SEGMENT_CACHE_ENTRIES, len(stream_index)))]:
+                if key not in stream_index:
+                    cache.pop(key).close()
     results = [None] * len(sols)
     for n, sol in enumerate(sols):
         mine = [k for k, o in enumerate(owner) if o[0] == n]

@@ -77,30 +77,44 @@ def test_simulate_one_case_statistics_equal_the_reference(c):
     assert [[s.name, int(s.num_requests), float(s.goodput), float(s.latency_p99)] for s in stats.per_model_stats] == c["per_model"]
 
 
-def test_evaluator_with_the_event_driven_method_and_the_approximation_agree_roughly():
+@pytest.mark.parametrize("load", ["light", "overloaded"])
+def test_evaluator_with_the_event_driven_method_and_the_approximation_agree_roughly(backend, load):
     """PlacementEvaluator(method != "fast_simulator") goes through simulate_one_case (base_policy.py:172-224 of the
     reference).  The two simulators model different overheads, so they only agree roughly -- which is the use of the
-    slow one: a fidelity check of the fast one."""
-    import oracle_backend
-    mp = pytest.MonkeyPatch()
-    try:
-        oracle_backend.install(mp)
-        model_datas = [ModelData(f"m{i}", 1.0, 4, 1, load_test_prof_result("test-2GB-100ms")) for i in range(3)]
-        cluster_env = ClusterEnv(4, 64 * GB)
-        sol = ModelPlacement([ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 2)], [[0, 1, 2], [0, 1, 2]])
-        ws = [GammaProcess(md.rate, md.cv).generate_workload(md.name, 0, 60, slo=md.slo, seed=i)
-              for i, md in enumerate(model_datas)]
-        wl = Workload.merge(*ws)
-        np.random.seed(3)
-        slow = PlacementEvaluator(model_datas, cluster_env, wl, "simulator", False)
-        fast = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
-        g_slow, per_model, groups, stats = slow.get_stats([sol])[0]
-        g_fast = fast.get_stats([sol])[0][0]
-        assert sum(groups) == len(wl) and len(per_model) == 3
-        assert abs(g_slow - g_fast) < 0.05
-        assert abs(slow.get_scores([sol])[0] - fast.get_scores([sol])[0]) < 0.05
-    finally:
-        mp.undo()
+    slow one: a fidelity check of the fast one.  Runs with the oracle standing in for the library and (marked gpu)
+    with the fast path on the GPU; ``overloaded`` is a case in which both simulators drop a good part of the requests
+    (the reference records 0.016 as the largest gap between its simulator and a real cluster; the two simulators are
+    allowed 0.05 of each other here)."""
+    rate, slo = (4, 1.0) if load == "light" else (14, 0.6)
+    model_datas = [ModelData(f"m{i}", slo, rate, 2 if load == "overloaded" else 1,
+                             load_test_prof_result("test-2GB-100ms")) for i in range(3)]
+    cluster_env = ClusterEnv(4, 64 * GB)
+    sols = [ModelPlacement([ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 2)], [[0, 1, 2], [0, 1, 2]]),
+            ModelPlacement([ParallelConfig(1, 1, 1)] * 4, [[0, 1], [1, 2], [0, 2], [0, 1, 2]]),
+            ModelPlacement([ParallelConfig(1, 1, 4)], [[0, 1, 2]])]
+    ws = [GammaProcess(md.rate, md.cv).generate_workload(md.name, 0, 60, slo=md.slo, seed=i)
+          for i, md in enumerate(model_datas)]
+    wl = Workload.merge(*ws)
+    np.random.seed(3)
+    slow = PlacementEvaluator(model_datas, cluster_env, wl, "simulator", False)
+    fast = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+    slow_stats, fast_stats = slow.get_stats(sols), fast.get_stats(sols)
+    slow_scores, fast_scores = slow.get_scores(sols), fast.get_scores(sols)
+    for k, sol in enumerate(sols):
+        g_slow, per_model, groups, stats = slow_stats[k]
+        g_fast, per_model_fast, groups_fast, _ = fast_stats[k]
+        assert sum(groups) == len(wl) == sum(groups_fast) and len(per_model) == 3
+        assert abs(g_slow - g_fast) < 0.05, (k, g_slow, g_fast)
+        assert abs(slow_scores[k] - fast_scores[k]) < 0.05
+        assert np.allclose(per_model, per_model_fast, atol=0.08)
+        if load == "overloaded":
+            assert 0.2 < g_fast < 0.97 and 0.2 < g_slow < 0.97     # both drop requests
+        else:
+            assert g_fast > 0.97
+    # both rank the placements alike where they differ by more than the simulators do
+    order_fast = np.argsort(fast_scores)
+    if fast_scores[order_fast[-1]] - fast_scores[order_fast[0]] > 0.1:
+        assert slow_scores[order_fast[-1]] > slow_scores[order_fast[0]]
 
 
 def test_trace_replay_to_workload():

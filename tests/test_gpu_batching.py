@@ -88,10 +88,10 @@ def test_batches_of_sixteen_and_more(eng):
 
 
 @pytest.mark.parametrize("lanes", [8, 64])
-def test_batch_sizes_that_are_not_powers_of_two(eng, monkeypatch, lanes):
+def test_batch_sizes_that_are_not_powers_of_two(eng, opts, lanes):
     """The latency column of a batch size is floor(log2(size)) (controller.py:668, :716), so sizes such as 3 and 5
     share columns with 2 and 4; the kernel's shortcut for sizes 1, 2, 4, ... must not be taken then."""
-    monkeypatch.setenv("MMSIM_BATCHING_LANES", str(lanes))
+    opts(batching_lanes=lanes)
     odd = [1, 2, 3, 5, 8, 9, 17]        # floor(log2) = 0, 1, 1, 2, 3, 3, 4
     grown = 0
     for seed in range(60):
@@ -113,11 +113,11 @@ def test_batch_sizes_that_are_not_powers_of_two(eng, monkeypatch, lanes):
 
 @pytest.mark.parametrize("lanes", [8, 16, 32, 64])
 @pytest.mark.parametrize("lds_tables", [0, 1, 2, 3])
-def test_every_kernel_variant(eng, monkeypatch, lanes, lds_tables):
+def test_every_kernel_variant(eng, opts, lanes, lds_tables):
     """Tile width (simulating lanes per wavefront), which tables are read from LDS, and the number of latency
     columns held in registers (4, 8 or 16) are picked from the input's size; here each is forced."""
-    monkeypatch.setenv("MMSIM_BATCHING_LANES", str(lanes))
-    monkeypatch.setenv("MMSIM_BATCHING_LDS_TABLES", str(lds_tables))
+    opts(batching_lanes=lanes)
+    opts(batching_lds_tables=lds_tables)
     all_bss = [1 << k for k in range(16)]
     for seed, nb in enumerate([1, 3, 4, 5, 8, 9, 16] * 4):
         c = random_case(4_000_000 + 100 * lanes + 10 * lds_tables + seed, max_m=7, max_g=5, max_s=6, max_r=150,
@@ -133,10 +133,10 @@ def test_every_kernel_variant(eng, monkeypatch, lanes, lds_tables):
 
 
 @pytest.mark.parametrize("lanes", [8, 16])
-def test_many_groups_many_pending_events(eng, monkeypatch, lanes):
+def test_many_groups_many_pending_events(eng, opts, lanes):
     """More than 64 groups busy at once: the idle events fill more than eight chunks of the event list, so
     the scan of the chunk minima takes several rounds."""
-    monkeypatch.setenv("MMSIM_BATCHING_LANES", str(lanes))
+    opts(batching_lanes=lanes)
     for seed in (12, 19, 22, 44, 50, 70):      # 74 to 90 groups each, up to 23 replicas per model
         c = random_case(6_000_000 + seed, max_m=40, max_g=90, max_s=2, max_r=1500, nb=3, load=60.0,
                         inf_slo=False, tie_prob=0.1, p_member=0.15)
@@ -153,17 +153,17 @@ def test_many_groups_many_pending_events(eng, monkeypatch, lanes):
 
 
 @pytest.mark.parametrize("lanes", [8, 16])
-def test_a_simulation_that_runs_out_of_event_slots_is_reported(eng, monkeypatch, lanes):
+def test_a_simulation_that_runs_out_of_event_slots_is_reported(eng, opts, lanes):
     """With fewer event slots than busy groups the simulation stops and the call fails with MMSIM_E_OVERFLOW
     instead of returning numbers (the slots are provisioned from the group count; here they are forced down)."""
-    monkeypatch.setenv("MMSIM_BATCHING_LANES", str(lanes))
-    monkeypatch.setenv("MMSIM_BATCHING_EVENT_SLOTS", "8")
+    opts(batching_lanes=lanes)
+    opts(batching_event_slots=8)
     c = random_case(6_000_012, max_m=40, max_g=90, max_s=2, max_r=1500, nb=3, load=60.0,
                     inf_slo=False, tie_prob=0.1, p_member=0.15)
     with pytest.raises(_lib.MmsimError) as err:
         _single(eng, c, BSS[:3])
     assert err.value.code == _lib.E_OVERFLOW
-    monkeypatch.delenv("MMSIM_BATCHING_EVENT_SLOTS")
+    opts(batching_event_slots=0)
     _single(eng, c, BSS[:3])                 # and the context is fine afterwards
 
 

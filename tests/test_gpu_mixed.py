@@ -161,6 +161,36 @@ def test_config4_subsample_counts_and_a_few_full_traces(eng):
     assert (~ref["good"]).all(axis=0).mean() > 0.2      # many requests are rejected by all 64 placements
 
 
+def test_config4_every_seed_against_the_oracle(eng):
+    """The headline batch runs eight arrival seeds; here 64 placements spread over the candidate list are
+    compared with the oracle on every one of them at full stream length (8 x 64 x ~1M evaluations), at the
+    scores level (the kernel the benchmark times) and at the counts level."""
+    from concurrent.futures import ThreadPoolExecutor
+    cfg = make_config(4)
+    assert len(cfg.base_seeds) == 8
+    sols = cfg.placements[37::256][:64]
+    assert len(sols) == 64
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(sols, table)
+    streams = [cfg.stream(s) for s in cfg.base_seeds]
+    dws = [E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models) for st in streams]
+    with ThreadPoolExecutor(8) as pool:             # the oracle call releases the GIL
+        refs = list(pool.map(lambda st: oracle_batch(st, table, packed), streams))
+    for flags in (0, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS):
+        batch = E.Batch(eng, dws, table, packed, flags)
+        batch.run()
+        batch.sync()
+        out = batch.fetch()
+        name = batch.kernel_name()
+        batch.close()
+        assert name.endswith("true>"), name         # the loop over runs, as in the benchmark
+        for s, ref in enumerate(refs):
+            assert_batch_matches(out, ref, s, packed[0], where=f"cfg4 seed {cfg.base_seeds[s]}, flags {flags}")
+    assert len({int(r["n_good"].sum()) for r in refs}) == 8      # the seeds are different streams
+    for dw in dws:
+        dw.close()
+
+
 @pytest.mark.parametrize("depths", [(1, 2, 4), (1, 2, 4, 8, 16), (1, 2, 3, 4), (1, 3, 5, 8, 11, 16)])
 @pytest.mark.parametrize("uniform", [True, False])
 def test_stage_walk_variants(eng, depths, uniform):
@@ -218,7 +248,7 @@ COUNTS_IN_LDS = -2          # the same counts, per-group counters in LDS
 @pytest.mark.parametrize("flags", [0, COUNTS_IN_REGISTERS, COUNTS_IN_LDS, ALL])
 @pytest.mark.parametrize("groups,regions,segment,spin", [(1, 1, 64, None), (3, 2, 256, None), (5, 8, 512, None),
                                                         (64, 8, 16384, None), (1, 8, 64, 0), (2, 5, 128, 1)])
-def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, groups, regions, segment, spin):
+def test_scheduled_launch_with_items_taking_turns(eng, opts, flags, groups, regions, segment, spin):
     """The loop over runs is launched as a schedule: a workgroup owns several (tile, stream) items, its
     LDS is cut into regions sized by the items' clock slots, and its wavefronts simulate the items a
     segment at a time, clocks parked in device memory in between.  Forced here on a small batch with
@@ -231,14 +261,14 @@ def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, group
     from mms_amd.profiling import ParallelConfig
     from mms_amd.placement_policy.base_policy import ModelPlacement
     from mms_amd.profiling import synthetic_profile
-    monkeypatch.setenv("MMSIM_RUNS", "1")
-    monkeypatch.setenv("MMSIM_SCHED_GROUPS", str(groups))
-    monkeypatch.setenv("MMSIM_WAVES_PER_CU", str(regions))
-    monkeypatch.setenv("MMSIM_SEGMENT_REQUESTS", str(segment))
+    opts(request_loop=1)
+    opts(sched_groups=groups)
+    opts(waves_per_cu=regions)
+    opts(segment_requests=segment)
     if spin is not None:
-        monkeypatch.setenv("MMSIM_SCHED_SPIN_LIMIT", str(spin))
+        opts(sched_spin_limit=spin)
     if flags in (COUNTS_IN_REGISTERS, COUNTS_IN_LDS):
-        monkeypatch.setenv("MMSIM_COUNTS_LDS", "0" if flags == COUNTS_IN_REGISTERS else "1")
+        opts(counts_in_lds=0 if flags == COUNTS_IN_REGISTERS else 1)
         flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
     traces = bool(flags & _lib.WANT_PER_REQUEST)
     rng = np.random.default_rng(77)
@@ -281,14 +311,14 @@ def test_scheduled_launch_with_items_taking_turns(eng, monkeypatch, flags, group
 
 
 @pytest.mark.parametrize("mode", ["chunks", "runs", "batching"])
-def test_paired_placements_and_streams(eng, monkeypatch, mode):
+def test_paired_placements_and_streams(eng, opts, mode):
     """mmsim_eval_pairs simulates placement b on stream stream_of[b] only (the segments of placements that
     replace one another).  Every result must equal the [stream][placement] entry of the full cross product
     that mmsim_eval_batch computes: 150 placements over 3 streams of different lengths, tiles ragged at the
     stream boundaries, both request loops of the plain simulator and the batching simulator."""
     cfg = make_config(5 if mode == "batching" else 2, 150)
     if mode != "batching":
-        monkeypatch.setenv("MMSIM_RUNS", "1" if mode == "runs" else "0")
+        opts(request_loop=1 if mode == "runs" else 0)
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
     packed = E.pack_placements(cfg.placements, table)
     lens = (2500, 1700, 3001)
@@ -313,10 +343,10 @@ def test_paired_placements_and_streams(eng, monkeypatch, mode):
                     assert np.array_equal(got[k][b], want), (k, b)
 
 
-def test_eight_wavefronts_per_workgroup(eng, monkeypatch):
+def test_eight_wavefronts_per_workgroup(eng, opts):
     """Large batches of small placements run 8 wavefronts per workgroup (two per SIMD); forced here on
     520 placements of configuration 2 (16 clock slots)."""
-    monkeypatch.setenv("MMSIM_WAVES_PER_CU", "8")
+    opts(waves_per_cu=8)
     cfg = make_config(2, 520)
     for flags in (0, ALL):
         out, table, packed, streams, info = _run_config(eng, cfg, cfg.placements, [0, 3], flags)
@@ -335,7 +365,7 @@ def test_scores_only_mode_equals_full_mode(eng):
 
 
 @pytest.mark.parametrize("n_placements", [200, 640])
-def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placements):
+def test_scores_only_on_bursty_streams_matches_oracle(eng, opts, n_placements):
     """A scores-only run keeps the chosen group from request to request while no lane accepts, and does
     not simulate requests that every lane of a wavefront must reject.  Configuration 4's bursts (nine in
     ten requests repeat the model of the one before) exercise both: goodput and latency sums equal the
@@ -348,8 +378,8 @@ def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placem
     ref = oracle_batch(st, table, packed)
     dw = E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, cfg.num_models)
     for runs, skip in (("1", "1"), ("1", "0"), ("0", "1")):   # loop over runs (with / without skipping), chunked loop
-        monkeypatch.setenv("MMSIM_RUNS", runs)
-        monkeypatch.setenv("MMSIM_SKIP_AHEAD", skip)
+        opts(request_loop=int(runs))
+        opts(skip_ahead=int(skip))
         batch = E.Batch(eng, [dw], table, packed, 0)
         batch.run()
         batch.sync()
@@ -360,8 +390,8 @@ def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placem
     # per-model and per-group counts: requests that are not simulated still count for the group they would have chosen
     # (group counters in LDS, or in registers with adds to global rows when a lane's group changes)
     for runs, lds in (("1", "1"), ("1", "0"), ("0", "0")):
-        monkeypatch.setenv("MMSIM_RUNS", runs)
-        monkeypatch.setenv("MMSIM_COUNTS_LDS", lds)
+        opts(request_loop=int(runs))
+        opts(counts_in_lds=int(lds))
         batch = E.Batch(eng, [dw], table, packed, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
         for _ in range(2):      # a second run starts from zeroed counters again
             batch.run()
@@ -374,14 +404,14 @@ def test_scores_only_on_bursty_streams_matches_oracle(eng, monkeypatch, n_placem
 
 @pytest.mark.parametrize("loop", ["runs", "chunks"])
 @pytest.mark.parametrize("flags", [0, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS, _lib.WANT_GROUP_COUNTS + 1000, ALL])
-def test_runs_of_one_model_with_odd_requests(eng, monkeypatch, loop, flags):
+def test_runs_of_one_model_with_odd_requests(eng, opts, loop, flags):
     """Runs of equal models with tied arrival times, SLOs that change inside a run (also inf and NaN),
     unknown models, streams that end inside a block of 64, several seeds: results equal the oracle's for
     every placement of configuration 2, with either request loop, scores only and with every output."""
-    monkeypatch.setenv("MMSIM_RUNS", "1" if loop == "runs" else "0")
+    opts(request_loop=1 if loop == "runs" else 0)
     if flags >= 1000:       # per-group counts alone, kept in registers and added to global rows
         flags -= 1000
-        monkeypatch.setenv("MMSIM_COUNTS_LDS", "0")
+        opts(counts_in_lds=0)
     cfg = make_config(2)
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
     packed = E.pack_placements(cfg.placements, table)

@@ -61,10 +61,10 @@ def test_plain_simulator_two_streams_every_window(eng):
     assert 0 < out["good"].mean() < 1       # both accepted and rejected requests took part
 
 
-def test_more_simulations_than_scratch_rows_take_several_launches(eng, monkeypatch):
+def test_more_simulations_than_scratch_rows_take_several_launches(eng, opts):
     cfg = make_config(2, 11)
     R = len(cfg.stream(0).tstamps)
-    monkeypatch.setenv("MMSIM_STATS_SCRATCH_BYTES", str(3 * 8 * R + 100))   # three simulations per launch, 22 in all
+    opts(stats_scratch_bytes=3 * 8 * R + 100)   # three simulations per launch, 22 in all
     _check(eng, cfg, cfg.placements, (0, 1), [(0, 0), (R // 9, R // 8)])
 
 
@@ -127,4 +127,11 @@ def test_requires_per_request_outputs_and_the_same_streams(eng):
     batch.workloads = [other]
     with pytest.raises(_lib.MmsimError, match="streams the batch was created with"):
         batch.model_stats([0])
+    # another stream of the same length and model count is refused too: the batch knows its workloads
+    twin = E.DeviceWorkload(eng, st.tstamps, np.roll(st.model_ids, 1), st.slos, cfg.num_models)
+    batch.workloads = [twin]
+    with pytest.raises(_lib.MmsimError, match="streams the batch was created with"):
+        batch.model_stats([0])
+    batch.workloads = [dw]
+    batch.model_stats([0])
     batch.close()

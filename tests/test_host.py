@@ -53,6 +53,68 @@ def test_struct_layouts_match_the_header():
     header = open(os.path.join(ROOT, "include", "mmsim.h")).read()
     body = re.search(r"typedef struct \{([^}]*)\} mmsim_model_stats;", header).group(1)
     assert re.findall(r"\*(\w+);", body) == [f[0] for f in _lib.ModelStats._fields_]
+    # mmsim_options: field order and size, and the defaults the library fills in (no GPU needed)
+    body = re.search(r"typedef struct \{([^}]*)\} mmsim_options;", header).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    assert re.findall(r"int(?:32|64)_t (\w+);", body) == [f[0] for f in _lib.Options._fields_]
+    assert ctypes.sizeof(_lib.Options) == 14 * 4 + 8
+    opt = _lib.Options()
+    _lib.load().mmsim_options_default(ctypes.byref(opt))
+    assert opt.struct_size == ctypes.sizeof(_lib.Options)
+    assert (opt.request_loop, opt.counts_in_lds, opt.skip_ahead, opt.sched_spin_limit, opt.batching_lds_tables) == (-1,) * 5
+    assert (opt.waves_per_cu, opt.sched_groups, opt.segment_requests, opt.batching_lanes, opt.stats_scratch_bytes) == (0,) * 5
+
+
+def test_a_failed_simulation_is_an_error_not_a_score(monkeypatch):
+    """A batching simulation whose status is not 0 ran out of event slots (or met an unsupported input); its
+    counts and per-request outputs are partly unwritten.  Whatever turns results into scores or statistics must
+    raise instead of using them: the evaluator, the replacement path and the device statistics."""
+    import oracle_backend
+    from mms_amd.placement_policy import ModelPlacementWithReplacement, PlacementEvaluator, gen_train_workload
+    from mms_amd.simulator import controller as sim
+    oracle_backend.install(monkeypatch)
+    ok = E.check_status(np.zeros((2, 3), np.int32))
+    assert ok is None
+    with pytest.raises(_lib.MmsimError) as err:
+        E.check_status(np.array([[0, 0, 0], [0, _lib.E_OVERFLOW, 0]], np.int32))
+    assert err.value.code == _lib.E_OVERFLOW and "(1, 1)" in str(err.value)
+
+    model_datas = [ModelData(f"m{i}", 1.0, 4, 1, load_test_prof_result("test-2GB-100ms")) for i in range(3)]
+    cluster_env = ClusterEnv(4, 64 * GB)
+    sol = ModelPlacement([ParallelConfig(1, 1, 2), ParallelConfig(1, 1, 2)], [[0, 1, 2], [0, 1, 2]])
+    wl = gen_train_workload(model_datas, simulation_min_samples=2000)
+    forced = {"code": _lib.E_OVERFLOW}
+
+    def failing(fn):
+        def wrapped(*a, **k):
+            out = fn(*a, **k)
+            out["status"] = np.full_like(out["status"], forced["code"])
+            if not k.get("allow_failed", False):
+                E.check_status(out["status"])
+            return out
+        return wrapped
+    monkeypatch.setattr(E, "evaluate", failing(E.evaluate))
+    monkeypatch.setattr(E, "eval_pairs", failing(E.eval_pairs))
+    ev = PlacementEvaluator(model_datas, cluster_env, wl, "fast_simulator", False)
+    for call in (lambda: ev.get_scores([sol]), lambda: ev.get_stats([sol]),
+                 lambda: ev.get_scores([ModelPlacementWithReplacement([0, 50], [sol, sol])])):
+        with pytest.raises(_lib.MmsimError) as err:
+            call()
+        assert err.value.code == _lib.E_OVERFLOW
+
+    class FailingBatch(oracle_backend._HostBatch):
+        def fetch(self, per_request=True, allow_failed=False):
+            out = super().fetch(per_request)
+            out["status"] = np.full_like(out["status"], _lib.E_UNSUPPORTED)
+            if not allow_failed:
+                E.check_status(out["status"])
+            return out
+    monkeypatch.setattr(E, "Batch", FailingBatch)
+    ev._prepare()
+    model_ids, slos, names, profs = wl.cached_data
+    with pytest.raises(_lib.MmsimError) as err:
+        sim.device_compute_stats(wl, [sol], names, profs, model_ids, slos, 10)
+    assert err.value.code == _lib.E_UNSUPPORTED
 
 
 # ---- table build (controller.py:412-476) --------------------------------------------------

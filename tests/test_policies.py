@@ -30,13 +30,6 @@ from mms_amd.simulator.workload import GammaProcess, Workload
 from mms_amd.util import GB, ServingCase
 
 
-@pytest.fixture(params=["oracle", pytest.param("gpu", marks=pytest.mark.gpu)])
-def backend(request, monkeypatch):
-    if request.param == "oracle":
-        oracle_backend.install(monkeypatch)
-    return request.param
-
-
 def four_models(slo=1, rate=5, cv=1, prof="test-2GB-100ms"):
     return [ModelData(f"m{i}", slo, rate, cv, load_test_prof_result(prof)) for i in range(4)]
 
