@@ -145,67 +145,235 @@ def model_stats_bench(args, cfg, streams):
     print(json.dumps(result), flush=True)
 
 
+class _StopSearch(Exception):
+    """Raised by the bench's evaluator hook to end a search after a given number of evaluator calls."""
+
+
+class _CallLog:
+    """Counts and times the evaluator's library calls of one search (whatever backend is installed in
+    mms_amd.engine), keeps a digest of what every call returned, and can end the search after `max_calls`
+    calls or once the calls have used `budget_s` seconds."""
+
+    def __init__(self, engine_module, max_calls=None, budget_s=None):
+        self.E = engine_module
+        self.max_calls, self.budget_s = max_calls, budget_s
+        self.calls, self.placements, self.in_calls = 0, 0, 0.0
+        self.stamps, self.digests = [], []
+
+    def __enter__(self):
+        import hashlib
+        self._saved = (self.E.evaluate, self.E.evaluate_successors)
+        self.t0 = time.perf_counter()
+
+        def wrap(fn, count):
+            def hooked(*a, **k):
+                if (self.max_calls is not None and self.calls >= self.max_calls) or \
+                        (self.budget_s is not None and self.in_calls >= self.budget_s):
+                    raise _StopSearch()
+                t = time.perf_counter()
+                out = fn(*a, **k)
+                self.in_calls += time.perf_counter() - t
+                self.calls += 1
+                self.placements += count(a)
+                self.stamps.append(time.perf_counter() - self.t0)
+                h = hashlib.sha256(np.ascontiguousarray(out["n_good"]).tobytes())
+                h.update(np.ascontiguousarray(out["latency_sum"]).tobytes())
+                self.digests.append(h.hexdigest()[:12])
+                return out
+            return hooked
+        self.E.evaluate = wrap(self._saved[0], lambda a: len(a[3]))
+        self.E.evaluate_successors = wrap(self._saved[1], lambda a: len(a[3]) + len(a[4]))
+        return self
+
+    def __exit__(self, *exc):
+        self.E.evaluate, self.E.evaluate_successors = self._saved
+        self.seconds = time.perf_counter() - self.t0
+        return exc[0] is _StopSearch
+
+
 def search_bench(args):
-    """Wall clock of whole placement searches (the callers of the hot path): the three greedy policies on a
-    synthetic problem of 32 models, 32 devices and a training workload of about 1.1e5 requests, with and without
-    the one-step look-ahead of the greedy search.  Prints one JSON line; `value` is greedy steps per second of
-    `ModelParallelismSearch` with the look-ahead."""
+    """Wall clock of whole placement searches (the callers of the hot path) on the GPU, each with the SAME search
+    code timed beside it on one host core (`cpu_baseline`: the C oracle behind the evaluator, one placement after
+    another as the reference's loop does, plain greedy loop).  Greedy searches are sequential (one placement per
+    step): the GPU runs them with the one-step look-ahead; beam, layout-enumeration and evolutionary searches send
+    hundreds to thousands of placements per call.  A CPU leg that would take minutes is cut after about
+    `--cpu-budget` seconds of evaluator calls and compared with the GPU's time for the same calls (the calls must
+    have returned the same numbers).  Also measured: how long one evaluator call takes against its number of
+    placements on both sides, i.e. from how many placements per call the GPU pays.  Prints one JSON line; `value`
+    is placements scored per second over the batch-shaped searches."""
+    import pytest
+    import oracle_backend
+    from mms_amd import engine as E
     from mms_amd.placement_policy import (ClusterEnv, ModelData, ModelParallelismGreedy, ModelParallelismSearch,
-                                          SelectiveReplicationGreedy)
+                                          ModelPlacement, PlacementEvaluator, SelectiveReplicationGreedy,
+                                          SelectiveReplicationSearch)
     from mms_amd.placement_policy import base_policy
+    from mms_amd.placement_policy.base_policy import evolutionary_search, replica_placement_beam_search
     from mms_amd.profiling import ParallelConfig, synthetic_profile
     from mms_amd.simulator.workload import GammaProcess, Workload
     from mms_amd.synthetic import power_law_rates
     GB = 1 << 30
-    num_models, num_devices, total_rate, duration = 32, 32, 60.0, 1800.0
-    configs = [ParallelConfig(1, 1, pp) for pp in (1, 2, 4, 8)]
-    rates = power_law_rates(num_models, total_rate, 0.6)
-    model_datas = []
-    for i in range(num_models):
-        base = [0.15, 0.25, 0.5][i % 3]
-        prof = synthetic_profile(f"p{i % 3}", base, configs, weight_bytes=[2.6, 5.2, 13.4][i % 3] * GB)
-        model_datas.append(ModelData(f"m{i}", base * 5, float(rates[i]), 4.0, prof))
-    workload = Workload.merge(*[GammaProcess(md.rate, md.cv).generate_workload(md.name, 0, duration, slo=md.slo, seed=100 + i)
-                                for i, md in enumerate(model_datas)])
-    cluster_env = ClusterEnv(num_devices, 13 * GB)
-    log(f"[bench] search problem: {num_models} models, {num_devices} devices, {len(workload)} requests")
 
-    calls = [0]
-    run = base_policy.PlacementEvaluator._run
+    def problem(num_models, num_devices, total_rate, duration, configs):
+        rates = power_law_rates(num_models, total_rate, 0.6)
+        model_datas = []
+        for i in range(num_models):
+            base = [0.15, 0.25, 0.5][i % 3]
+            prof = synthetic_profile(f"p{i % 3}", base, configs, weight_bytes=[2.6, 5.2, 13.4][i % 3] * GB)
+            model_datas.append(ModelData(f"m{i}", base * 5, float(rates[i]), 4.0, prof))
+        workload = Workload.merge(*[GammaProcess(md.rate, md.cv).generate_workload(md.name, 0, duration, slo=md.slo, seed=100 + i)
+                                    for i, md in enumerate(model_datas)])
+        return model_datas, ClusterEnv(num_devices, 13 * GB), workload
 
-    def counted(self, sols, flags):
-        calls[0] += 1
-        return run(self, sols, flags)
-    base_policy.PlacementEvaluator._run = counted
-    policies = [("ModelParallelismSearch", lambda: ModelParallelismSearch(verbose=0)),
-                ("SelectiveReplicationGreedy", lambda: SelectiveReplicationGreedy(verbose=0)),
-                ("ModelParallelismGreedy(group_size=4)", lambda: ModelParallelismGreedy(group_size=4))]
-    ModelParallelismSearch(verbose=0).solve_placement(model_datas[:4], ClusterEnv(4, 13 * GB), workload)  # warm-up: library, context
-    rows, same = {}, True
-    for name, make in policies:
-        out = {}
-        for mode in ("lookahead", "plain"):
-            base_policy.FAST_GREEDY_LOOKAHEAD = mode == "lookahead"
-            calls[0] = 0
+    # (profiles up to 32 stages: the evolutionary search merges groups into deeper pipelines)
+    pipe = [ParallelConfig(1, 1, pp) for pp in (1, 2, 4, 8, 16, 32)]
+    md32, env32, wl32 = problem(32, 32, 60.0, 1800.0 * args.search_scale, pipe)
+    wide = sorted({ParallelConfig(1, op, pp) for op in (1, 2, 4) for pp in (1, 2, 4, 8, 16, 32)})
+    md64, env64, wl64 = problem(64, 64, 120.0, 900.0 * args.search_scale, wide)
+    log(f"[bench] search problems: 32 models / 32 devices / {len(wl32)} requests; 64 models / 64 devices / {len(wl64)} requests")
+
+    def evo(model_datas, env, wl, iters):
+        def run():
+            np.random.seed(0)
+            ev = PlacementEvaluator(model_datas, env, wl, "fast_simulator", False)
+            # start: every device its own group with one of the small models; the search does the rest
+            init = ModelPlacement([ParallelConfig(1, 1, 1)] * env.num_devices,
+                                  [[(3 * g) % len(model_datas)] for g in range(env.num_devices)])
+            return evolutionary_search([init], model_datas, env, ev, iters, 0)
+        return run
+
+    def beam_pp4(model_datas, env, wl):
+        def run():
+            ev = PlacementEvaluator(model_datas, env, wl, "fast_simulator", False)
+            n = env.num_devices // 4
+            init = ModelPlacement([ParallelConfig(1, 1, 4)] * n, [[] for _ in range(n)])
+            return replica_placement_beam_search(init, model_datas, env, wl, ev, 3, 0)
+        return run
+
+    # name -> (search, kind).  "sequential": one placement per step; "batch": many placements per call
+    searches = [
+        ("ModelParallelismSearch, 32 models / 32 devices (3 layouts, greedy)",
+         lambda: ModelParallelismSearch(verbose=0).solve_placement(md32, env32, wl32)[0], "sequential"),
+        ("SelectiveReplicationGreedy, 32 / 32",
+         lambda: SelectiveReplicationGreedy(verbose=0).solve_placement(md32, env32, wl32)[0], "sequential"),
+        ("ModelParallelismGreedy(group_size=4), 32 / 32",
+         lambda: ModelParallelismGreedy(group_size=4).solve_placement(md32, env32, wl32)[0], "sequential"),
+        ("ModelParallelismSearch, 64 models / 64 devices (12 layouts in lockstep, greedy)",
+         lambda: ModelParallelismSearch(verbose=0).solve_placement(md64, env64, wl64)[0], "sequential"),
+        ("SelectiveReplicationSearch (beam 3), 32 / 32",
+         lambda: SelectiveReplicationSearch(verbose=0).solve_placement(md32, env32, wl32)[0], "batch"),
+        ("replica_placement_beam_search (beam 3) on 8 groups of 4 stages, 32 / 32", beam_pp4(md32, env32, wl32), "batch"),
+        ("evolutionary_search (population 1024, 8 iterations), 32 / 32", evo(md32, env32, wl32, 8), "batch"),
+        ("evolutionary_search (population 1024, 4 iterations), 64 / 64", evo(md64, env64, wl64, 4), "batch"),
+    ]
+
+    # warm-up: library, context, first launches
+    ModelParallelismSearch(verbose=0).solve_placement(md32[:4], ClusterEnv(4, 13 * GB), wl32)
+
+    rows = {}
+    batch_placements, batch_seconds = 0, 0.0
+    all_same = True
+    for name, run, kind in searches:
+        row = {"kind": kind}
+        base_policy.FAST_GREEDY_LOOKAHEAD = True
+        with _CallLog(E) as gpu:
+            sol = run()
+        row["gpu"] = {"seconds": gpu.seconds, "evaluator_calls": gpu.calls, "placements_scored": gpu.placements,
+                      "seconds_inside_calls": gpu.in_calls}
+        if kind == "sequential":    # the same search without the look-ahead, for the record
+            base_policy.FAST_GREEDY_LOOKAHEAD = False
+            with _CallLog(E) as plain:
+                sol_plain = run()
+            row["gpu_without_lookahead"] = {"seconds": plain.seconds, "evaluator_calls": plain.calls}
+            row["same_placement_with_and_without_lookahead"] = str(sol) == str(sol_plain)
+            all_same = all_same and row["same_placement_with_and_without_lookahead"]
+        if not args.no_cpu:
+            # the same search code on one host core: the C oracle behind the evaluator, plain greedy loop
+            mp = pytest.MonkeyPatch()
+            oracle_backend.install(mp)
+            base_policy.FAST_GREEDY_LOOKAHEAD = False
+            try:
+                with _CallLog(E, budget_s=args.cpu_budget if kind == "batch" else None) as cpu:
+                    sol_cpu = run()
+                    cpu.finished = True
+            finally:
+                mp.undo()
+                base_policy.FAST_GREEDY_LOOKAHEAD = True
+            finished = getattr(cpu, "finished", False)
+            if finished:
+                gpu_same_work = gpu.seconds
+                same = str(sol) == str(sol_cpu)
+            else:           # cut short: compare with the GPU's time up to the same call, the calls must agree
+                k = cpu.calls
+                gpu_same_work = gpu.stamps[k - 1] if 0 < k <= len(gpu.stamps) else float("nan")
+                same = k > 0 and cpu.digests[:k] == gpu.digests[:k]
+                cpu.seconds = cpu.stamps[k - 1] if k else float("nan")
+            row["cpu_baseline"] = {
+                "seconds": cpu.seconds, "cores": 1, "kind": "port", "evaluator_calls": cpu.calls,
+                "placements_scored": cpu.placements, "complete_search": finished,
+                "sample": "the whole search" if finished else f"the first {cpu.calls} evaluator calls of the search "
+                          f"({cpu.placements} placements; cut after {args.cpu_budget:.0f} s inside the calls)",
+                "gpu_seconds_for_the_same_work": gpu_same_work,
+                "gpu_speedup_over_one_core": cpu.seconds / gpu_same_work,
+                "same_result_as_gpu": bool(same)}
+            all_same = all_same and bool(same)
+        if kind == "batch":
+            batch_placements += gpu.placements
+            batch_seconds += gpu.seconds
+        rows[name] = row
+        cb = row.get("cpu_baseline", {})
+        log(f"[bench] {name}: GPU {gpu.seconds:.2f} s / {gpu.calls} calls / {gpu.placements} placements"
+            + (f"; one core {cb['seconds']:.2f} s ({'whole search' if cb['complete_search'] else str(cb['evaluator_calls']) + ' calls'}), "
+               f"GPU for the same work {cb['gpu_seconds_for_the_same_work']:.2f} s -> {cb['gpu_speedup_over_one_core']:.2f}x, "
+               f"same result {cb['same_result_as_gpu']}" if cb else ""))
+
+    # One evaluator call against its number of placements (counts level, what get_stats asks for), on both sides:
+    # the GPU's call time is flat until the chip fills, one core's grows linearly; they cross where the GPU pays.
+    crossover = {"placements_per_call": [], "gpu_ms": [], "cpu_ms": []}
+    ev = PlacementEvaluator(md32, env32, wl32, "fast_simulator", False)
+    final, _ = SelectiveReplicationGreedy(verbose=0).solve_placement(md32, env32, wl32)
+    rng = np.random.default_rng(0)
+    pool = []
+    for _ in range(4096):      # placements like the ones the searches score: the greedy result with a few replicas dropped
+        rows_ = [list(ms) for ms in final.group_models]
+        for _ in range(4):
+            g = int(rng.integers(len(rows_)))
+            if len(rows_[g]) > 1:
+                rows_[g].pop(int(rng.integers(len(rows_[g]))))
+        pool.append(ModelPlacement(final.group_configs, rows_))
+    ev.get_stats(pool[:2])
+    cpu_ms_per_placement = None
+    if not args.no_cpu:
+        mp = pytest.MonkeyPatch()
+        oracle_backend.install(mp)
+        try:
+            ev_cpu = PlacementEvaluator(md32, env32, wl32, "fast_simulator", False)
             t0 = time.perf_counter()
-            sol, _ = make().solve_placement(model_datas, cluster_env, workload)
-            out[mode] = {"seconds": time.perf_counter() - t0, "evaluator_calls": calls[0], "placement": str(sol)}
-        same = same and out["lookahead"]["placement"] == out["plain"]["placement"]
-        rows[name] = {m: {k: v for k, v in r.items() if k != "placement"} for m, r in out.items()}
-        log(f"[bench] {name}: look-ahead {out['lookahead']['seconds']:.2f} s / {out['lookahead']['evaluator_calls']} calls, "
-            f"plain {out['plain']['seconds']:.2f} s / {out['plain']['evaluator_calls']} calls")
-    base_policy.FAST_GREEDY_LOOKAHEAD = True
-    base_policy.PlacementEvaluator._run = run
-    head = rows["ModelParallelismSearch"]
-    steps = head["plain"]["evaluator_calls"]   # one greedy step of every layout per call of the plain loop
+            ev_cpu.get_stats(pool[:64])
+            cpu_ms_per_placement = (time.perf_counter() - t0) * 1e3 / 64
+        finally:
+            mp.undo()
+    for n in (1, 8, 64, 256, 1024, 4096):
+        t0 = time.perf_counter()
+        for _ in range(3):
+            ev.get_stats(pool[:n])
+        crossover["placements_per_call"].append(n)
+        crossover["gpu_ms"].append((time.perf_counter() - t0) * 1e3 / 3)
+        crossover["cpu_ms"].append(None if cpu_ms_per_placement is None else cpu_ms_per_placement * n)
+    if cpu_ms_per_placement is not None:
+        crossover["cpu_ms_per_placement"] = cpu_ms_per_placement
+        crossover["gpu_pays_from_placements_per_call"] = crossover["gpu_ms"][0] / cpu_ms_per_placement
+    log(f"[bench] one get_stats call: {crossover}")
+
     print(json.dumps({
-        "metric": "greedy placement search, steps of all layouts per second (ModelParallelismSearch, look-ahead)",
-        "value": steps / head["lookahead"]["seconds"], "unit": "steps/s", "n_gpus": 1, "steps": 1, "warmup": 1,
-        "ms_per_step": head["lookahead"]["seconds"] * 1e3 / steps, "higher_is_better": True, "scaling": "weak",
+        "metric": "placements scored per second inside whole batch-shaped placement searches (beam, evolutionary)",
+        "value": batch_placements / batch_seconds, "unit": "placements/s", "n_gpus": 1, "steps": 1, "warmup": 1,
+        "ms_per_step": batch_seconds * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f64", "data": "synthetic",
-        "config": {"workload": f"placement search: {num_models} models, {num_devices} devices, {len(workload)} requests in the "
-                               f"training workload, 13 GB per device"},
-        "searches": rows, "same_placements_with_and_without_lookahead": bool(same)}), flush=True)
+        "config": {"workload": f"placement searches: 32 models / 32 devices / {len(wl32)} training requests and "
+                               f"64 models / 64 devices / {len(wl64)} training requests, 13 GB per device"},
+        "searches": rows, "one_evaluator_call": crossover, "every_search_gave_the_same_result_on_both_sides": bool(all_same)}),
+        flush=True)
 
 
 def main():
@@ -229,8 +397,12 @@ def main():
                          "instead of the simulation; the per-request outputs of every simulation stay on the device, so "
                          "it defaults to --placements 64 --seeds 1")
     ap.add_argument("--search", action="store_true",
-                    help="time whole greedy placement searches (the callers of the hot path) with and without the "
-                         "one-step look-ahead instead of the simulation")
+                    help="time whole placement searches (the callers of the hot path: greedy, layout enumeration, beam, "
+                         "evolutionary) on the GPU and, the same search code, on one host core, instead of the simulation")
+    ap.add_argument("--search-scale", type=float, default=1.0,
+                    help="--search: scales the length of the training workloads (for a quick run)")
+    ap.add_argument("--cpu-budget", type=float, default=15.0,
+                    help="--search: seconds of evaluator calls after which the one-core leg of a batch-shaped search is cut")
     args = ap.parse_args()
     if args.model_stats:    # 9 bytes per (simulation, request): the full batch would not fit
         args.placements = 64 if args.placements is None else args.placements

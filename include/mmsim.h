@@ -282,6 +282,34 @@ int mmsim_eval_pairs(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
                      const int32_t *stream_of, uint32_t flags, mmsim_result *out);
 
 /*
+ * mmsim_eval_batch for candidates given as "a placement plus one more replica":
+ * what the searches of the reference build one Python object at a time with
+ * sol.add_model(group, model).normalize() before they score the list
+ * (alpa_serve/placement_policy/base_policy.py:392, :453-458; ModelPlacement.add_model
+ * / normalize :24-35).  The batch holds the B base placements followed by the
+ * n successors; successor k is base placement parent[k] with model[k] appended
+ * to its group group[k].  With normalize != 0 the successor is then brought
+ * into the form ModelPlacement.normalize() gives: the models of every group in
+ * ascending order, the groups in the stable order of their model tuples (a
+ * tuple that is a prefix of another comes first), every group keeping its
+ * configuration.  The order of the groups decides which replica wins a clock
+ * tie, so it is part of the result; the per-group counts of a successor are in
+ * that order.  Results are laid out as for mmsim_eval_batch with B + n
+ * placements: simulation l = seed * (B + n) + index, index < B for a base
+ * placement and B + k for successor k.
+ */
+typedef struct {
+    int32_t n;
+    const int32_t *parent; /* [n] index of the base placement          */
+    const int32_t *group;  /* [n] group of the parent that gets a replica */
+    const int32_t *model;  /* [n] the model replicated                  */
+    int32_t normalize;
+} mmsim_successors;
+int mmsim_eval_successors(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                          const mmsim_tables *tables, const mmsim_placements *base,
+                          const mmsim_successors *successors, uint32_t flags, mmsim_result *out);
+
+/*
  * mmsim_eval_batch without any device allocation or free.  It has no
  * counterpart in the reference; it is for callers that cannot allocate device
  * memory: tight search or serving loops, harnesses that forbid hipMalloc.

@@ -49,6 +49,10 @@ class Result(C.Structure):
                 ("finish", _p_f64), ("good", _p_u8), ("status", _p_i32), ("fp_ops", _p_i64)]
 
 
+class Successors(C.Structure):
+    _fields_ = [("n", C.c_int32), ("parent", _p_i32), ("group", _p_i32), ("model", _p_i32), ("normalize", C.c_int32)]
+
+
 class Options(C.Structure):
     """mmsim_options: -1 (switches) / 0 (numbers) leave the choice to the library."""
     _fields_ = [("struct_size", C.c_int32), ("request_loop", C.c_int32), ("waves_per_cu", C.c_int32),
@@ -105,6 +109,9 @@ SIGNATURES = {
     "mmsim_batch_kernel_name": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t]),
     "mmsim_eval_batch": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
                                     C.POINTER(Placements), C.c_uint32, C.POINTER(Result)]),
+    "mmsim_eval_successors": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
+                                         C.POINTER(Placements), C.POINTER(Successors), C.c_uint32,
+                                         C.POINTER(Result)]),
     "mmsim_eval_pairs": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),
                                     C.POINTER(Placements), _p_i32, C.c_uint32, C.POINTER(Result)]),
     "mmsim_eval_batch_static": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(Tables),

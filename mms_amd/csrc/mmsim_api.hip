@@ -292,6 +292,103 @@ int lists_from_placements(const mmsim_placements *p, int32_t M, int32_t C, RepLi
     return MMSIM_OK;
 }
 
+// Base placements followed by their successors ("parent + one more replica"), as one placement list.
+// With normalize the successor is what ModelPlacement.add_model(group, model).normalize() gives
+// (alpa_serve/placement_policy/base_policy.py:24-35): the models of every group ascending, the groups in
+// the (stable) order of their model tuples, each group keeping its configuration.
+struct ExpandedPlacements {
+    std::vector<int32_t> num_groups, group_cfg, gm_idx;
+    std::vector<int64_t> gm_off;
+    mmsim_placements view{};
+};
+
+int expand_successors(const mmsim_placements *base, const mmsim_successors *sc, int32_t M, ExpandedPlacements *out) {
+    if (!base || !base->num_groups || !base->group_cfg || !base->gm_off) return fail(MMSIM_E_INVALID, "placements: null pointer");
+    if (base->B < 1 || base->Gmax < 1) return fail(MMSIM_E_INVALID, "placements: B and Gmax must be >= 1");
+    if (!sc || sc->n < 0 || (sc->n > 0 && (!sc->parent || !sc->group || !sc->model)))
+        return fail(MMSIM_E_INVALID, "successors: null pointer or negative count");
+    const int32_t B0 = base->B, Gmax = base->Gmax;
+    const int64_t total = (int64_t)B0 + sc->n;
+    if (total > 0x7FFFFFFF) return fail(MMSIM_E_UNSUPPORTED, "successors: too many placements");
+    int64_t members = 0;  // entries of gm_idx
+    for (int32_t b = 0; b < B0; ++b) {
+        const int32_t G = base->num_groups[b];
+        if (G < 0 || G > Gmax) return fail(MMSIM_E_INVALID, "placements: num_groups[b] outside 0..Gmax");
+        const int64_t *off = base->gm_off + (size_t)b * (Gmax + 1);
+        for (int32_t g = 0; g < G; ++g)
+            if (off[g + 1] < off[g]) return fail(MMSIM_E_INVALID, "placements: gm_off not monotone");
+        if (G > 0 && off[G] > off[0] && !base->gm_idx) return fail(MMSIM_E_INVALID, "placements: gm_idx is null");
+        members += G > 0 ? off[G] - off[0] : 0;
+    }
+    for (int32_t k = 0; k < sc->n; ++k) {
+        const int32_t p = sc->parent[k];
+        if (p < 0 || p >= B0) return fail(MMSIM_E_INVALID, "successors: parent outside 0..B-1");
+        if (sc->group[k] < 0 || sc->group[k] >= base->num_groups[p]) return fail(MMSIM_E_INVALID, "successors: group outside the parent's groups");
+        if (sc->model[k] < 0 || sc->model[k] >= M) return fail(MMSIM_E_INVALID, "successors: model index outside 0..M-1");
+        const int64_t *off = base->gm_off + (size_t)p * (Gmax + 1);
+        members += (base->num_groups[p] > 0 ? off[base->num_groups[p]] - off[0] : 0) + 1;
+    }
+    out->num_groups.resize((size_t)total);
+    out->group_cfg.assign((size_t)total * Gmax, 0);
+    out->gm_off.assign((size_t)total * (Gmax + 1), 0);
+    out->gm_idx.resize((size_t)members);
+    int64_t at = 0;
+    for (int32_t b = 0; b < B0; ++b) {  // the base placements as they are
+        const int32_t G = base->num_groups[b];
+        const int64_t *off = base->gm_off + (size_t)b * (Gmax + 1);
+        out->num_groups[(size_t)b] = G;
+        int64_t *dst = out->gm_off.data() + (size_t)b * (Gmax + 1);
+        for (int32_t g = 0; g < G; ++g) {
+            out->group_cfg[(size_t)b * Gmax + g] = base->group_cfg[(size_t)b * Gmax + g];
+            dst[g] = at;
+            for (int64_t x = off[g]; x < off[g + 1]; ++x) out->gm_idx[(size_t)at++] = base->gm_idx[x];
+        }
+        for (int32_t g = G; g <= Gmax; ++g) dst[g] = at;
+    }
+    parallel_slices(sc->n, 256, [&](int64_t k0, int64_t k1) {
+        // where each successor's members start: the parents' sizes are known, so slices write disjoint ranges
+        int64_t pos = at;
+        for (int64_t k = 0; k < k0; ++k) {
+            const int32_t p = sc->parent[k];
+            const int64_t *off = base->gm_off + (size_t)p * (Gmax + 1);
+            pos += (base->num_groups[p] > 0 ? off[base->num_groups[p]] - off[0] : 0) + 1;
+        }
+        std::vector<std::vector<int32_t>> rows;
+        std::vector<int32_t> order;
+        for (int64_t k = k0; k < k1; ++k) {
+            const int32_t p = sc->parent[k], G = base->num_groups[p];
+            const int64_t *off = base->gm_off + (size_t)p * (Gmax + 1);
+            rows.resize((size_t)G);
+            order.resize((size_t)G);
+            for (int32_t g = 0; g < G; ++g) {
+                rows[(size_t)g].assign(base->gm_idx + off[g], base->gm_idx + off[g + 1]);
+                if (g == sc->group[k]) rows[(size_t)g].push_back(sc->model[k]);
+                if (sc->normalize) std::sort(rows[(size_t)g].begin(), rows[(size_t)g].end());
+                order[(size_t)g] = g;
+            }
+            if (sc->normalize)
+                std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) { return rows[(size_t)x] < rows[(size_t)y]; });
+            const size_t q = (size_t)B0 + (size_t)k;
+            out->num_groups[q] = G;
+            int64_t *dst = out->gm_off.data() + q * (Gmax + 1);
+            for (int32_t g = 0; g < G; ++g) {
+                const int32_t src = order[(size_t)g];
+                out->group_cfg[q * Gmax + g] = base->group_cfg[(size_t)p * Gmax + src];
+                dst[g] = pos;
+                for (int32_t m : rows[(size_t)src]) out->gm_idx[(size_t)pos++] = m;
+            }
+            for (int32_t g = G; g <= Gmax; ++g) dst[g] = pos;
+        }
+    });
+    out->view.B = (int32_t)total;
+    out->view.Gmax = Gmax;
+    out->view.num_groups = out->num_groups.data();
+    out->view.group_cfg = out->group_cfg.data();
+    out->view.gm_off = out->gm_off.data();
+    out->view.gm_idx = out->gm_idx.data();
+    return MMSIM_OK;
+}
+
 // Builds every device table of a batch from replica lists and launches nothing.
 int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seeds, const mmsim_tables *t,
                 const RepLists &rl, uint32_t flags, mmsim_batch **out, const int32_t *stream_of = nullptr,
@@ -1623,6 +1720,18 @@ int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
     if (rc == MMSIM_OK) rc = mmsim_batch_fetch(b, out);
     mmsim_batch_destroy(b);
     return rc;
+}
+
+int mmsim_eval_successors(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                          const mmsim_tables *tables, const mmsim_placements *base, const mmsim_successors *successors,
+                          uint32_t flags, mmsim_result *out) {
+    if (!ctx || !out) return fail(MMSIM_E_INVALID, "eval_successors: null pointer");
+    int rc = check_tables(tables);
+    if (rc) return rc;
+    ExpandedPlacements all;
+    rc = expand_successors(base, successors, tables->M, &all);
+    if (rc) return rc;
+    return mmsim_eval_batch(ctx, workloads, n_seeds, tables, &all.view, flags, out);
 }
 
 int mmsim_eval_pairs(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_streams,

@@ -278,6 +278,26 @@ def eval_batch(engine: "Engine", workloads, table: "LatencyTable", packed, flags
     return _shape_results(out, n_seeds, B, allow_failed)
 
 
+def evaluate_successors(engine: "Engine", workloads, table: "LatencyTable", bases: Sequence, parent, group, model,
+                        flags: int = 0, normalize: bool = True, fixed_overhead: float = FIXED_OVERHEAD):
+    """One call of ``mmsim_eval_successors``: the placements ``bases`` followed by their successors, successor k
+    being ``bases[parent[k]].add_model(group[k], model[k])`` (``.normalize()`` with ``normalize``), built inside
+    the library instead of as Python objects.  Result arrays are [n_seeds][len(bases) + len(parent)][...]; the
+    per-group counts of a successor are in its own (normalized) group order."""
+    workloads = list(workloads)
+    t, p, wl, keep = _abi_inputs(workloads, table, pack_placements(bases, table), fixed_overhead)
+    par, grp, mod = (_lib.carray(x, np.int32) for x in (parent, group, model))
+    assert len(par) == len(grp) == len(mod)
+    sc = _lib.Successors(len(par), _lib.ptr(par, C.c_int32), _lib.ptr(grp, C.c_int32), _lib.ptr(mod, C.c_int32),
+                         1 if normalize else 0)
+    n_seeds, B = len(workloads), p.B + len(par)
+    out, r = _result_arrays(flags, n_seeds, B, t.M, p.Gmax, max(w.R for w in workloads))
+    _lib.check(engine.lib.mmsim_eval_successors(engine._h, wl, n_seeds, C.byref(t), C.byref(p), C.byref(sc),
+                                                int(flags), C.byref(r)))
+    del keep
+    return _shape_results(out, n_seeds, B)
+
+
 def eval_pairs(engine: "Engine", workloads, table: "LatencyTable", packed, stream_of, flags: int = 0,
                fixed_overhead: float = FIXED_OVERHEAD, allow_failed: bool = False):
     """One call of ``mmsim_eval_pairs``: placement b on ``workloads[stream_of[b]]`` only.

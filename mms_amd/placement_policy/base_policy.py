@@ -164,6 +164,41 @@ class BasePlacementPolicy:
         controller.sync()
 
 
+class _PerModelFastStats:
+    """The ``per_model_stats`` list of the fast statistics (controller.py:397-400), its
+    ``PerModelStatsResult`` entries made when they are read: a search that scores a thousand
+    placements per call reads the entries of the few it goes on with."""
+
+    def __init__(self, names, num_requests, goodputs, interval):
+        self._names, self._req, self._goodputs, self._interval = names, num_requests, goodputs, interval
+
+    def __len__(self):
+        return len(self._names)
+
+    def _entry(self, i):
+        req = self._req[i]
+        return PerModelStatsResult(self._names[i], req, self._goodputs[i], req / self._interval,
+                                   0, 0, 0, 0, [], [], [])
+
+    def __getitem__(self, key):
+        if isinstance(key, slice):
+            return [self._entry(i) for i in range(*key.indices(len(self)))]
+        if key < 0:
+            key += len(self)
+        if not 0 <= key < len(self):
+            raise IndexError(key)
+        return self._entry(key)
+
+    def __iter__(self):
+        return (self._entry(i) for i in range(len(self)))
+
+    def __eq__(self, other):
+        return list(self) == list(other)
+
+    def __repr__(self):
+        return repr(list(self))
+
+
 class PlacementEvaluator:
     """Scores lists of placements with the approximate simulator.
 
@@ -291,29 +326,41 @@ class PlacementEvaluator:
         stats_of = self.get_stats_lazy(sols)
         return [stats_of(b) for b in range(len(sols))]
 
-    def get_stats_lazy(self, sols: List[ModelPlacement]):
+    def get_stats_lazy(self, sols: List[ModelPlacement], successors=None):
         """One batch for all of ``sols`` like ``get_stats``; returns a function
         that builds the ``get_stats`` entry of placement ``b`` when asked.  For
         callers that evaluate more placements than they will read (the look-ahead
-        of the greedy search).  Plain placements and the fast simulator only."""
+        of the greedy search).  Plain placements and the fast simulator only.
+
+        ``successors`` = (parent, group, model) index lists: the batch then also holds,
+        behind ``sols``, the placements ``sols[parent[k]].add_model(group[k],
+        model[k]).normalize()``, built inside the library (``mmsim_eval_successors``)
+        instead of as Python objects; entry ``len(sols) + k`` is successor k."""
         assert self.method == "fast_simulator" and self._is_plain(sols)
-        out = self._run(sols, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS)
+        flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
+        num_groups = [len(s.group_configs) for s in sols]
+        if successors is None or len(successors[0]) == 0:
+            out = self._run(sols, flags)
+        else:
+            self._prepare()
+            parent, group, model = successors
+            out = _engine.evaluate_successors(self._engine, [self._device_workload], self._table, sols, parent, group,
+                                              model, flags | (_lib.BATCHING if self.enable_batching else 0))
+            num_groups = num_groups + [num_groups[p] for p in parent]
         arrivals = self.workload.arrivals
         R = len(arrivals)
         interval = arrivals[-1] - arrivals[0]
+        # per-model goodput of every placement at once: good / (requests + eps), the division of controller.py:399
+        model_goodput = out["model_num_good"][0] / (out["model_num_requests"][0] + eps)
+        goodputs = out["n_good"][0].astype(np.float64) / R
+        latency_means = out["latency_sum"][0] / R
 
         def stats_of(b):
-            sol = sols[b]
-            mreq = out["model_num_requests"][0, b]
-            mgood = out["model_num_good"][0, b]
-            greq = out["group_num_requests"][0, b, :len(sol.group_configs)]
-            per_model = [PerModelStatsResult(
-                self._names[i], mreq[i], mgood[i] / (mreq[i] + eps), mreq[i] / interval,
-                0, 0, 0, 0, [], [], []) for i in range(len(self._names))]
-            goodput = np.float64(out["n_good"][0, b]) / R
-            latency_mean = out["latency_sum"][0, b] / R
-            stats = StatsResult(per_model, tuple(greq), goodput, latency_mean, R, R / interval)
-            return (stats.goodput, [x.goodput for x in per_model], stats.group_num_requests, stats)
+            greq = out["group_num_requests"][0, b, :num_groups[b]]
+            per_model_goodput = list(model_goodput[b])
+            per_model = _PerModelFastStats(self._names, out["model_num_requests"][0, b], per_model_goodput, interval)
+            stats = StatsResult(per_model, tuple(greq), goodputs[b], latency_means[b], R, R / interval)
+            return (stats.goodput, per_model_goodput, stats.group_num_requests, stats)
         return stats_of
 
     # -- one placement at a time, same signatures as the reference's static methods -----
@@ -486,7 +533,7 @@ def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], mode
                 and hasattr(evaluator, "get_stats_lazy"))
     it = 0
     while running:
-        batch, first, kids_of = [], {}, {}
+        kids_of, kids_at = {}, {}
         look = can_look and all(isinstance(sols[i], ModelPlacement) for i in running)
         if look:
             for i in running:
@@ -494,13 +541,17 @@ def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], mode
             # (the batching simulator runs eight placements per wavefront instead of sixty-four)
             cap = FAST_GREEDY_LOOKAHEAD_LANES // (8 if getattr(evaluator, "enable_batching", False) else 1)
             look = len(running) + sum(len(k) for k in kids_of.values()) <= cap
-        for i in running:
-            first[i] = len(batch)
-            batch.append(sols[i])
-            if look:
-                batch.extend([sols[i].add_model_normalized(g, m) for g, m in kids_of[i]])
+        batch = [sols[i] for i in running]
+        first = {i: at for at, i in enumerate(running)}
         if look:
-            stats_of = evaluator.get_stats_lazy(batch)
+            # the successors are named, not built: (parent, group, model) each; the library makes the placements
+            parent, group, model = [], [], []
+            for i in running:
+                kids_at[i] = len(batch) + len(parent)
+                parent += [first[i]] * len(kids_of[i])
+                group += [g for g, _ in kids_of[i]]
+                model += [m for _, m in kids_of[i]]
+            stats_of = evaluator.get_stats_lazy(batch, (parent, group, model))
         else:
             all_stats = evaluator.get_stats(batch)
             stats_of = all_stats.__getitem__
@@ -515,9 +566,7 @@ def replica_placement_fast_greedy_lockstep(init_sols: List[ModelPlacement], mode
                 print(f"iter: {it}, search: {i}, score: {stats[0]:.4f}, elapsed: {time.time() - tic:.2f}, "
                       f"best placement: {sols[i]}, ")
             if look and choice in kids_of[i]:
-                at = first[i] + 1 + kids_of[i].index(choice)
-                assert batch[at] == sols[i]
-                stats = stats_of(at)
+                stats = stats_of(kids_at[i] + kids_of[i].index(choice))
                 choice = _fast_greedy_step(sols[i], stats, weight_mems[i], cluster_env)
                 if choice is None:
                     continue
@@ -696,6 +745,8 @@ def merge_two_groups(group_configs, group_models, model_num_unserved, weight_mem
         return
     old = group_configs[g1]
     new_cfg = ParallelConfig(old.dp, old.op, old.pp * 2)
+    if new_cfg not in weight_mem:
+        return          # no model is profiled for the deeper pipeline (the reference raises KeyError here)
     merged = list(set(group_models[g1] + group_models[g2]))
     fit_mem_budget(new_cfg, merged, model_num_unserved, weight_mem, mem_budget)
     group_configs[g1] = new_cfg
@@ -725,6 +776,19 @@ def split_one_group(group_configs, group_models, model_num_unserved, weight_mem,
     group_models.append(half_b)
 
 
+def _choice_cdf(p):
+    """What ``np.random.choice(len(p), p=p)`` makes of ``p`` before it draws."""
+    cdf = np.asarray(p, dtype=np.float64).cumsum()
+    cdf /= cdf[-1]
+    return cdf
+
+
+def _weighted_choice(cdf):
+    """``np.random.choice(len(p), p=p)`` with ``cdf = _choice_cdf(p)``: the same single draw from
+    numpy's global generator and the same index, without re-validating ``p`` on every call."""
+    return int(cdf.searchsorted(np.random.random_sample(), side="right"))
+
+
 def evolutionary_search(init_sols: List[ModelPlacement], model_datas: List[ModelData],
                         cluster_env: ClusterEnv, evaluator: PlacementEvaluator, num_iter: int,
                         verbose: int):
@@ -751,6 +815,7 @@ def evolutionary_search(init_sols: List[ModelPlacement], model_datas: List[Model
         stats = evaluator.get_stats(cur_sols)
         scores = np.array([x[0] for x in stats])
         weights = scores / np.sum(scores)
+        parent_cdf = _choice_cdf(weights)
         unserved_cache = [None] * len(stats)
 
         top = np.argmax(scores)
@@ -759,13 +824,14 @@ def evolutionary_search(init_sols: List[ModelPlacement], model_datas: List[Model
 
         next_sols = []
         while len(next_sols) < pop_size:
-            idx = np.random.choice(len(scores), p=weights)
+            idx = _weighted_choice(parent_cdf)      # np.random.choice(len(scores), p=weights)
             sol = cur_sols[idx]
             if unserved_cache[idx] is None:
                 goodputs, fullstats = stats[idx][1], stats[idx][3]
                 raw = [s.num_requests * (1 - gp) for s, gp in zip(fullstats.per_model_stats, goodputs)]
-                unserved_cache[idx] = raw / np.sum(raw)
-            unserved = unserved_cache[idx]
+                share = raw / np.sum(raw)
+                unserved_cache[idx] = (share, _choice_cdf(share))
+            unserved, unserved_cdf = unserved_cache[idx]
 
             group_configs = list(sol.group_configs)
             group_models = [list(x) for x in sol.group_models]
@@ -776,7 +842,7 @@ def evolutionary_search(init_sols: List[ModelPlacement], model_datas: List[Model
             for g in range(len(group_models)):
                 for i in range(len(group_models[g])):
                     if np.random.uniform() < mutate_one_model_prob:
-                        new_m = np.random.choice(num_models, p=unserved)
+                        new_m = _weighted_choice(unserved_cdf)      # np.random.choice(num_models, p=unserved)
                         if new_m not in group_models[g]:
                             group_models[g][i] = new_m
             child = ModelPlacement(group_configs, group_models).normalize()

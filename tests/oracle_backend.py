@@ -53,6 +53,16 @@ def _evaluate(engine, workloads, table, sols, flags=0, fixed_overhead=0.011):
     return res
 
 
+def _evaluate_successors(engine, workloads, table, bases, parent, group, model, flags=0, normalize=True,
+                         fixed_overhead=0.011):
+    """The successors as Python objects (what the library builds itself), then the plain oracle."""
+    kids = []
+    for p, g, m in zip(parent, group, model):
+        kid = bases[int(p)].add_model(int(g), int(m))
+        kids.append(kid.normalize() if normalize else kid)
+    return _evaluate(engine, workloads, table, list(bases) + kids, flags, fixed_overhead)
+
+
 def _eval_pairs(engine, workloads, table, packed, stream_of, flags=0, fixed_overhead=0.011):
     """Placement b on workloads[stream_of[b]] only; result arrays [B][...]."""
     lat, pp = table.arrays()
@@ -111,7 +121,7 @@ def model_stats_numpy(tstamps, model_ids, finish, good, skip, M):
 class _HostBatch:
     """Stand-in for engine.Batch: run / sync / fetch / model_stats on the oracle's outputs."""
 
-    def __init__(self, engine, workloads, table, packed, flags, fixed_overhead=0.011):
+    def __init__(self, engine, workloads, table, packed, flags, fixed_overhead=0.011, options=None):
         self.workloads, self.table, self.packed = list(workloads), table, packed
         self.flags, self.fixed_overhead = int(flags), fixed_overhead
         self.n_seeds, self.B, self.M = len(self.workloads), packed[1].shape[0], table.arrays()[0].shape[0]
@@ -139,7 +149,7 @@ class _HostBatch:
     def sync(self):
         return 0.0
 
-    def fetch(self, per_request=True):
+    def fetch(self, per_request=True, allow_failed=False):
         return {k: v for k, v in self.out.items() if per_request or k not in ("finish", "good")}
 
     def model_stats(self, skip):
@@ -183,6 +193,7 @@ def install(monkeypatch):
     monkeypatch.setattr(E.Engine, "default", classmethod(lambda cls: host))
     monkeypatch.setattr(E, "DeviceWorkload", _HostWorkload)
     monkeypatch.setattr(E, "evaluate", _evaluate)
+    monkeypatch.setattr(E, "evaluate_successors", _evaluate_successors)
     monkeypatch.setattr(E, "Batch", _HostBatch)
     monkeypatch.setattr(E, "eval_pairs", _eval_pairs)
     monkeypatch.setattr(E, "simulate_requests_mixed", _simulate_requests_mixed)

@@ -343,6 +343,51 @@ def test_paired_placements_and_streams(eng, opts, mode):
                     assert np.array_equal(got[k][b], want), (k, b)
 
 
+@pytest.mark.parametrize("config", [2, 5])
+@pytest.mark.parametrize("normalize", [True, False])
+def test_successors_built_by_the_library(eng, config, normalize):
+    """mmsim_eval_successors builds "placement + one more replica" candidates itself; every output must equal
+    what the same candidates give when they are built as Python objects (add_model / normalize) and sent through
+    mmsim_eval_batch -- including the order of the per-group counts, which is the order normalize() puts the
+    groups in.  Bases: placements as generated (rows unsorted, groups in no particular order), placements with
+    empty groups, and normalized ones; both simulators."""
+    from mms_amd.placement_policy.base_policy import ModelPlacement
+    cfg = make_config(config, 40)
+    rng = np.random.default_rng(11 + config)
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    bases = list(cfg.placements[:30]) + [p.normalize() for p in cfg.placements[30:40]]
+    emptied = cfg.placements[3]
+    bases.append(ModelPlacement(list(emptied.group_configs), [[] for _ in emptied.group_models]))
+    parent, group, model = [], [], []
+    for b, sol in enumerate(bases):
+        for _ in range(5):
+            g = int(rng.integers(len(sol.group_configs)))
+            free = [m for m in range(cfg.num_models) if m not in sol.group_models[g]]
+            parent.append(b)
+            group.append(g)
+            model.append(int(rng.choice(free)))
+    kids = [bases[p].add_model(g, m) for p, g, m in zip(parent, group, model)]
+    if normalize:
+        kids = [k.normalize() for k in kids]
+    st = cfg.stream(cfg.base_seeds[0])
+    n = 6000
+    dw = E.DeviceWorkload(eng, st.tstamps[:n], st.model_ids[:n], st.slos[:n], cfg.num_models)
+    flags = _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS | (_lib.BATCHING if cfg.batching else 0)
+    want = E.evaluate(eng, [dw], table, bases + kids, flags)
+    got = E.evaluate_successors(eng, [dw], table, bases, parent, group, model, flags, normalize=normalize)
+    for k in ("n_good", "latency_sum", "model_num_requests", "model_num_good", "group_num_requests", "group_num_good"):
+        assert np.array_equal(got[k], want[k]), k
+    assert len({tuple(r) for r in want["group_num_requests"][0].tolist()}) > len(bases)     # the counts tell groups apart
+    # nothing to add: the bases alone
+    alone = E.evaluate_successors(eng, [dw], table, bases, [], [], [], flags)
+    assert np.array_equal(alone["n_good"][0], want["n_good"][0][:len(bases)])
+    for bad in (([len(bases)], [0], [0]), ([0], [99], [0]), ([0], [0], [cfg.num_models])):
+        with pytest.raises(_lib.MmsimError) as err:
+            E.evaluate_successors(eng, [dw], table, bases, *bad, flags)
+        assert err.value.code == _lib.E_INVALID
+    dw.close()
+
+
 def test_eight_wavefronts_per_workgroup(eng, opts):
     """Large batches of small placements run 8 wavefronts per workgroup (two per SIMD); forced here on
     520 placements of configuration 2 (16 clock slots)."""

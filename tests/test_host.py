@@ -65,6 +65,26 @@ def test_struct_layouts_match_the_header():
     assert (opt.waves_per_cu, opt.sched_groups, opt.segment_requests, opt.batching_lanes, opt.stats_scratch_bytes) == (0,) * 5
 
 
+def test_weighted_choice_is_numpys_choice():
+    """The evolutionary search draws parents and models with np.random.choice(n, p=...) in the reference
+    (base_policy.py:662, 679); the drop-in's shortcut must consume the same draw and return the same index."""
+    from mms_amd.placement_policy.base_policy import _choice_cdf, _weighted_choice
+    rng = np.random.default_rng(0)
+    for trial in range(300):
+        n = int(rng.integers(1, 40))
+        p = rng.random(n) ** 3
+        p[rng.random(n) < 0.2] = 0.0
+        if p.sum() == 0:
+            p[0] = 1.0
+        p = p / np.sum(p)
+        cdf = _choice_cdf(p)
+        np.random.seed(trial)
+        want = [np.random.choice(n, p=p) for _ in range(5)] + [np.random.uniform()]
+        np.random.seed(trial)
+        got = [_weighted_choice(cdf) for _ in range(5)] + [np.random.uniform()]
+        assert got == want
+
+
 def test_a_failed_simulation_is_an_error_not_a_score(monkeypatch):
     """A batching simulation whose status is not 0 ran out of event slots (or met an unsupported input); its
     counts and per-request outputs are partly unwritten.  Whatever turns results into scores or statistics must
