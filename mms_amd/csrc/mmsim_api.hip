@@ -190,6 +190,12 @@ struct mmsim_batch {
     DevBuf<float> lat_nb;
     std::vector<uint8_t> hosted;  // [B][M] model has a replica (batching: decides model_num_requests)
     BatchingArgs bargs{};
+    // device buffers of mmsim_batch_model_stats, made by its first call and kept for the next ones
+    DevBuf<const MqEntry *> st_mq;
+    DevBuf<int64_t> st_i64;   // mq_off | lo | hi | sim_base
+    DevBuf<int32_t> st_i32;   // sim_stream | model_req | model_good
+    DevBuf<double> st_f64;    // the seven double results
+    DevBuf<uint64_t> st_scratch;
 
     MixedArgs args{};
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
@@ -1621,22 +1627,26 @@ int mmsim_batch_model_stats(mmsim_batch *b, const mmsim_workload *const *workloa
             sim_base[sim] = wave * b->Rmax * kWave + b->pos[p] % kWave;
         }
     const size_t cells = (size_t)n_sims * (size_t)M;
-    DevBuf<const MqEntry *> d_mq;
-    DevBuf<int64_t> d_i64;   // mq_off | lo | hi | sim_base
-    DevBuf<int32_t> d_i32;   // sim_stream | model_req | model_good
-    DevBuf<double> d_f64;    // the seven double results
-    DevBuf<uint64_t> d_scratch;
-    HIP_TRY(d_mq.alloc(mq.size()));
-    HIP_TRY(d_i64.alloc(mqo.size() + 2 * (size_t)n_streams + (size_t)n_sims));
-    HIP_TRY(d_i32.alloc((size_t)n_sims + 2 * cells));
-    HIP_TRY(d_f64.alloc(7 * cells));
-    HIP_TRY(d_scratch.alloc((size_t)rows * (size_t)pitch));
+    // (the buffers belong to the batch: the first call makes them, later calls allocate nothing)
+    DevBuf<const MqEntry *> &d_mq = b->st_mq;
+    DevBuf<int64_t> &d_i64 = b->st_i64;
+    DevBuf<int32_t> &d_i32 = b->st_i32;
+    DevBuf<double> &d_f64 = b->st_f64;
+    DevBuf<uint64_t> &d_scratch = b->st_scratch;
+    if (d_mq.n < mq.size()) HIP_TRY(d_mq.alloc(mq.size()));
+    if (d_i64.n < mqo.size() + 2 * (size_t)n_streams + (size_t)n_sims) HIP_TRY(d_i64.alloc(mqo.size() + 2 * (size_t)n_streams + (size_t)n_sims));
+    if (d_i32.n < (size_t)n_sims + 2 * cells) HIP_TRY(d_i32.alloc((size_t)n_sims + 2 * cells));
+    if (d_f64.n < 7 * cells) HIP_TRY(d_f64.alloc(7 * cells));
+    if (d_scratch.n < (size_t)rows * (size_t)pitch) HIP_TRY(d_scratch.alloc((size_t)rows * (size_t)pitch));
     HIP_TRY(hipMemcpyAsync(d_mq.p, mq.data(), sizeof(mq[0]) * mq.size(), hipMemcpyHostToDevice, st));
     int64_t *i64 = d_i64.p;
-    HIP_TRY(hipMemcpyAsync(i64, mqo.data(), sizeof(int64_t) * mqo.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(hipMemcpyAsync(i64 + mqo.size(), lo.data(), sizeof(int64_t) * lo.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(hipMemcpyAsync(i64 + mqo.size() + lo.size(), hi.data(), sizeof(int64_t) * hi.size(), hipMemcpyHostToDevice, st));
-    HIP_TRY(hipMemcpyAsync(i64 + mqo.size() + 2 * lo.size(), sim_base.data(), sizeof(int64_t) * sim_base.size(), hipMemcpyHostToDevice, st));
+    std::vector<int64_t> up;  // one upload: mq_off | lo | hi | sim_base (alive until the stream is waited for below)
+    up.reserve(mqo.size() + 2 * lo.size() + sim_base.size());
+    up.insert(up.end(), mqo.begin(), mqo.end());
+    up.insert(up.end(), lo.begin(), lo.end());
+    up.insert(up.end(), hi.begin(), hi.end());
+    up.insert(up.end(), sim_base.begin(), sim_base.end());
+    HIP_TRY(hipMemcpyAsync(i64, up.data(), sizeof(int64_t) * up.size(), hipMemcpyHostToDevice, st));
     HIP_TRY(hipMemcpyAsync(d_i32.p, sim_stream.data(), sizeof(int32_t) * sim_stream.size(), hipMemcpyHostToDevice, st));
     StatsArgs f{};
     f.finish = b->finish.p;
@@ -1661,13 +1671,17 @@ int mmsim_batch_model_stats(mmsim_batch *b, const mmsim_workload *const *workloa
         hipError_t e = launch_model_stats(f, (int)std::min<int64_t>(rows, n_sims - sim0), st, &err);
         if (e != hipSuccess) return fail(MMSIM_E_HIP, err.empty() ? std::string("model_stats launch: ") + hipGetErrorString(e) : err);
     }
-    HIP_TRY(hipMemcpyAsync(out->model_num_requests, f.model_req, sizeof(int32_t) * cells, hipMemcpyDeviceToHost, st));
-    HIP_TRY(hipMemcpyAsync(out->model_num_good, f.model_good, sizeof(int32_t) * cells, hipMemcpyDeviceToHost, st));
+    // two copies back (the integer results, the double results), then into the caller's arrays
+    std::vector<int32_t> h_i32(2 * cells);
+    std::vector<double> h_f64(7 * cells);
+    HIP_TRY(hipMemcpyAsync(h_i32.data(), f.model_req, sizeof(int32_t) * 2 * cells, hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipMemcpyAsync(h_f64.data(), d, sizeof(double) * 7 * cells, hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    std::memcpy(out->model_num_requests, h_i32.data(), sizeof(int32_t) * cells);
+    std::memcpy(out->model_num_good, h_i32.data() + cells, sizeof(int32_t) * cells);
     double *const o64[7] = {out->first_start, out->last_start, out->latency_sum, out->latency_mean,
                             out->latency_std, out->latency_p90, out->latency_p99};
-    for (int k = 0; k < 7; ++k)
-        HIP_TRY(hipMemcpyAsync(o64[k], d + (size_t)k * cells, sizeof(double) * cells, hipMemcpyDeviceToHost, st));
-    HIP_TRY(hipStreamSynchronize(st));
+    for (int k = 0; k < 7; ++k) std::memcpy(o64[k], h_f64.data() + (size_t)k * cells, sizeof(double) * cells);
     return MMSIM_OK;
 }
 

@@ -452,6 +452,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     };
     const ScanAddr no_addr{};
     auto nothing = []() {};
+    // Loop over runs: LDS addresses of the last-stage clocks of the run's listed replicas, worked out once per run
+    // (they depend on the descriptors only) and pinned there.
+    uint32_t run_ca[RREG] = {};
 
     // (PLAIN: the caller has seen that the tile lists one to four replicas for the model: the scan has no case to
     // tell, reads where `sa` says, and calls `meanwhile` once its reads are under way)
@@ -484,10 +487,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                 if constexpr (plain_scan) {
                     k[j].c = lds_f64(sa.c[j]);
                     k[j].l = lds_f32(sa.l[j]);
+                } else if constexpr (RUNS) {
+                    k[j].c = lds_f64(run_ca[j0 + j]);
+                    k[j].l = 0.0f;  // (the winner's latency is read after the tournament instead, one read for eight)
                 } else {
                     k[j].c = lds_f64(rep_addr(k[j].d) + rel_base);
-                    // (loop over runs: the winner's latency is read after the tournament instead, one read for eight)
-                    k[j].l = RUNS ? 0.0f : lrow_m[rep_lat_last(k[j].d)];
+                    k[j].l = lrow_m[rep_lat_last(k[j].d)];
                 }
                 return true;
             });
@@ -713,14 +718,17 @@ asm volatile(NAME##_TEXT                                                        
     if constexpr (RUNS) {
         // Descriptors of the run about to start (fetched while the run before it is simulated).
         uint4 nda = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty), ndb = nda;
-        auto fetch_run = [&](int model) {  // model < 0: any row will do, nothing is simulated
+        // (the second half of a row, replicas 4-7, is only read by runs whose tile lists more than four replicas
+        // for the model; the other runs load the first half twice -- the second load hits the line the first one
+        // just brought in -- which costs no branch and no memory traffic)
+        auto fetch_run = [&](int model, bool more_than_four) {  // model < 0: any row will do, nothing is simulated
             const uint4 *row = rep_tile + (size_t)(model < 0 ? 0 : model) * (2 * kWave);
             nda = row[0];
-            ndb = row[kWave];
+            ndb = row[more_than_four ? kWave : 0];
         };
         {
             const int z0 = __builtin_amdgcn_readlane(ahead.z, 0);
-            fetch_run(r0 < r1 ? z0 : -1);
+            fetch_run(r0 < r1 ? z0 : -1, true);
         }
 
         for (int64_t blk = r0; blk < r1; blk += kWave) {
@@ -757,13 +765,22 @@ asm volatile(NAME##_TEXT                                                        
                         zn = __builtin_amdgcn_readlane(r.z, s1);
                     else if (blk + kWave < r1)
                         zn = __builtin_amdgcn_readlane(ahead.z, 0);
-                    fetch_run(zn < 0 ? -1 : (zn & 0xFFFFFF));
+                    // (a word of this block carries the tile's replica bound; the first word of the next block does
+                    // not yet, so its row is fetched whole)
+                    fetch_run(zn < 0 ? -1 : (zn & 0xFFFFFF), s1 >= nblk || (zn >> 24) > 4);
                 }
                 const int w = __builtin_amdgcn_readlane(r.z, s0);
                 const int m = w >= 0 ? (w & 0xFFFFFF) : -1;  // wave-uniform model id (or -1)
                 const int n = w >= 0 ? (w >> 24) : 0;        // replica bound of the tile; 0: nothing to simulate
                 const uint64_t run = (s1 >= 64 ? ~0ull : ((1ull << s1) - 1ull)) & (~0ull << s0) & valid;
                 const int32_t good_before = n_good;  // model_per_run
+                static_while<0, RREG>([&](auto J) {
+                    constexpr int j = decltype(J)::value;
+                    run_ca[j] = rep_addr(pick_desc<j>(da, db)) + rel_base;
+                    return true;
+                });
+                asm volatile("" : "+v"(run_ca[0]), "+v"(run_ca[1]), "+v"(run_ca[2]), "+v"(run_ca[3]), "+v"(run_ca[4]),
+                                  "+v"(run_ca[5]), "+v"(run_ca[6]), "+v"(run_ca[7]));
 
                 auto request = [&](int i) {
                     return simulate(blk + i, m, n, da, db,

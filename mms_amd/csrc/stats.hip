@@ -13,7 +13,11 @@
 // Percentiles are order statistics: sorted[int(q * n)] (workload.py:344-346), found exactly with a
 // radix selection on a 64-bit key that orders like the latency (its bit pattern with the sign handled): eight
 // passes of eight bits, most significant first, counting into 256 bins in LDS the elements that match
-// the digits fixed so far; both percentiles in the same passes (two histograms).  The first pass also
+// the digits fixed so far; both percentiles in the same passes (two histograms).  Latencies are spread
+// out, so after two or three digits only a handful of elements still match: once no more than 1024 do
+// (for either percentile), they are collected in LDS and ranked there directly, which ends the
+// selection in one more sweep instead of up to six (equal latencies by the thousand, as an idle system
+// produces, simply run all eight passes).  The first pass also
 // counts and sums (n decides the two ranks), the second one sums the squared deviations.  Sums are
 // compensated (Neumaier) per thread and added up in a fixed order, so mean and deviation are within a
 // few ulp of the exact value, as numpy's pairwise sums are; they are not bit-equal to numpy's.
@@ -35,6 +39,7 @@ struct Accum {
 };
 
 constexpr int kStatsThreads = 1024;
+constexpr int kSmallSelect = 1024;  // candidates that are ranked directly in LDS
 // Latencies are selected by a 64-bit key that orders like the double (sign flipped for positive values, all bits
 // for negative ones: the batching simulator can finish a request before it arrived, when a group that became idle
 // earlier picks it up with its old idle time, controller.py:739-744, :715-720).  All ones is the key of a NaN
@@ -64,7 +69,8 @@ __global__ __launch_bounds__(kStatsThreads) void model_stats_kernel(StatsArgs a)
     __shared__ int32_t part_n[kStatsThreads / kWave];
     __shared__ long long part_first[kStatsThreads / kWave], part_last[kStatsThreads / kWave];
     __shared__ uint64_t sh_pre[2];
-    __shared__ uint32_t sh_k[2];
+    __shared__ uint32_t sh_k[2], sh_cand[2], sh_cnt[2];
+    __shared__ uint64_t cand[2][kSmallSelect];
     __shared__ double sh_total;
     const int tid = threadIdx.x, wv = tid / kWave, ln = tid % kWave;
     const int row = blockIdx.x, sim = a.sim0 + row, m = blockIdx.y;  // row: the simulation's scratch row in this launch
@@ -188,8 +194,37 @@ __global__ __launch_bounds__(kStatsThreads) void model_stats_kernel(StatsArgs a)
             }
             sh_pre[tid] |= (uint64_t)sel << shift;
             sh_k[tid] = k - before;
+            sh_cand[tid] = found ? hh[sel] : 0u;  // elements that match the digits fixed so far
+            sh_cnt[tid] = 0;
         }
         __syncthreads();
+        if (pass >= 1 && pass < 7 && sh_cand[0] <= (uint32_t)kSmallSelect && sh_cand[1] <= (uint32_t)kSmallSelect) {
+            // few candidates left: collect them (in any order) and rank them directly; rank sh_k among the
+            // candidates of a percentile is its order statistic (equal keys are told apart by their place)
+            const uint64_t fixed = ~0ull << shift;
+            const uint64_t pre0 = sh_pre[0], pre1 = sh_pre[1];
+            for (int64_t e = e0 + tid; e < e1; e += kStatsThreads) {
+                const uint64_t bits = scr[e];
+                if (bits == kNotAccepted) continue;
+                if ((bits & fixed) == pre0) cand[0][atomicAdd(&sh_cnt[0], 1u)] = bits;
+                if ((bits & fixed) == pre1) cand[1][atomicAdd(&sh_cnt[1], 1u)] = bits;
+            }
+            __syncthreads();
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t c = sh_cnt[h];
+                if ((uint32_t)tid < c) {
+                    const uint64_t mine = cand[h][tid];
+                    uint32_t rank = 0;
+                    for (uint32_t j = 0; j < c; ++j) {
+                        const uint64_t other = cand[h][j];
+                        rank += (other < mine || (other == mine && j < (uint32_t)tid)) ? 1u : 0u;
+                    }
+                    if (rank == sh_k[h]) sh_pre[h] = mine;
+                }
+            }
+            __syncthreads();
+            break;
+        }
         for (int b = tid; b < 2 * kBins; b += kStatsThreads) (&hist[0][0])[b] = 0;
         __syncthreads();
     }
