@@ -811,6 +811,9 @@ def evolutionary_search(init_sols: List[ModelPlacement], model_datas: List[Model
     best_score, best_sol = -1, None
     visited = set()
     cur_sols = init_sols
+    # np.random.uniform() of the reference (:672-678) is 0.0 + 1.0 * random_sample(): the same draw and the same
+    # value from numpy's global generator, at a tenth of the call cost (a child takes some fifty of them)
+    uniform = np.random.random_sample
     for it in range(num_iter):
         stats = evaluator.get_stats(cur_sols)
         scores = np.array([x[0] for x in stats])
@@ -828,20 +831,24 @@ def evolutionary_search(init_sols: List[ModelPlacement], model_datas: List[Model
             sol = cur_sols[idx]
             if unserved_cache[idx] is None:
                 goodputs, fullstats = stats[idx][1], stats[idx][3]
-                raw = [s.num_requests * (1 - gp) for s, gp in zip(fullstats.per_model_stats, goodputs)]
+                per_model = fullstats.per_model_stats
+                if isinstance(per_model, _PerModelFastStats):   # the same products, without making the entries
+                    raw = per_model._req * (1 - np.asarray(goodputs, dtype=np.float64))
+                else:
+                    raw = [s.num_requests * (1 - gp) for s, gp in zip(per_model, goodputs)]
                 share = raw / np.sum(raw)
                 unserved_cache[idx] = (share, _choice_cdf(share))
             unserved, unserved_cdf = unserved_cache[idx]
 
             group_configs = list(sol.group_configs)
             group_models = [list(x) for x in sol.group_models]
-            if np.random.uniform() < merge_group_prob:
+            if uniform() < merge_group_prob:
                 merge_two_groups(group_configs, group_models, unserved, weight_mem, mem_budget)
-            if np.random.uniform() < split_group_prob:
+            if uniform() < split_group_prob:
                 split_one_group(group_configs, group_models, unserved, weight_mem, mem_budget)
             for g in range(len(group_models)):
                 for i in range(len(group_models[g])):
-                    if np.random.uniform() < mutate_one_model_prob:
+                    if uniform() < mutate_one_model_prob:
                         new_m = _weighted_choice(unserved_cdf)      # np.random.choice(num_models, p=unserved)
                         if new_m not in group_models[g]:
                             group_models[g][i] = new_m
