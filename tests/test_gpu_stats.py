@@ -94,6 +94,30 @@ def test_a_handful_of_simulations(eng, config, placements, seeds, shrink, flags)
                                              tuple(R // 2 + 3 for _ in seeds)], flags=flags)
 
 
+def test_equal_latencies_by_the_thousand_and_few_distinct_ones(eng):
+    """The selection ranks the last candidates directly once at most 1024 still match the digits fixed so far.  An idle
+    system gives thousands of requests the very same latency, so the candidates never thin out and all eight
+    passes run; two latency values with a few thousand requests each thin out only at the last differing digit; a
+    short stream is small from the start.  All three against numpy."""
+    from types import SimpleNamespace
+    from mms_amd.placement_policy.base_policy import ModelPlacement
+    from mms_amd.profiling import ParallelConfig, synthetic_profile
+    pcs = [ParallelConfig(1, 1, 1), ParallelConfig(1, 1, 2)]
+    profiles = [synthetic_profile("a", 0.1, pcs), synthetic_profile("b", 0.1000001, pcs)]
+    sols = [ModelPlacement([pcs[0], pcs[0]], [[0], [1]]), ModelPlacement([pcs[1]], [[0, 1]])]
+    for R, gap in ((20000, 1.0), (6000, 0.12), (300, 1.0), (1025, 1.0), (2049, 1.0)):
+        t = np.arange(R) * gap                                   # gap 1.0: every request finds its group idle
+        m = (np.arange(R) % 2).astype(np.int32)
+        cfg = SimpleNamespace(profiles=profiles, batch_sizes=[1], num_models=2,
+                              stream=lambda s, t=t, m=m: SimpleNamespace(tstamps=t, model_ids=m, slos=np.full(len(t), 5.0, np.float32)))
+        out = _check(eng, cfg, sols, (0,), [(0,), (R // 7,)])
+        lat = out["finish"][0, 0, :R] - t
+        assert out["good"][0, 0].all()
+        if R == 20000:      # (the latency only changes in its last bits from one binade of the arrival time to the next)
+            for model in (0, 1):
+                assert np.unique(lat[m == model], return_counts=True)[1].max() > 2 * 1024
+
+
 def test_negative_latencies_of_the_batching_simulator(eng):
     """A group that became idle earlier can pick a request up with its old idle time and finish it before it arrived
     (controller.py:739-744, :715-720; the oracle does the same): the selection must order negative latencies below
