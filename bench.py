@@ -403,6 +403,9 @@ def main():
                     help="--search: scales the length of the training workloads (for a quick run)")
     ap.add_argument("--cpu-budget", type=float, default=15.0,
                     help="--search: seconds of evaluator calls after which the one-core leg of a batch-shaped search is cut")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="a field of the library's options (mmsim_options in include/mmsim.h), e.g. batching_lds_tables=2; "
+                         "repeatable; the default run sets none")
     args = ap.parse_args()
     if args.model_stats:    # 9 bytes per (simulation, request): the full batch would not fit
         args.placements = 64 if args.placements is None else args.placements
@@ -444,6 +447,8 @@ def main():
     eng = E.Engine.default()
     dev = eng.device_info()
     log(f"[bench] device: {dev}")
+    if args.option:
+        eng.set_options(**{k: int(v) for k, v in (kv.split("=", 1) for kv in args.option)})
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
     t0 = time.perf_counter()
     packed = E.pack_placements(cfg.placements, table)
@@ -537,7 +542,8 @@ def main():
                    "workgroups": info["workgroups"], "wavefronts_per_workgroup": info["waves_per_group"],
                    "lds_bytes_per_workgroup": info["lds_bytes"], "stream_segments": info["segments"],
                    "placements": B, "seeds": len(seeds), "requests_per_seed": R_total // len(seeds),
-                   "lanes": lanes, "outputs": args.flags, "inputs_resident_in_hbm": True},
+                   "lanes": lanes, "outputs": args.flags, "inputs_resident_in_hbm": True,
+                   **({"options": args.option} if args.option else {})},
         "placements_per_sec": lanes / sec_per_step,
         "kernel_ms": kernel_s * 1e3,
         "goodput_mean": float(out["n_good"].sum() / evals_per_step),

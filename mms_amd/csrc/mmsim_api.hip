@@ -484,12 +484,12 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     //      latencies for configuration 0, then configuration 1, ... (the cfg_pp[c] real
     //      stages only).  When every (model, config) has one latency for all its stages the
     //      row is just one value per configuration.
-    bool uniform_stages = !batching;  // the batching kernel reads per-stage, per-batch-size latencies
+    bool uniform_stages = true;  // (the batching kernel reads every batch size's column: all of them must agree)
     for (int32_t m = 0; m < M && uniform_stages; ++m)
         for (int c = 0; c < C && uniform_stages; ++c) {
             const float *row = t->cfg_lat + ((size_t)m * C + c) * t->Smax * t->NB;
             for (int k = 1; k < t->cfg_pp[c]; ++k)
-                if (std::memcmp(&row[(size_t)k * t->NB], &row[0], sizeof(float)) != 0) uniform_stages = false;
+                if (std::memcmp(&row[(size_t)k * t->NB], &row[0], sizeof(float) * (batching ? (size_t)t->NB : 1)) != 0) uniform_stages = false;
         }
     std::vector<int32_t> lat_off(C + 1, 0);
     for (int c = 0; c < C; ++c) lat_off[c + 1] = lat_off[c] + (uniform_stages ? 1 : t->cfg_pp[c]);
@@ -846,8 +846,12 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     std::vector<uint32_t> rep32, repx32;
     std::vector<uint64_t> rep8;
     std::vector<uint8_t> repx;
+    // Tiles of eight simulations (octets): a row of rep8 is read as 64 descriptors instead, one per lane of the
+    // wavefront -- lane 8 * simulation + j holds the descriptor of the j-th replica (kEmpty: none); the second half
+    // of the row is not used.
+    const bool octets = batching && blanes == 8;
     if (batching) {
-        rep8.assign((size_t)b->tiles * M * kWave, none8);
+        rep8.assign((size_t)b->tiles * M * kWave, octets ? ((uint64_t)kEmpty << 32 | kEmpty) : none8);
         repx.assign((size_t)b->tiles * M * RX * kWave, (uint8_t)Gmax);
     } else {
         rep32.resize((size_t)b->tiles * M * 2 * kWave * 4);
@@ -901,7 +905,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 const int32_t g = rl.grp[(size_t)x];
                 const int j = (int)(x - lo);
                 if (batching) {
-                    if (j < kPackedReplicas)
+                    if (j < kPackedReplicas && octets)
+                        reinterpret_cast<uint32_t *>(rep8.data())[((size_t)tile * M + m) * 2 * kWave + (size_t)lane * 8 + (size_t)j] =
+                            ginfo[((size_t)tile * (Gmax + 1) + g) * kWave + lane];
+                    else if (j < kPackedReplicas)
                         word = (word & ~(0xFFull << (8 * j))) | ((uint64_t)g << (8 * j));
                     else
                         repx[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = (uint8_t)g;
@@ -916,7 +923,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                         repx32[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = d;
                 }
             }
-            if (batching) rep8[((size_t)tile * M + m) * kWave + lane] = word;
+            if (batching && !octets) rep8[((size_t)tile * M + m) * kWave + lane] = word;
         }
     }
     });
@@ -968,7 +975,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         lat_nb.resize((size_t)M * lat_row * t->NB);
         for (int32_t m = 0; m < M; ++m)
             for (int c = 0; c < C; ++c)
-                for (int k = 0; k < t->cfg_pp[c]; ++k)
+                for (int k = 0; k < (uniform_stages ? 1 : t->cfg_pp[c]); ++k)
                     for (int q = 0; q < t->NB; ++q) {
                         const float v = t->cfg_lat[(((size_t)m * C + c) * t->Smax + k) * t->NB + q];
                         if (v != v || v < 0.0f) return fail(MMSIM_E_INVALID, "tables: a stage latency is NaN or negative");
@@ -996,8 +1003,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         for (int hc = heap_cap; hc >= heap_try_min; hc -= 8) {
             const size_t wb = batching_bytes_for(blanes, hc);
             for (int per_cu = 1; per_cu <= 2; ++per_cu)  // workgroups meant to share a CU (each gets that share of LDS)
-                for (int opt = 0; opt < 4; ++opt) {      // both, table only, lists only, neither: the first that gives most wavefronts
-                    const bool want_lat = opt < 2, want_g2m = opt == 0 || opt == 2;
+                for (int opt = 0; opt < 4; ++opt) {      // both, lists only, table only, neither: the first that gives most wavefronts
+                    // (the lists before the table: a selection reads them in two dependent steps, while the table is
+                    // read beside the queue's entries, which come from memory anyway; measured 2.19 s against 2.42 s)
+                    const bool want_lat = opt == 0 || opt == 2, want_g2m = opt < 2;
                     if ((want_lat && !(allowed & 1)) || (want_g2m && !(allowed & 2))) continue;
                     const size_t per = wb + (want_g2m ? g2m_b : 0), shared = want_lat ? lat_b : 0;
                     if (shared + per > cap / per_cu) continue;
@@ -1223,6 +1232,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         q.lat_lds_bytes = (int32_t)batching_lat_lds;
         q.g2m_in_lds = batching_g2m_lds;
         q.lane_stride = blanes;
+        q.uniform_stages = uniform_stages ? 1 : 0;
         q.tile_seed = b->tile_seed.p;
         q.paired = b->paired ? 1 : 0;
         q.Rmax = b->Rmax;

@@ -181,6 +181,7 @@ struct BatchingArgs {
     int32_t lat_lds_bytes;       // > 0: the workgroup keeps a copy of lat in LDS (that many bytes, 16-aligned)
     int32_t g2m_in_lds;          // 1: each wavefront keeps its g2m_off / g2m_idx rows in LDS
     int32_t lane_stride;         // 64, 32 or 16: lanes of a wavefront that simulate; pitch of the per-lane LDS arrays
+    int32_t uniform_stages;      // 1: a configuration's stages all have the same latencies and lat holds them once ([M][lat_row][NB], one row per configuration)
     const int32_t *tile_seed;    // as in MixedArgs
     int32_t paired;
     int64_t Rmax;

@@ -87,6 +87,15 @@ __device__ __forceinline__ double oct_get(double v, int k) {
     return __hiloint2double((int)oct_get((uint32_t)__double2hiint(v), k), (int)oct_get((uint32_t)__double2loint(v), k));
 }
 __device__ __forceinline__ float oct_get(float v, int k) { return __uint_as_float(oct_get(__float_as_uint(v), k)); }
+// the value of the octet's first lane: the first lane of each quad to its quad, then the lanes of the octet's second
+// quad take the lane four below (two DPP moves, no trip through the LDS crossbar)
+__device__ __forceinline__ uint32_t oct_first(uint32_t v) {
+    const int q = __builtin_amdgcn_update_dpp(0, (int)v, 0x00 /* quad_perm 0,0,0,0 */, 0xF, 0xF, false);
+    return (uint32_t)__builtin_amdgcn_update_dpp(q, q, 0x114 /* row_shr:4 */, 0xF, 0xA /* lanes 4-7 and 12-15 of a row */, false);
+}
+__device__ __forceinline__ double oct_first(double v) {
+    return __hiloint2double((int)oct_first((uint32_t)__double2hiint(v)), (int)oct_first((uint32_t)__double2loint(v)));
+}
 // The lanes of an octet run in lockstep; this marks the places where that matters (all have read a
 // value before any of them overwrites it).  No instruction.
 __device__ __forceinline__ void oct_sync() { __builtin_amdgcn_wave_barrier(); }
@@ -135,7 +144,12 @@ __device__ __forceinline__ lds_vu32 *as_lds_vu32(void *p) { return (lds_vu32 *)p
 // OCT: tiles of eight simulations, each worked on by an octet of consecutive lanes (lane = 8 * simulation
 // + helper).  The lanes of an octet hold the same state and take the same branches; the scans (event
 // slots, models of a group, replicas, heads' deadlines, latency columns) are split among them.
-template <int NBT, bool LATLDS, bool G2MLDS, bool OCT>
+// UNIF: every (model, configuration) has the same latencies in all of its stages, and the table holds them
+// once (a row of NB columns per configuration): a pass over a group's stages loads its latency once.
+// SH (octets only): at most 64 event slots per simulation.  Which slots are in use is a 64-bit mask in registers
+// and lane c of an octet keeps the earliest time of chunk c in a register: neither the free-slot stack nor the
+// chunk minima are read from LDS.
+template <int NBT, bool LATLDS, bool G2MLDS, bool OCT, bool UNIF, bool SH>
 __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching_kernel(const BatchingArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
@@ -236,6 +250,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const int64_t R = a.stream_off[seed + 1] - off;
     const Req *__restrict__ reqs = a.streams + off;
     const uint64_t *__restrict__ rep_tile = a.rep8 + (size_t)tile * M * kWave + sl;
+    // octets: the row of a model holds a descriptor per lane (the j-th replica's group for lane 8 * simulation + j)
+    const uint32_t *__restrict__ repd_tile = reinterpret_cast<const uint32_t *>(a.rep8) + (size_t)tile * M * 2 * kWave + lane;
+    auto row_of = [&](int mx) -> uint64_t {
+        const size_t mr = (size_t)(mx < 0 ? 0 : mx);
+        if constexpr (OCT) return repd_tile[mr * 2 * kWave];
+        return rep_tile[mr * kWave];
+    };
     const uint8_t *__restrict__ repx_tile = a.repx + (size_t)tile * M * a.rep_extra * kWave + sl;
     const uint16_t *g2m_off_glb = a.g2m_off + (size_t)tile * (Gmax + 1) * kWave + sl;
     const uint16_t *g2m_idx_glb = a.g2m_idx + (size_t)tile * a.members_max * kWave + sl;
@@ -252,6 +273,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     int32_t n_good = 0;
     double lat_sum = 0.0;
     int nfree = a.heap_cap;  // free event slots of this lane (heap_cap - nfree events are pending)
+    uint64_t used = 0;       // SH: bit e = event slot e holds an event
+    double my_cm = __builtin_inf();  // SH: the earliest event time of chunk oj (this lane's place in its octet)
+    static_assert(!SH || OCT, "registers for the event slots' bookkeeping go with octets");
     double next_due = __builtin_inf();  // the earliest of them (+inf if none): arrivals before it skip the event list
     int dead = sim ? 0 : 1;  // nonzero: this lane simulates nothing (more): out of event slots, unsupported input, or a spare lane of a narrow tile
 
@@ -324,6 +348,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     auto batch_times = [&](double t0, const double *gclk, int stages, uint32_t lat_mg, double(&tb)[NBT]) {
 #pragma unroll
         for (int b = 0; b < NBT; ++b) tb[b] = t0;
+        float lu[NBT];
+        if constexpr (UNIF) {
+#pragma unroll
+            for (int b = 0; b < NBT; ++b) lu[b] = lat_at(lat_mg + (uint32_t)(b < NB ? b : NB - 1));
+        }
         for (int k0 = 0; k0 < stages; k0 += 4) {
             double c[4];
             float l[4][NBT];
@@ -332,7 +361,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 const int k = k0 + u < stages ? k0 + u : stages - 1;
                 c[u] = gclk[k * LS];
 #pragma unroll
-                for (int b = 0; b < NBT; ++b) l[u][b] = lat_at(lat_mg + (uint32_t)(k * NB + (b < NB ? b : NB - 1)));
+                for (int b = 0; b < NBT; ++b) l[u][b] = UNIF ? lu[b] : lat_at(lat_mg + (uint32_t)(k * NB + (b < NB ? b : NB - 1)));
             }
 #pragma unroll
             for (int u = 1; u < 4; ++u)
@@ -350,9 +379,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     };
 
     // the same for one latency column (the octet's lanes take one column each)
-    // c0 / l0: the clocks and this column's latencies of the first four stages as read (the commit reuses them)
-    auto batch_time_col = [&](double t0, const double *gclk, int stages, uint32_t lat_mg, int col, double(&c0)[4],
-                              float(&l0)[4]) -> double {
+    // c0: the group's clocks of the first four stages, read by the caller (they do not change before the commit, which
+    // uses them again); lu: with UNIF, the column's latency; l0: otherwise, the column's latencies of the first four
+    // stages as read here (the commit takes them from the lane that had its column)
+    auto batch_time_col = [&](double t0, const double *gclk, int stages, uint32_t lat_mg, int col, const double(&c0)[4],
+                              float lu, float(&l0)[4]) -> double {
         double t = t0;
         for (int k0 = 0; k0 < stages; k0 += 4) {
             double c[4];
@@ -360,15 +391,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int k = k0 + u < stages ? k0 + u : stages - 1;
-                c[u] = gclk[k * LS];
-                l[u] = lat_at(lat_mg + (uint32_t)(k * NB + col));
+                c[u] = k0 == 0 ? c0[u] : gclk[k * LS];
+                l[u] = UNIF ? lu : lat_at(lat_mg + (uint32_t)(k * NB + col));
             }
             if (k0 == 0) {
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    c0[u] = c[u];
-                    l0[u] = l[u];
-                }
+                for (int u = 0; u < 4; ++u) l0[u] = l[u];
             }
 #pragma unroll
             for (int u = 1; u < 4; ++u)
@@ -389,6 +417,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         const uint32_t g = desc_group(d);
         const int stages = (int)desc_stages_m1(d) + 1;
         double *gclk = clk + (desc_last_slot(d) - desc_stages_m1(d)) * LS;
+        // COOP: the clocks of the group's first four stages (the same for every queue tried below)
+        double c0[4] = {0.0, 0.0, 0.0, 0.0};
+        if constexpr (COOP) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) c0[u] = gclk[(u < stages ? u : stages - 1) * LS];
+        }
         for (;;) {
             const uint32_t lat_mg = ((uint32_t)m * (uint32_t)a.lat_row + desc_lat_off(d)) * (uint32_t)NB;  // the (model, group) rows of the table
             const int64_t base = mq_off[m];
@@ -410,7 +444,6 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             int2 ir = {0, 0};
             int32_t rank8 = 0;
             int kfirst = 0;
-            double c0[4] = {0.0, 0.0, 0.0, 0.0};
             float l0[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             if constexpr (COOP) {
                 // lane j of the octet takes entry j from the head of the queue on -- all of it, whether it has arrived
@@ -419,8 +452,11 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 hv = *reinterpret_cast<const double2 *>(ep);
                 ir = *reinterpret_cast<const int2 *>(&ep->idx);
                 rank8 = ep[8].rank;
-                const double tcol = batch_time_col(t0, gclk, stages, lat_mg, oj < NB ? oj : NB - 1, c0, l0);
-                const double alone = oct_get(tcol, 0) + overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
+                const int mycol = oj < NB ? oj : NB - 1;
+                float lu = 0.0f;
+                if constexpr (UNIF) lu = lat_at(lat_mg + (uint32_t)mycol);
+                const double tcol = batch_time_col(t0, gclk, stages, lat_mg, mycol, c0, lu, l0);
+                const double alone = oct_first(tcol) + overhead;  // check_slo(..., batch size 1, deadline) == (alone <= deadline)
                 for (;;) {
                     const uint32_t pass = oct_ballot(oj < avail && alone <= hv.y);
                     const int k = pass ? __ffs((int)pass) - 1 : avail;  // the heads before k are dropped
@@ -534,6 +570,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             }
             double t = t0 + overhead;
             double idle_at = 0.0;
+            float lu = 0.0f;  // UNIF: the latency of every stage at this batch size
+            if constexpr (UNIF && COOP) {
+                lu = oct_get(l0[0], col);
+            } else if constexpr (UNIF) {
+                lu = lat_at(lat_mg + (uint32_t)col);
+            }
             for (int k0 = 0; k0 < stages; k0 += 4) {
                 double c[4];
                 float l[4];
@@ -541,14 +583,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
                         c[u] = c0[u];
-                        l[u] = oct_get(l0[u], col);
+                        l[u] = UNIF ? lu : oct_get(l0[u], col);
                     }
                 } else {
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
                         const int k = k0 + u < stages ? k0 + u : stages - 1;
                         c[u] = gclk[k * LS];
-                        l[u] = lat_at(lat_mg + (uint32_t)(k * NB + col));
+                        l[u] = UNIF ? lu : lat_at(lat_mg + (uint32_t)(k * NB + col));
                     }
                 }
                 if constexpr (OCT) oct_sync();
@@ -614,11 +656,18 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                 return;
             }
             nfree -= 1;
-            const int slot = fstack[nfree * LS];
+            int slot;
+            if constexpr (SH) {
+                slot = __ffsll((long long)~used) - 1;  // the lowest free slot: events gather in the first chunks
+                used |= 1ull << slot;
+                if (oj == (slot >> 3)) my_cm = fmin(my_cm, idle_at);
+            } else {
+                slot = fstack[nfree * LS];
+                double *cm = cm_t + (slot >> 3) * LS;
+                *cm = fmin(*cm, idle_at);
+            }
             ev_t[slot * LS] = idle_at;
             ev_g[slot * LS] = d;  // the descriptor, not the index: it orders like the index and saves the look-up when the event is due
-            double *cm = cm_t + (slot >> 3) * LS;
-            *cm = fmin(*cm, idle_at);
             next_due = fmin(next_due, idle_at);
             return;
         }
@@ -630,6 +679,14 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         T = __builtin_inf();
         others = __builtin_inf();
         cj = 0;
+        if constexpr (SH) {  // at most eight chunks, their minima in the octet's registers
+            const double mn = oct_min(my_cm);
+            const int first = __ffs((int)oct_ballot(my_cm == mn)) - 1;
+            others = oct_min(oj == first ? __builtin_inf() : my_cm);
+            T = mn;
+            cj = first;
+            return;
+        }
         if constexpr (OCT) {
             for (int c0 = 0; c0 < nch; c0 += 8) {  // one chunk minimum per lane
                 const double v = cm_t[(c0 + oj) * LS];
@@ -669,8 +726,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         int be = cj << 3;
         if (others == T) {
             // several chunks hold an event at time T: the smallest group among all of them (rare)
+            const uint32_t tied = SH ? oct_ballot(my_cm == T) : 0u;
             for (int c = 0; c < nch; ++c) {
-                if (cm_t[c * LS] != T) continue;
+                if (SH ? !((tied >> c) & 1u) : cm_t[c * LS] != T) continue;
                 for (int u = 0; u < 8; ++u) {
                     const int e = (c << 3) + u;
                     const uint32_t g = ev_g[e * LS];
@@ -694,8 +752,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             const double left = oct_min(e == be ? __builtin_inf() : t);  // earliest time left in the chunk
             ev_t[be * LS] = __builtin_inf();
             ev_g[be * LS] = 0xFFFFFFFFu;
-            cm_t[cj * LS] = left;
-            fstack[nfree * LS] = (uint16_t)be;
+            if constexpr (SH) {
+                if (oj == cj) my_cm = left;
+                used &= ~(1ull << be);
+            } else {
+                cm_t[cj * LS] = left;
+                fstack[nfree * LS] = (uint16_t)be;
+            }
             nfree += 1;
             next_due = left < others ? left : others;
             return bg;
@@ -734,7 +797,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             const int64_t at = i + lane < R ? i + lane : R - 1;
             blk_req = reqs[at];
             const int m0 = __builtin_amdgcn_readlane(blk_req.m, 0);
-            g8_next = rep_tile[(size_t)(m0 < 0 ? 0 : m0) * kWave];
+            g8_next = row_of(m0);
         }
         const double tstamp = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(blk_req.t), j),
                                                __builtin_amdgcn_readlane(__double2loint(blk_req.t), j));
@@ -743,7 +806,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         const uint64_t g8 = g8_next;
         if (j != kWave - 1) {  // the first request of a block gets its list when the block is fetched
             const int mn = __builtin_amdgcn_readlane(blk_req.m, j + 1);
-            g8_next = rep_tile[(size_t)(mn < 0 ? 0 : mn) * kWave];
+            g8_next = row_of(mn);
         }
 
         // ---- idle events that are due (:739-744)
@@ -767,25 +830,75 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         // ---- the arrival (:746-778)
         bool queued = false;
         uint32_t gsel = none;
+        if constexpr (OCT) {
+            // One replica per lane: the lane's word is the descriptor of that replica's group.  The clocks of its
+            // last and of its first stage and the model's arrival count are read together; the first of the smallest
+            // last-stage clocks wins, as in a scan with "<" (:760-770), and whether that group is idle (:776) is one
+            // bit of a ballot over the first-stage clocks.
+            const uint32_t dj = (uint32_t)g8;
+            const bool valid = (int32_t)dj >= 0 && m >= 0;
+            const uint32_t last = desc_last_slot(dj);
+            const double c = clk[last * LS];                             // slot 0 for a lane without a replica: not used
+            const double cf = clk[(last - desc_stages_m1(dj)) * LS];
+            uint32_t seen = 0;
+            if (m >= 0) seen = arrived[m];
+            const uint32_t vb = oct_ballot(valid);
+            uint32_t dsel = kEmpty;  // the chosen group's descriptor, once it is needed
+            int selj = -1;           // the lane of the octet whose replica was chosen
+            bool ready = false;
+            if ((vb & 1u) && !dead) {
+                double best = 1e100;
+                const double mn = oct_min(valid ? c : __builtin_inf());
+                if (mn < best) {
+                    best = mn;
+                    selj = __ffs((int)oct_ballot(valid && c == mn)) - 1;
+                    ready = ((oct_ballot(tstamp >= cf) >> selj) & 1u) != 0;
+                }
+                if (vb >> 7)  // the list may go on
+                    for (int x = 0; x < a.rep_extra; ++x) {
+                        const uint32_t g = repx_tile[((size_t)m * a.rep_extra + x) * kWave];
+                        if (g == none) break;
+                        const uint32_t d2 = ginfo[g * LS];
+                        const double c2 = clk[desc_last_slot(d2) * LS];
+                        if (c2 < best) {
+                            best = c2;
+                            selj = -1;
+                            dsel = d2;
+                            ready = tstamp >= clk[(desc_last_slot(d2) - desc_stages_m1(d2)) * LS];
+                        }
+                    }
+                queued = true;
+            }
+            if (m >= 0) {
+                // every lane sees the same arrival count and writes the same count + 1; lanes that do not host m never
+                // read it (a wavefront's LDS accesses are carried out in program order)
+                __builtin_amdgcn_wave_barrier();
+                arrived[m] = seen + 1u;
+                __builtin_amdgcn_wave_barrier();
+            }
+            if (!queued) {
+                if (want_req && !dead) {
+                    fin_out[(size_t)i * kWave] = tstamp;
+                    good_out[(size_t)i * kWave] = 0;
+                }
+            } else if (selj < 0 && dsel == kEmpty) {
+                // every replica's clock is infinite (only after a batch with infinite latency was accepted under an
+                // infinite SLO): the reference's g_id stays -1 here, which its arrays take as "the last group"
+                // (controller.py:760-778); that accident is not reproduced
+                dead = MMSIM_E_UNSUPPORTED;
+            } else if (ready) {  // :776-778
+                if (selj >= 0) dsel = oct_get(dj, selj);
+                handle(tstamp, m, dsel);
+            }
+            continue;
+        }
         if (m >= 0) {
             const bool hosted = (uint32_t)(g8 & 0xFFu) != none;
             if (hosted && !dead) {
                 // group with the strictly smallest last-stage clock (:760-770)
                 double best = 1e100;
                 bool more = true;  // the list may go on
-                if constexpr (OCT) {
-                    // one replica per lane; the first of the smallest clocks wins, as in a scan with "<"
-                    const uint32_t g = (uint32_t)(g8 >> (8 * oj)) & 0xFFu;
-                    const double c = clk[desc_last_slot(ginfo[g * LS]) * LS];  // the empty row for unused bytes
-                    const double mn = oct_min(g != none ? c : __builtin_inf());
-                    if (mn < best) {
-                        best = mn;
-                        const int first = __ffs((int)oct_ballot(g != none && c == mn)) - 1;
-                        gsel = (uint32_t)(g8 >> (8 * first)) & 0xFFu;
-                    }
-                    more = ((uint32_t)(g8 >> 56) & 0xFFu) != none;
-                }
-                for (int j0 = 0; !OCT && j0 < kPackedReplicas && more; j0 += 4) {  // four replicas at a time: their reads overlap
+                for (int j0 = 0; j0 < kPackedReplicas && more; j0 += 4) {  // four replicas at a time: their reads overlap
                     uint32_t g[4], d[4];
                     double c[4];
 #pragma unroll
@@ -868,12 +981,14 @@ hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_byt
         e = hipErrorInvalidValue;
     } else {
         const bool ll = args.lat_lds_bytes > 0, gl = args.g2m_in_lds != 0;
-        const bool oct = args.lane_stride == 8;
+        const bool oct = args.lane_stride == 8, unif = args.uniform_stages != 0;
+        const bool small_heap = oct && args.heap_cap <= 64;
         void (*kern)(const BatchingArgs) = nullptr;
-#define MMSIM_PICK2(NBT, O)                                                                         \
-    (ll ? (gl ? sim_batching_kernel<NBT, true, true, O> : sim_batching_kernel<NBT, true, false, O>) \
-        : (gl ? sim_batching_kernel<NBT, false, true, O> : sim_batching_kernel<NBT, false, false, O>))
-#define MMSIM_PICK(NBT) kern = oct ? MMSIM_PICK2(NBT, true) : MMSIM_PICK2(NBT, false)
+#define MMSIM_PICK4(NBT, O, U, S)                                                                               \
+    (ll ? (gl ? sim_batching_kernel<NBT, true, true, O, U, S> : sim_batching_kernel<NBT, true, false, O, U, S>) \
+        : (gl ? sim_batching_kernel<NBT, false, true, O, U, S> : sim_batching_kernel<NBT, false, false, O, U, S>))
+#define MMSIM_PICK3(NBT, O, S) (unif ? MMSIM_PICK4(NBT, O, true, S) : MMSIM_PICK4(NBT, O, false, S))
+#define MMSIM_PICK(NBT) kern = !oct ? MMSIM_PICK3(NBT, false, false) : small_heap ? MMSIM_PICK3(NBT, true, true) : MMSIM_PICK3(NBT, true, false)
         if (args.NB <= 4)
             MMSIM_PICK(4);
         else if (args.NB <= 8)
@@ -881,7 +996,8 @@ hipError_t launch_sim_batching(const BatchingArgs &args, int wpb, size_t lds_byt
         else
             MMSIM_PICK(16);
 #undef MMSIM_PICK
-#undef MMSIM_PICK2
+#undef MMSIM_PICK3
+#undef MMSIM_PICK4
         if (lds_bytes > 64 * 1024)
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)lds_bytes);
@@ -900,7 +1016,8 @@ std::string sim_batching_kernel_name(const BatchingArgs &args) {
     const int nbt = args.NB <= 4 ? 4 : args.NB <= 8 ? 8 : 16;
     auto tf = [](bool v) { return v ? "true" : "false"; };
     return "sim_batching_kernel<" + std::to_string(nbt) + ", " + tf(args.lat_lds_bytes > 0) + ", " + tf(args.g2m_in_lds != 0) +
-           ", " + tf(args.lane_stride == 8) + ">";
+           ", " + tf(args.lane_stride == 8) + ", " + tf(args.uniform_stages != 0) + ", " +
+           tf(args.lane_stride == 8 && args.heap_cap <= 64) + ">";
 }
 
 }  // namespace mmsim
