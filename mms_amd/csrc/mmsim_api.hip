@@ -607,8 +607,10 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         // of eight (the kernel keeps them in chunks of eight).
         auto bytes_for = [&](int lanes, int slots) {
             const size_t nch8 = (size_t)((slots / 8 + 7) & ~7);
-            return ((size_t)(Gmax + 1) * lanes * 4 + (size_t)nslots * lanes * 8 + (size_t)2 * M * lanes * 4 +
-                    (size_t)slots * lanes * (8 + 4 + 2) + nch8 * lanes * 8 +
+            // (octet tiles with at most 64 event slots keep the free slots and the chunk minima in registers)
+            const bool in_regs = lanes == 8 && slots <= 64;
+            return ((lanes == 8 ? 0 : (size_t)(Gmax + 1) * lanes * 4) + (size_t)nslots * lanes * 8 + (size_t)2 * M * lanes * 4 +
+                    (size_t)slots * lanes * (8 + 4 + (in_regs ? 0 : 2)) + (in_regs ? 0 : nch8 * lanes * 8) +
                     (((size_t)M * 4 + 15) & ~(size_t)15) + (((size_t)(M + 1) * 8 + 15) & ~(size_t)15) +
                     (((size_t)t->NB * 4 + 15) & ~(size_t)15) + 15) & ~(size_t)15;
         };

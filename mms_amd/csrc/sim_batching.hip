@@ -182,22 +182,24 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         for (int i = (int)threadIdx.x; i < n; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
     }
     unsigned char *mine = lds_raw + a.lat_lds_bytes + wv * a.wave_lds_bytes;
+    // (octet tiles get a group's descriptor with the replica lists and keep no copy of the table: the replicas past
+    // the eighth of a model, rare, are looked up in global memory)
     uint32_t *ginfo = reinterpret_cast<uint32_t *>(mine) + sl;
-    size_t o = (size_t)(Gmax + 1) * LS * 4;
+    size_t o = OCT ? 0 : (size_t)(Gmax + 1) * LS * 4;
     double *clk = reinterpret_cast<double *>(mine + o) + sl;
     o += (size_t)a.nslots * LS * 8;
     double *ev_t = reinterpret_cast<double *>(mine + o) + sl;
     o += (size_t)a.heap_cap * LS * 8;
-    double *cm_t = reinterpret_cast<double *>(mine + o) + sl;  // earliest event time of each chunk
-    o += (size_t)nch8 * LS * 8;
+    double *cm_t = reinterpret_cast<double *>(mine + o) + sl;  // earliest event time of each chunk (not with SH)
+    if constexpr (!SH) o += (size_t)nch8 * LS * 8;
     uint32_t *head = reinterpret_cast<uint32_t *>(mine + o) + sl;
     o += (size_t)M * LS * 4;
     int32_t *hrank = reinterpret_cast<int32_t *>(mine + o) + sl;  // rank of the arrival at head[m] (already known before it arrives)
     o += (size_t)M * LS * 4;
     uint32_t *ev_g = reinterpret_cast<uint32_t *>(mine + o) + sl;
     o += (size_t)a.heap_cap * LS * 4;
-    uint16_t *fstack = reinterpret_cast<uint16_t *>(mine + o) + sl;  // free event slots, the next one to use on top
-    o += (size_t)a.heap_cap * LS * 2;
+    uint16_t *fstack = reinterpret_cast<uint16_t *>(mine + o) + sl;  // free event slots, the next one to use on top (not with SH)
+    if constexpr (!SH) o += (size_t)a.heap_cap * LS * 2;
     // [M], same for all lanes; written by lane 0 and read by all, hence volatile (and spelled as an LDS
     // pointer: volatile accesses are not rewritten from generic to LDS by the compiler)
     lds_vu32 *arrived = as_lds_vu32(mine + o);
@@ -217,14 +219,16 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     const bool sim = sl < LS;  // the other lanes of a narrow tile only help fetching requests
     if (live && sim) {
         const uint32_t *gsrc = a.ginfo + (size_t)tile * (Gmax + 1) * kWave + sl;
-        for (int g = 0; g <= Gmax; ++g) ginfo[g * LS] = gsrc[g * kWave];
+        if constexpr (!OCT)
+            for (int g = 0; g <= Gmax; ++g) ginfo[g * LS] = gsrc[g * kWave];
         for (int s = 0; s < a.nslots; ++s) clk[s * LS] = 0.0;
         for (int e = 0; e < a.heap_cap; ++e) {  // free event slots never win a minimum scan
             ev_t[e * LS] = __builtin_inf();
             ev_g[e * LS] = 0xFFFFFFFFu;
-            fstack[e * LS] = (uint16_t)(a.heap_cap - 1 - e);  // slot 0 is used first, so events gather in the first chunks
+            if constexpr (!SH) fstack[e * LS] = (uint16_t)(a.heap_cap - 1 - e);  // slot 0 is used first, so events gather in the first chunks
         }
-        for (int c = 0; c < nch8; ++c) cm_t[c * LS] = __builtin_inf();
+        if constexpr (!SH)
+            for (int c = 0; c < nch8; ++c) cm_t[c * LS] = __builtin_inf();
         {
             const int64_t *mo = a.mq_off + (size_t)seed * (M + 1);
             for (int m = lane; m <= M; m += fill) mq_off[m] = mo[m];
@@ -679,12 +683,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         T = __builtin_inf();
         others = __builtin_inf();
         cj = 0;
-        if constexpr (SH) {  // at most eight chunks, their minima in the octet's registers
-            const double mn = oct_min(my_cm);
-            const int first = __ffs((int)oct_ballot(my_cm == mn)) - 1;
-            others = oct_min(oj == first ? __builtin_inf() : my_cm);
-            T = mn;
-            cj = first;
+        if constexpr (SH) {
+            // at most eight chunks, their minima in the octet's registers; the earliest time of all is next_due, which
+            // is kept exact.  The earliest of the other chunks is left to pop_event, which computes it while it waits
+            // for the chunk's slots.
+            T = next_due;
+            cj = __ffs((int)oct_ballot(my_cm == T)) - 1;  // -1: there is no event (T is +inf, and so are the minima: 0)
+            cj = cj < 0 ? 0 : cj;
             return;
         }
         if constexpr (OCT) {
@@ -721,14 +726,51 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
     // removes the lexicographically smallest (time, group) event, whose time T and chunk cj chunk_scan
     // found (others as returned by it); returns its word (the group's descriptor, which orders like the group's
     // index) and sets next_due to the earliest time left
+    // SH: the same in one piece, for the time T and chunk cj that chunk_scan gave
+    auto pop_event = [&](double T, int cj) -> uint32_t {
+        uint32_t bg = 0xFFFFFFFFu;
+        int be = cj << 3;
+        const uint32_t tied = oct_ballot(my_cm == T);
+        const bool tie = (tied & (tied - 1u)) != 0;
+        if (tie) {  // several chunks hold an event at time T: the smallest group among all of them (rare)
+            for (int c = 0; c < nch; ++c) {
+                if (!((tied >> c) & 1u)) continue;
+                for (int u = 0; u < 8; ++u) {
+                    const int e = (c << 3) + u;
+                    const uint32_t g = ev_g[e * LS];
+                    if (ev_t[e * LS] == T && g < bg) {
+                        bg = g;
+                        be = e;
+                    }
+                }
+            }
+            cj = be >> 3;
+        }
+        const int e = (cj << 3) + oj;  // one slot of the chunk per lane
+        const double t = ev_t[e * LS];
+        const uint32_t g = ev_g[e * LS];
+        const double others = oct_min(oj == cj ? __builtin_inf() : my_cm);  // (with a tie: T again, whichever chunk was taken)
+        if (!tie) {
+            bg = oct_min(t == T ? g : 0xFFFFFFFFu);
+            be = (cj << 3) + __ffs((int)oct_ballot(t == T && g == bg)) - 1;
+        }
+        const double left = oct_min(e == be ? __builtin_inf() : t);  // earliest time left in the chunk
+        ev_t[be * LS] = __builtin_inf();
+        ev_g[be * LS] = 0xFFFFFFFFu;
+        if (oj == cj) my_cm = left;
+        used &= ~(1ull << be);
+        nfree += 1;
+        next_due = left < others ? left : others;
+        return bg;
+    };
     auto take_event = [&](double T, int cj, double others) -> uint32_t {
+        if constexpr (SH) return pop_event(T, cj);
         uint32_t bg = 0xFFFFFFFFu;
         int be = cj << 3;
         if (others == T) {
             // several chunks hold an event at time T: the smallest group among all of them (rare)
-            const uint32_t tied = SH ? oct_ballot(my_cm == T) : 0u;
             for (int c = 0; c < nch; ++c) {
-                if (SH ? !((tied >> c) & 1u) : cm_t[c * LS] != T) continue;
+                if (cm_t[c * LS] != T) continue;
                 for (int u = 0; u < 8; ++u) {
                     const int e = (c << 3) + u;
                     const uint32_t g = ev_g[e * LS];
@@ -752,13 +794,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             const double left = oct_min(e == be ? __builtin_inf() : t);  // earliest time left in the chunk
             ev_t[be * LS] = __builtin_inf();
             ev_g[be * LS] = 0xFFFFFFFFu;
-            if constexpr (SH) {
-                if (oj == cj) my_cm = left;
-                used &= ~(1ull << be);
-            } else {
-                cm_t[cj * LS] = left;
-                fstack[nfree * LS] = (uint16_t)be;
-            }
+            cm_t[cj * LS] = left;
+            fstack[nfree * LS] = (uint16_t)be;
             nfree += 1;
             next_due = left < others ? left : others;
             return bg;
@@ -790,15 +827,15 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
         return bg;
     };
 
-    for (int64_t i = 0; i < R; ++i) {
-        // requests are fetched 64 at a time (one coalesced load) and handed out lane by lane
-        const int j = (int)(i & (kWave - 1));
-        if (j == 0) {
-            const int64_t at = i + lane < R ? i + lane : R - 1;
-            blk_req = reqs[at];
-            const int m0 = __builtin_amdgcn_readlane(blk_req.m, 0);
-            g8_next = row_of(m0);
-        }
+    for (int64_t i0 = 0; i0 < R; i0 += kWave) {
+    {
+        const int64_t at = i0 + lane < R ? i0 + lane : R - 1;
+        blk_req = reqs[at];
+        g8_next = row_of(__builtin_amdgcn_readlane(blk_req.m, 0));
+    }
+    const int nj = R - i0 < kWave ? (int)(R - i0) : kWave;
+    for (int j = 0; j < nj; ++j) {
+        const int64_t i = i0 + j;
         const double tstamp = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(blk_req.t), j),
                                                __builtin_amdgcn_readlane(__double2loint(blk_req.t), j));
         const int m = __builtin_amdgcn_readlane(blk_req.m, j);
@@ -858,7 +895,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
                     for (int x = 0; x < a.rep_extra; ++x) {
                         const uint32_t g = repx_tile[((size_t)m * a.rep_extra + x) * kWave];
                         if (g == none) break;
-                        const uint32_t d2 = ginfo[g * LS];
+                        const uint32_t d2 = a.ginfo[((size_t)tile * (Gmax + 1) + g) * kWave + sl];
                         const double c2 = clk[desc_last_slot(d2) * LS];
                         if (c2 < best) {
                             best = c2;
@@ -951,6 +988,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlockBatching *kWave) void sim_batching
             const double idle_since = clk[(desc_last_slot(d) - desc_stages_m1(d)) * LS];
             if (tstamp >= idle_since) handle(tstamp, m, d);  // :776-778
         }
+    }
     }
     // ---- drain (:781-787)
     while (!dead && nfree < a.heap_cap) {
