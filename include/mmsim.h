@@ -106,7 +106,7 @@ typedef struct {
                                      that still gives a CU eight wavefronts                                    */
     int32_t batching_event_slots; /* batching simulator: idle-event slots per simulation (a multiple of eight);
                                      0: from the group count.  Too few makes a simulation stop with
-                                     MMSIM_E_OVERFLOW                                                           */
+                                     MMSIM_E_OVERFLOW (the one-call entry points then try again with more)     */
     int32_t batching_lds_tables;  /* batching simulator: bit 0 latency table, bit 1 models of each group may be
                                      copied to LDS; -1: both, subject to fit                                    */
     int32_t reserved;
@@ -347,7 +347,12 @@ int mmsim_batch_get_info(const mmsim_batch *batch, mmsim_batch_info *out);
  * (e.g. "sim_mixed_kernel<16, true, true, true, 0, true>"); measurement aid, no counterpart in the reference. */
 int mmsim_batch_kernel_name(const mmsim_batch *batch, char *buf, size_t size);
 
-/* create + run + sync + fetch + destroy */
+/* create + run + sync + fetch + destroy.  With MMSIM_BATCHING, a simulation that runs out of idle-event slots
+ * (status MMSIM_E_OVERFLOW: the reference's heap of idle events has no bound, the kernel's list of them has) is
+ * simulated again inside this call with twice the slots, until it fits or LDS cannot hold more; only then does it
+ * keep that status.  mmsim_eval_successors and mmsim_simulate_requests_mixed_batching do the same; a batch
+ * (mmsim_batch_fetch) and mmsim_eval_pairs report the status and leave the choice to the caller
+ * (mmsim_options.batching_event_slots). */
 int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
                      const mmsim_tables *tables, const mmsim_placements *placements,
                      uint32_t flags, mmsim_result *out);

@@ -1735,17 +1735,112 @@ int mmsim_batch_kernel_name(const mmsim_batch *b, char *buf, size_t size) {
     return MMSIM_OK;
 }
 
-int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
-                     const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
-                     mmsim_result *out) {
-    if (!out) return fail(MMSIM_E_INVALID, "eval_batch: out is null");
+namespace {
+
+// One-call evaluation with the given options (nullptr: the context's).  event_slots (optional) receives the event
+// slots per simulation that the batching simulator was given.
+int eval_once(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds, const mmsim_tables *tables,
+              const mmsim_placements *placements, uint32_t flags, const mmsim_options *options, mmsim_result *out,
+              int *event_slots) {
     mmsim_batch *b = nullptr;
-    int rc = mmsim_batch_create(ctx, workloads, n_seeds, tables, placements, flags, &b);
+    int rc = mmsim_batch_create_ex(ctx, workloads, n_seeds, tables, placements, flags, options, &b);
+    if (rc == MMSIM_OK && event_slots) *event_slots = b->bargs.heap_cap;
     if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
     if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
     if (rc == MMSIM_OK) rc = mmsim_batch_fetch(b, out);
     mmsim_batch_destroy(b);
     return rc;
+}
+
+}  // namespace
+
+int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                     const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
+                     mmsim_result *out) {
+    if (!out) return fail(MMSIM_E_INVALID, "eval_batch: out is null");
+    // The batching simulator gives every simulation a fixed number of idle-event slots (what the reference's heap
+    // is seen to need, and what fits in LDS); a simulation that needs more stops with MMSIM_E_OVERFLOW.  Those are
+    // simulated again here, alone and with twice the slots, until they fit or LDS says no (they then keep that status).
+    std::vector<int32_t> own_status;
+    mmsim_result res = *out;
+    const bool watch = (flags & MMSIM_BATCHING) != 0 && placements && n_seeds > 0 && placements->B > 0;
+    if (watch && !res.status) {
+        own_status.assign((size_t)n_seeds * placements->B, 0);
+        res.status = own_status.data();
+    }
+    int slots = 0;
+    int rc = eval_once(ctx, workloads, n_seeds, tables, placements, flags, nullptr, &res, &slots);
+    if (rc != MMSIM_OK || !watch) return rc;
+    const int32_t B = placements->B, Gmax = placements->Gmax, M = tables->M;
+    const size_t G1 = (size_t)Gmax + 1;
+    int64_t Rmax = 0;
+    for (int s = 0; s < n_seeds; ++s) Rmax = std::max(Rmax, workloads[s]->R);
+    for (int round = 0; round < 8; ++round) {
+        std::vector<int32_t> again;
+        for (int32_t p = 0; p < B; ++p)
+            for (int s = 0; s < n_seeds; ++s)
+                if (res.status[(size_t)s * B + p] == MMSIM_E_OVERFLOW) {
+                    again.push_back(p);
+                    break;
+                }
+        if (again.empty()) break;
+        slots *= 2;
+        const int32_t B2 = (int32_t)again.size();
+        std::vector<int32_t> ng(B2), gc((size_t)B2 * Gmax), idx;
+        std::vector<int64_t> off((size_t)B2 * G1);
+        for (int32_t k = 0; k < B2; ++k) {
+            const int32_t p = again[k];
+            ng[k] = placements->num_groups[p];
+            std::copy(placements->group_cfg + (size_t)p * Gmax, placements->group_cfg + (size_t)(p + 1) * Gmax, gc.begin() + (size_t)k * Gmax);
+            for (size_t g = 0; g < G1; ++g) {
+                const int64_t lo = placements->gm_off[(size_t)p * G1 + g];
+                off[(size_t)k * G1 + g] = (int64_t)idx.size();
+                if (g < (size_t)ng[k]) idx.insert(idx.end(), placements->gm_idx + lo, placements->gm_idx + placements->gm_off[(size_t)p * G1 + g + 1]);
+            }
+        }
+        if (idx.empty()) idx.push_back(0);
+        const mmsim_placements sub = {B2, Gmax, ng.data(), gc.data(), off.data(), idx.data()};
+        const size_t L2 = (size_t)n_seeds * B2;
+        std::vector<int64_t> n_good(L2);
+        std::vector<double> lat_sum(L2), finish;
+        std::vector<int32_t> mreq, mgood, greq, ggood, status(L2);
+        std::vector<uint8_t> good;
+        mmsim_result r2{};
+        r2.n_good = n_good.data();
+        r2.latency_sum = lat_sum.data();
+        r2.status = status.data();
+        if (flags & MMSIM_WANT_MODEL_COUNTS) {
+            mreq.resize(L2 * M), mgood.resize(L2 * M);
+            r2.model_num_requests = mreq.data(), r2.model_num_good = mgood.data();
+        }
+        if (flags & MMSIM_WANT_GROUP_COUNTS) {
+            greq.resize(L2 * Gmax), ggood.resize(L2 * Gmax);
+            r2.group_num_requests = greq.data(), r2.group_num_good = ggood.data();
+        }
+        if ((flags & MMSIM_WANT_PER_REQUEST) && res.finish && res.good) {
+            finish.resize(L2 * (size_t)Rmax), good.resize(L2 * (size_t)Rmax);
+            r2.finish = finish.data(), r2.good = good.data();
+        }
+        mmsim_options o = ctx->opt;
+        o.batching_event_slots = slots;
+        if (eval_once(ctx, workloads, n_seeds, tables, &sub, flags, &o, &r2, nullptr) != MMSIM_OK) break;  // (does not fit in LDS)
+        for (int32_t k = 0; k < B2; ++k)
+            for (int s = 0; s < n_seeds; ++s) {
+                const size_t src = (size_t)s * B2 + k, dst = (size_t)s * B + again[k];
+                if (res.n_good) res.n_good[dst] = n_good[src];
+                if (res.latency_sum) res.latency_sum[dst] = lat_sum[src];
+                res.status[dst] = status[src];
+                if (r2.model_num_requests && res.model_num_requests) std::copy(&mreq[src * M], &mreq[(src + 1) * M], res.model_num_requests + dst * M);
+                if (r2.model_num_good && res.model_num_good) std::copy(&mgood[src * M], &mgood[(src + 1) * M], res.model_num_good + dst * M);
+                if (r2.group_num_requests && res.group_num_requests) std::copy(&greq[src * Gmax], &greq[(src + 1) * Gmax], res.group_num_requests + dst * Gmax);
+                if (r2.group_num_good && res.group_num_good) std::copy(&ggood[src * Gmax], &ggood[(src + 1) * Gmax], res.group_num_good + dst * Gmax);
+                if (r2.finish) {
+                    std::copy(&finish[src * (size_t)Rmax], &finish[(src + 1) * (size_t)Rmax], res.finish + dst * (size_t)Rmax);
+                    std::copy(&good[src * (size_t)Rmax], &good[(src + 1) * (size_t)Rmax], res.good + dst * (size_t)Rmax);
+                }
+            }
+    }
+    return MMSIM_OK;
 }
 
 int mmsim_eval_successors(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
@@ -2019,27 +2114,33 @@ int mmsim_simulate_requests_mixed_batching(mmsim_ctx *ctx, double *finish, uint8
     mmsim_workload *wl = nullptr;
     rc = mmsim_workload_create(ctx, num_requests, M, tstamps, model_ids, slos, &wl);
     if (rc) return rc;
-    mmsim_batch *b = nullptr;
     const mmsim_workload *wls[1] = {wl};
     const uint32_t flags = MMSIM_BATCHING | MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS | MMSIM_WANT_PER_REQUEST;
-    rc = build_batch(ctx, wls, 1, &t, rl, flags, &b);
-    if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
-    if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
-    if (rc == MMSIM_OK) {
-        int64_t ng = 0;
-        double ls = 0.0;
-        mmsim_result r{};
-        r.n_good = &ng;
-        r.latency_sum = &ls;
-        r.model_num_requests = model_num_requests;
-        r.model_num_good = model_num_good_requests;
-        r.group_num_requests = group_num_requests;
-        r.group_num_good = group_num_good_requests;
-        r.finish = finish;
-        r.good = good;
-        rc = mmsim_batch_fetch(b, &r);
+    // (a simulation that runs out of idle-event slots is run again with twice as many, as in mmsim_eval_batch)
+    mmsim_options o = ctx->opt;
+    for (int attempt = 0; attempt < 8; ++attempt) {
+        mmsim_batch *b = nullptr;
+        rc = build_batch(ctx, wls, 1, &t, rl, flags, &b, nullptr, &o);
+        if (rc == MMSIM_OK) o.batching_event_slots = 2 * b->bargs.heap_cap;
+        if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
+        if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
+        if (rc == MMSIM_OK) {
+            int64_t ng = 0;
+            double ls = 0.0;
+            mmsim_result r{};
+            r.n_good = &ng;
+            r.latency_sum = &ls;
+            r.model_num_requests = model_num_requests;
+            r.model_num_good = model_num_good_requests;
+            r.group_num_requests = group_num_requests;
+            r.group_num_good = group_num_good_requests;
+            r.finish = finish;
+            r.good = good;
+            rc = mmsim_batch_fetch(b, &r);
+        }
+        mmsim_batch_destroy(b);
+        if (rc != MMSIM_E_OVERFLOW) break;
     }
-    mmsim_batch_destroy(b);
     mmsim_workload_destroy(wl);
     return rc;
 }

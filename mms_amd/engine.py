@@ -393,18 +393,10 @@ class Batch:
 
 def evaluate(engine: Engine, workloads: Sequence[DeviceWorkload], table: LatencyTable, sols: Sequence,
              flags: int = 0, fixed_overhead: float = FIXED_OVERHEAD):
-    """One-shot: pack, upload, simulate, fetch.  Result arrays are [n_seeds][B][...]."""
-    packed = pack_placements(sols, table)
-    batch = Batch(engine, workloads, table, packed, flags, fixed_overhead)
-    try:
-        batch.run()
-        ms = batch.sync()
-        out = batch.fetch()
-        out["kernel_ms"] = ms
-        out["info"] = batch.info()
-    finally:
-        batch.close()
-    return out
+    """One-shot: pack, upload, simulate, fetch (one call of ``mmsim_eval_batch``).  Result arrays are
+    [n_seeds][B][...].  A batching simulation that runs out of idle-event slots is simulated again with more
+    inside that call; ``Batch`` reports it in ``status`` instead."""
+    return eval_batch(engine, workloads, table, pack_placements(sols, table), flags, fixed_overhead)
 
 
 def simulate_requests_mixed(engine: Engine, finish, good, tstamps, model_ids, slos, m_id2g_id,

@@ -44,7 +44,7 @@ def _evaluate(engine, workloads, table, sols, flags=0, fixed_overhead=0.011):
             want_counts=True, want_per_request=bool(flags & _lib.WANT_PER_REQUEST)))
     res = {"n_good": np.stack([o["n_good"] for o in outs]),
            "latency_sum": np.stack([o["latency_sum"] for o in outs]),
-           "status": np.zeros((len(outs), len(sols)), np.int32), "kernel_ms": 0.0, "info": {}}
+           "status": np.zeros((len(outs), len(sols)), np.int32)}
     for k in ("model_num_requests", "model_num_good", "group_num_requests", "group_num_good"):
         res[k] = np.stack([o[k] for o in outs])
     if flags & _lib.WANT_PER_REQUEST:

@@ -153,16 +153,49 @@ def test_many_groups_many_pending_events(eng, opts, lanes):
 
 
 @pytest.mark.parametrize("lanes", [8, 16])
-def test_a_simulation_that_runs_out_of_event_slots_is_reported(eng, opts, lanes):
-    """With fewer event slots than busy groups the simulation stops and the call fails with MMSIM_E_OVERFLOW
-    instead of returning numbers (the slots are provisioned from the group count; here they are forced down)."""
+def test_a_simulation_that_runs_out_of_event_slots(eng, opts, lanes):
+    """With fewer event slots than the reference's heap holds entries a simulation stops with MMSIM_E_OVERFLOW (the
+    slots are provisioned from the group count; here they are forced down to eight).  A batch reports that in
+    status[] instead of returning numbers; the one-call entry points simulate such a simulation again with twice the
+    slots until it fits, so their results are the reference's."""
     opts(batching_lanes=lanes)
     opts(batching_event_slots=8)
     c = random_case(6_000_012, max_m=40, max_g=90, max_s=2, max_r=1500, nb=3, load=60.0,
                     inf_slo=False, tie_prob=0.1, p_member=0.15)
+    f0, g0, c0, max_heap = oracle_c.simulate_requests_mixed_batching(
+        c["tstamps"], c["model_ids"], c["slos"], c["m2g"], c["g2m"], c["num_stages"], c["lat"], BSS[:3])
+    assert max_heap > 32
+    fin, good, cnt = _single(eng, c, BSS[:3])      # 8 -> 16 -> 32 -> ... slots inside the call
+    assert np.array_equal(good, g0)
+    assert np.array_equal(fin.view(np.uint64), f0.view(np.uint64))
+    for a, b in zip(cnt, c0):
+        assert np.array_equal(a, b)
+
+    cfg = make_config(5, 24)
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+    packed = E.pack_placements(cfg.placements, table)
+    st = cfg.stream(0)
+    n = 30000
+    dw = E.DeviceWorkload(eng, st.tstamps[:n], st.model_ids[:n], st.slos[:n], cfg.num_models)
+    flags = _lib.BATCHING | _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS
+    batch = E.Batch(eng, [dw], table, packed, flags)
+    batch.run()
+    batch.sync()
     with pytest.raises(_lib.MmsimError) as err:
-        _single(eng, c, BSS[:3])
+        batch.fetch()
     assert err.value.code == _lib.E_OVERFLOW
+    assert (batch.fetch(allow_failed=True)["status"] == _lib.E_OVERFLOW).any()
+    batch.close()
+    out = E.evaluate(eng, [dw], table, cfg.placements, flags)
+    lat, pp = table.arrays()
+    ref = oracle_c.eval_placements(st.tstamps[:n], st.model_ids[:n], st.slos[:n], lat, pp, cfg.batch_sizes, *packed,
+                                   batching=True, want_counts=True)
+    assert not out["status"].any()
+    assert np.array_equal(out["n_good"][0], ref["n_good"])
+    np.testing.assert_allclose(out["latency_sum"][0], ref["latency_sum"], rtol=1e-12)
+    for k in ("model_num_requests", "model_num_good", "group_num_requests", "group_num_good"):
+        assert np.array_equal(out[k][0][:, :ref[k].shape[1]], ref[k]), k
+    dw.close()
     opts(batching_event_slots=0)
     _single(eng, c, BSS[:3])                 # and the context is fine afterwards
 
