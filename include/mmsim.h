@@ -350,8 +350,8 @@ int mmsim_batch_kernel_name(const mmsim_batch *batch, char *buf, size_t size);
 /* create + run + sync + fetch + destroy.  With MMSIM_BATCHING, a simulation that runs out of idle-event slots
  * (status MMSIM_E_OVERFLOW: the reference's heap of idle events has no bound, the kernel's list of them has) is
  * simulated again inside this call with twice the slots, until it fits or LDS cannot hold more; only then does it
- * keep that status.  mmsim_eval_successors and mmsim_simulate_requests_mixed_batching do the same; a batch
- * (mmsim_batch_fetch) and mmsim_eval_pairs report the status and leave the choice to the caller
+ * keep that status.  mmsim_eval_pairs, mmsim_eval_successors and mmsim_simulate_requests_mixed_batching do the
+ * same; a batch (mmsim_batch_fetch) reports the status and leaves the choice to the caller
  * (mmsim_options.batching_event_slots). */
 int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
                      const mmsim_tables *tables, const mmsim_placements *placements,

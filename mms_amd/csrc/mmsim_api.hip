@@ -1737,13 +1737,21 @@ int mmsim_batch_kernel_name(const mmsim_batch *b, char *buf, size_t size) {
 
 namespace {
 
-// One-call evaluation with the given options (nullptr: the context's).  event_slots (optional) receives the event
-// slots per simulation that the batching simulator was given.
-int eval_once(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds, const mmsim_tables *tables,
-              const mmsim_placements *placements, uint32_t flags, const mmsim_options *options, mmsim_result *out,
-              int *event_slots) {
+// One-call evaluation with the given options (nullptr: the context's): every placement on every stream, or, with
+// stream_of, placement b on workloads[stream_of[b]] only.  event_slots (optional) receives the event slots per
+// simulation that the batching simulator was given.
+int eval_once(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_streams, const mmsim_tables *tables,
+              const mmsim_placements *placements, const int32_t *stream_of, uint32_t flags, const mmsim_options *options,
+              mmsim_result *out, int *event_slots) {
+    int rc = check_tables(tables);
+    if (rc) return rc;
+    rc = check_options(options);
+    if (rc) return rc;
+    RepLists rl;
+    rc = lists_from_placements(placements, tables->M, tables->C, &rl);
+    if (rc) return rc;
     mmsim_batch *b = nullptr;
-    int rc = mmsim_batch_create_ex(ctx, workloads, n_seeds, tables, placements, flags, options, &b);
+    rc = build_batch(ctx, workloads, n_streams, tables, rl, flags, &b, stream_of, options);
     if (rc == MMSIM_OK && event_slots) *event_slots = b->bargs.heap_cap;
     if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
     if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
@@ -1752,33 +1760,30 @@ int eval_once(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_
     return rc;
 }
 
-}  // namespace
-
-int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
-                     const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
-                     mmsim_result *out) {
-    if (!out) return fail(MMSIM_E_INVALID, "eval_batch: out is null");
-    // The batching simulator gives every simulation a fixed number of idle-event slots (what the reference's heap
-    // is seen to need, and what fits in LDS); a simulation that needs more stops with MMSIM_E_OVERFLOW.  Those are
-    // simulated again here, alone and with twice the slots, until they fit or LDS says no (they then keep that status).
+// The batching simulator gives every simulation a fixed number of idle-event slots (what the reference's heap is
+// seen to need, and what fits in LDS); a simulation that needs more stops with MMSIM_E_OVERFLOW.  Those are
+// simulated again here, alone and with twice the slots, until they fit or LDS says no (they then keep that status).
+int eval_with_retry(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_streams, const mmsim_tables *tables,
+                    const mmsim_placements *placements, const int32_t *stream_of, uint32_t flags, mmsim_result *out) {
+    const bool watch = (flags & MMSIM_BATCHING) != 0 && placements && n_streams > 0 && placements->B > 0;
+    const int32_t rows = stream_of ? 1 : n_streams;  // simulations per placement
     std::vector<int32_t> own_status;
     mmsim_result res = *out;
-    const bool watch = (flags & MMSIM_BATCHING) != 0 && placements && n_seeds > 0 && placements->B > 0;
     if (watch && !res.status) {
-        own_status.assign((size_t)n_seeds * placements->B, 0);
+        own_status.assign((size_t)rows * placements->B, 0);
         res.status = own_status.data();
     }
     int slots = 0;
-    int rc = eval_once(ctx, workloads, n_seeds, tables, placements, flags, nullptr, &res, &slots);
+    int rc = eval_once(ctx, workloads, n_streams, tables, placements, stream_of, flags, nullptr, &res, &slots);
     if (rc != MMSIM_OK || !watch) return rc;
     const int32_t B = placements->B, Gmax = placements->Gmax, M = tables->M;
     const size_t G1 = (size_t)Gmax + 1;
     int64_t Rmax = 0;
-    for (int s = 0; s < n_seeds; ++s) Rmax = std::max(Rmax, workloads[s]->R);
+    for (int s = 0; s < n_streams; ++s) Rmax = std::max(Rmax, workloads[s]->R);
     for (int round = 0; round < 8; ++round) {
         std::vector<int32_t> again;
         for (int32_t p = 0; p < B; ++p)
-            for (int s = 0; s < n_seeds; ++s)
+            for (int s = 0; s < rows; ++s)
                 if (res.status[(size_t)s * B + p] == MMSIM_E_OVERFLOW) {
                     again.push_back(p);
                     break;
@@ -1786,11 +1791,12 @@ int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
         if (again.empty()) break;
         slots *= 2;
         const int32_t B2 = (int32_t)again.size();
-        std::vector<int32_t> ng(B2), gc((size_t)B2 * Gmax), idx;
+        std::vector<int32_t> ng(B2), gc((size_t)B2 * Gmax), idx, so(B2, 0);
         std::vector<int64_t> off((size_t)B2 * G1);
         for (int32_t k = 0; k < B2; ++k) {
             const int32_t p = again[k];
             ng[k] = placements->num_groups[p];
+            if (stream_of) so[k] = stream_of[p];
             std::copy(placements->group_cfg + (size_t)p * Gmax, placements->group_cfg + (size_t)(p + 1) * Gmax, gc.begin() + (size_t)k * Gmax);
             for (size_t g = 0; g < G1; ++g) {
                 const int64_t lo = placements->gm_off[(size_t)p * G1 + g];
@@ -1800,7 +1806,7 @@ int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
         }
         if (idx.empty()) idx.push_back(0);
         const mmsim_placements sub = {B2, Gmax, ng.data(), gc.data(), off.data(), idx.data()};
-        const size_t L2 = (size_t)n_seeds * B2;
+        const size_t L2 = (size_t)rows * B2;
         std::vector<int64_t> n_good(L2);
         std::vector<double> lat_sum(L2), finish;
         std::vector<int32_t> mreq, mgood, greq, ggood, status(L2);
@@ -1823,24 +1829,34 @@ int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
         }
         mmsim_options o = ctx->opt;
         o.batching_event_slots = slots;
-        if (eval_once(ctx, workloads, n_seeds, tables, &sub, flags, &o, &r2, nullptr) != MMSIM_OK) break;  // (does not fit in LDS)
+        if (eval_once(ctx, workloads, n_streams, tables, &sub, stream_of ? so.data() : nullptr, flags, &o, &r2, nullptr) != MMSIM_OK)
+            break;  // (does not fit in LDS)
         for (int32_t k = 0; k < B2; ++k)
-            for (int s = 0; s < n_seeds; ++s) {
+            for (int s = 0; s < rows; ++s) {
                 const size_t src = (size_t)s * B2 + k, dst = (size_t)s * B + again[k];
                 if (res.n_good) res.n_good[dst] = n_good[src];
                 if (res.latency_sum) res.latency_sum[dst] = lat_sum[src];
                 res.status[dst] = status[src];
-                if (r2.model_num_requests && res.model_num_requests) std::copy(&mreq[src * M], &mreq[(src + 1) * M], res.model_num_requests + dst * M);
-                if (r2.model_num_good && res.model_num_good) std::copy(&mgood[src * M], &mgood[(src + 1) * M], res.model_num_good + dst * M);
-                if (r2.group_num_requests && res.group_num_requests) std::copy(&greq[src * Gmax], &greq[(src + 1) * Gmax], res.group_num_requests + dst * Gmax);
-                if (r2.group_num_good && res.group_num_good) std::copy(&ggood[src * Gmax], &ggood[(src + 1) * Gmax], res.group_num_good + dst * Gmax);
+                if (r2.model_num_requests && res.model_num_requests) std::copy(&mreq[src * M], &mreq[src * M] + M, res.model_num_requests + dst * M);
+                if (r2.model_num_good && res.model_num_good) std::copy(&mgood[src * M], &mgood[src * M] + M, res.model_num_good + dst * M);
+                if (r2.group_num_requests && res.group_num_requests) std::copy(&greq[src * Gmax], &greq[src * Gmax] + Gmax, res.group_num_requests + dst * Gmax);
+                if (r2.group_num_good && res.group_num_good) std::copy(&ggood[src * Gmax], &ggood[src * Gmax] + Gmax, res.group_num_good + dst * Gmax);
                 if (r2.finish) {
-                    std::copy(&finish[src * (size_t)Rmax], &finish[(src + 1) * (size_t)Rmax], res.finish + dst * (size_t)Rmax);
-                    std::copy(&good[src * (size_t)Rmax], &good[(src + 1) * (size_t)Rmax], res.good + dst * (size_t)Rmax);
+                    std::copy(&finish[src * (size_t)Rmax], &finish[src * (size_t)Rmax] + Rmax, res.finish + dst * (size_t)Rmax);
+                    std::copy(&good[src * (size_t)Rmax], &good[src * (size_t)Rmax] + Rmax, res.good + dst * (size_t)Rmax);
                 }
             }
     }
     return MMSIM_OK;
+}
+
+}  // namespace
+
+int mmsim_eval_batch(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
+                     const mmsim_tables *tables, const mmsim_placements *placements, uint32_t flags,
+                     mmsim_result *out) {
+    if (!ctx || !out) return fail(MMSIM_E_INVALID, "eval_batch: null pointer");
+    return eval_with_retry(ctx, workloads, n_seeds, tables, placements, nullptr, flags, out);
 }
 
 int mmsim_eval_successors(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,
@@ -1859,18 +1875,7 @@ int mmsim_eval_pairs(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int
                      const mmsim_tables *tables, const mmsim_placements *placements, const int32_t *stream_of,
                      uint32_t flags, mmsim_result *out) {
     if (!ctx || !out || !stream_of) return fail(MMSIM_E_INVALID, "eval_pairs: null pointer");
-    int rc = check_tables(tables);
-    if (rc) return rc;
-    RepLists rl;
-    rc = lists_from_placements(placements, tables->M, tables->C, &rl);
-    if (rc) return rc;
-    mmsim_batch *b = nullptr;
-    rc = build_batch(ctx, workloads, n_streams, tables, rl, flags, &b, stream_of);
-    if (rc == MMSIM_OK) rc = mmsim_batch_run(b);
-    if (rc == MMSIM_OK) rc = mmsim_batch_sync(b, nullptr);
-    if (rc == MMSIM_OK) rc = mmsim_batch_fetch(b, out);
-    mmsim_batch_destroy(b);
-    return rc;
+    return eval_with_retry(ctx, workloads, n_streams, tables, placements, stream_of, flags, out);
 }
 
 int mmsim_eval_batch_static(mmsim_ctx *ctx, const mmsim_workload *const *workloads, int32_t n_seeds,

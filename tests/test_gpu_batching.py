@@ -195,6 +195,18 @@ def test_a_simulation_that_runs_out_of_event_slots(eng, opts, lanes):
     np.testing.assert_allclose(out["latency_sum"][0], ref["latency_sum"], rtol=1e-12)
     for k in ("model_num_requests", "model_num_good", "group_num_requests", "group_num_good"):
         assert np.array_equal(out[k][0][:, :ref[k].shape[1]], ref[k]), k
+    # ... and so does the paired entry point (placement b on stream b mod 2)
+    n2 = 20000
+    dw2 = E.DeviceWorkload(eng, st.tstamps[:n2], st.model_ids[:n2], st.slos[:n2], cfg.num_models)
+    stream_of = np.arange(len(cfg.placements), dtype=np.int32) % 2
+    got = E.eval_pairs(eng, [dw, dw2], table, packed, stream_of, flags)
+    ref2 = oracle_c.eval_placements(st.tstamps[:n2], st.model_ids[:n2], st.slos[:n2], lat, pp, cfg.batch_sizes, *packed,
+                                    batching=True, want_counts=True)
+    for b in range(len(cfg.placements)):
+        r = ref2 if stream_of[b] else ref
+        assert got["n_good"][b] == r["n_good"][b], b
+        assert np.array_equal(got["model_num_good"][b], r["model_num_good"][b]), b
+    dw2.close()
     dw.close()
     opts(batching_event_slots=0)
     _single(eng, c, BSS[:3])                 # and the context is fine afterwards
