@@ -341,6 +341,8 @@ typedef struct {
     int32_t segments;         /* pieces a stream is cut into so that a workgroup's items take turns  */
     int32_t launches;         /* kernel launches of one mmsim_batch_run                             */
     int32_t waves_per_group;  /* wavefronts of a workgroup that simulate side by side               */
+    int32_t event_slots;      /* batching simulator: idle-event slots per simulation; 0 otherwise   */
+    int32_t reserved;
 } mmsim_batch_info;
 int mmsim_batch_get_info(const mmsim_batch *batch, mmsim_batch_info *out);
 /* Name of the kernel template instance mmsim_batch_run launches for this batch, as a profiler prints it

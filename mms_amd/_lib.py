@@ -79,7 +79,8 @@ class BatchInfo(C.Structure):
                 ("smax_bucket", C.c_int32), ("max_replicas", C.c_int32), ("slots", C.c_int32),
                 ("lds_bytes", C.c_int32), ("requests_total", C.c_int64), ("table_bytes", C.c_int64),
                 ("stream_bytes", C.c_int64), ("workgroups", C.c_int32), ("segments", C.c_int32),
-                ("launches", C.c_int32), ("waves_per_group", C.c_int32)]
+                ("launches", C.c_int32), ("waves_per_group", C.c_int32), ("event_slots", C.c_int32),
+                ("reserved", C.c_int32)]
 
 
 # name -> (restype, argtypes); also the list of symbols the header declares

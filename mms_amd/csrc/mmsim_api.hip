@@ -1724,6 +1724,8 @@ int mmsim_batch_get_info(const mmsim_batch *b, mmsim_batch_info *out) {
     out->segments = b->max_nseg;
     out->launches = 1;
     out->waves_per_group = b->waves_per_block;
+    out->event_slots = (b->flags & MMSIM_BATCHING) ? b->bargs.heap_cap : 0;
+    out->reserved = 0;
     return MMSIM_OK;
 }
 

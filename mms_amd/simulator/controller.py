@@ -318,15 +318,30 @@ def device_compute_stats(workload, sols, model_names, prof_ress, model_ids, slos
     flags = _lib.WANT_GROUP_COUNTS | _lib.WANT_PER_REQUEST | (_lib.BATCHING if enable_batching else 0)
     own = device_workload is None
     dw = _engine.DeviceWorkload(eng, arrivals, model_ids, slos, len(model_names)) if own else device_workload
-    batch = _engine.Batch(eng, [dw], table, _engine.pack_placements(sols, table), flags)
+    packed = _engine.pack_placements(sols, table)
+    skip = warmup_skip(arrivals, warmup)
+    options = None
     try:
-        batch.run()
-        batch.sync()
-        out = batch.fetch(per_request=False)
-        skip = warmup_skip(arrivals, warmup)
-        ms = batch.model_stats([skip])
+        # The statistics are taken from what the run leaves on the device, so a batching simulation that runs out
+        # of idle-event slots (the reference's heap has no bound, the kernel's list is sized from the group count)
+        # sends the whole batch round again with twice the slots.
+        for attempt in range(6):
+            batch = _engine.Batch(eng, [dw], table, packed, flags, options=options)
+            try:
+                batch.run()
+                batch.sync()
+                try:
+                    out = batch.fetch(per_request=False)
+                except _lib.MmsimError as err:
+                    if err.code != _lib.E_OVERFLOW or attempt == 5:
+                        raise
+                    options = dict(getattr(eng, "_options", {}), batching_event_slots=2 * batch.info()["event_slots"])
+                    continue
+                ms = batch.model_stats([skip])
+                break
+            finally:
+                batch.close()
     finally:
-        batch.close()
         if own:
             dw.close()
 

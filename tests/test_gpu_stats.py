@@ -82,6 +82,33 @@ def test_batching_simulator(eng):
     _check(eng, cfg, cfg.placements, (0,), [(0,), (R // 9,)], flags=_lib.BATCHING)
 
 
+def test_statistics_of_a_batching_run_that_needs_more_event_slots(eng, opts):
+    """device_compute_stats (approximate_one_case without fast_stats) takes the statistics from what the run left on
+    the device; a simulation that runs out of idle-event slots (forced here: eight slots) makes it run the batch
+    again with twice the slots until every simulation fits.  The result is that of a run with the default slots."""
+    import types
+    from mms_amd.simulator import controller as sim
+    cfg = make_config(5, 6)
+    cfg.duration *= 0.05
+    st = cfg.stream(0)
+    wl = types.SimpleNamespace(arrivals=st.tstamps, requests=None)
+    names = [f"m{i}" for i in range(cfg.num_models)]
+    table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
+
+    def stats():
+        return sim.device_compute_stats(wl, cfg.placements, names, cfg.profiles, st.model_ids, st.slos, 10,
+                                        enable_batching=True, table=table)
+    want = stats()
+    opts(batching_event_slots=8)
+    got = stats()
+    assert len(got) == len(want) == 6
+    for g, w in zip(got, want):
+        assert g.goodput == w.goodput and g.latency_mean == w.latency_mean and g.num_requests == w.num_requests
+        assert list(g.group_num_requests) == list(w.group_num_requests)
+        for pg, pw in zip(g.per_model_stats, w.per_model_stats):
+            assert (pg.name, pg.num_requests, pg.goodput, pg.latency_p99) == (pw.name, pw.num_requests, pw.goodput, pw.latency_p99)
+
+
 @pytest.mark.parametrize("config, placements, seeds, shrink, flags", [
     (2, 5, (0, 1), 1.0, 0), (4, 1, (2,), 0.05, 0), (4, 16, (1,), 0.02, 0), (5, 3, (0,), 0.05, _lib.BATCHING)],
     ids=["cfg2-5x2", "cfg4-1", "cfg4-16", "cfg5-3-batching"])

@@ -47,7 +47,7 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.Tables) == 48
     assert ctypes.sizeof(_lib.Placements) == 40
     assert ctypes.sizeof(_lib.Result) == 10 * 8
-    assert ctypes.sizeof(_lib.BatchInfo) == 8 * 4 + 3 * 8 + 4 * 4
+    assert ctypes.sizeof(_lib.BatchInfo) == 8 * 4 + 3 * 8 + 6 * 4
     assert ctypes.sizeof(_lib.ModelStats) == 9 * 8
     # field order of mmsim_model_stats as the header declares it
     header = open(os.path.join(ROOT, "include", "mmsim.h")).read()
