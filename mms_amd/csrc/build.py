@@ -27,13 +27,15 @@ FLAGS = [
 ]
 
 
-# The plain simulator runs one or two wavefronts per SIMD (LDS decides how many), so
-# instruction-level parallelism inside a wavefront is what hides latency: schedule for it (measured
-# -7 % kernel time).  The batching kernel takes the max-ilp strategy (iterative-ilp fails on it; measured -1.6 %
-# with the block alignment).
+# The simulators run one or two wavefronts per SIMD (LDS decides how many), so instruction-level parallelism
+# inside a wavefront is what hides latency: schedule for it.  Measured on the plain simulator (configuration 4 /
+# its counts mode / configuration 3): max-ilp 531.4 / 606.1 / 23.9 ms, iterative-ilp 534.3 / 606.5 / 24.1 ms,
+# iterative-minreg 527.9 / 612.4 / 30.1 ms, the default strategy 7 % behind; on the batching simulator max-ilp with
+# the block alignment -1.6 % (iterative-ilp fails on it).
 # Blocks that are only reached by a branch start on a 64-byte boundary: a taken branch costs a lone wavefront
-# tens of cycles, less when its target starts an instruction cache line (measured: -1 % in the counts mode).
-SOURCE_FLAGS = {"sim_mixed.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp", "-mllvm", "-align-all-nofallthru-blocks=6"],
+# tens of cycles, less when its target starts an instruction cache line (measured: -1 % in the counts mode; 32- and
+# 128-byte boundaries, aligning every block, and switching block placement or tail duplication off are all slower).
+SOURCE_FLAGS = {"sim_mixed.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp", "-mllvm", "-align-all-nofallthru-blocks=6"],
                 "sim_batching.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp", "-mllvm", "-align-all-nofallthru-blocks=6"]}
 
 
