@@ -28,14 +28,16 @@ FLAGS = [
 
 
 # The simulators run one or two wavefronts per SIMD (LDS decides how many), so instruction-level parallelism
-# inside a wavefront is what hides latency: schedule for it.  Measured on the plain simulator (configuration 4 /
-# its counts mode / configuration 3): max-ilp 531.4 / 606.1 / 23.9 ms, iterative-ilp 534.3 / 606.5 / 24.1 ms,
-# iterative-minreg 527.9 / 612.4 / 30.1 ms, the default strategy 7 % behind; on the batching simulator max-ilp with
-# the block alignment -1.6 % (iterative-ilp fails on it).
+# inside a wavefront is what hides latency: schedule for it.  Measured on the plain simulator (configuration 4 / its
+# counts mode / configuration 3 / configuration 2 / its counts mode): iterative-ilp 534.3 / 606.5 / 24.1 / 4.56 /
+# 4.84 ms, max-ilp 531.4 / 606.1 / 23.9 / 4.72 / 5.13 ms (half a per cent on the large batch, three to six per cent
+# the other way on the small multi-stage batches that the searches send: iterative-ilp stays), iterative-minreg
+# 527.9 / 612.4 / 30.1 ms, the default strategy 7 % behind; on the batching simulator max-ilp with the block
+# alignment -1.6 % (iterative-ilp fails on it).
 # Blocks that are only reached by a branch start on a 64-byte boundary: a taken branch costs a lone wavefront
 # tens of cycles, less when its target starts an instruction cache line (measured: -1 % in the counts mode; 32- and
 # 128-byte boundaries, aligning every block, and switching block placement or tail duplication off are all slower).
-SOURCE_FLAGS = {"sim_mixed.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp", "-mllvm", "-align-all-nofallthru-blocks=6"],
+SOURCE_FLAGS = {"sim_mixed.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp", "-mllvm", "-align-all-nofallthru-blocks=6"],
                 "sim_batching.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp", "-mllvm", "-align-all-nofallthru-blocks=6"]}
 
 
