@@ -164,10 +164,13 @@ def body_pow2_straight(levels, flavour, lean=False):
                     a.append(f"ds_read_b32 v{L0 + kk}, %[lb] offset:{4 * kk}")
                     issued.append([("l", kk)])
         # reads return in order: an item is there when at most (reads issued after it) are outstanding
+        # (one latency per (model, config): the reads after the first are waited for two at a time -- a wait is an
+        # instruction like any other, and with two wavefronts on a SIMD the walk is bound by what it issues)
         arrive = {}
         for i, items in enumerate(issued):
+            upto = i if flavour == "N" or i == 0 else min(len(issued) - 1, i + i % 2)
             for it in items:
-                arrive[it] = len(issued) - 1 - i
+                arrive[it] = len(issued) - 1 - upto
         fill = []                               # independent instructions to drop into the chain's gaps
         waited = 99
         for k in range(D):

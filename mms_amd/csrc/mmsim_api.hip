@@ -507,6 +507,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
 
     // ---- which request loop: bursty streams (most requests repeat the model of the one before) get the loop over runs
     bool runs = false;
+    const bool more_than_scores = (flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT | MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) != 0;
     if (!batching) {
         int64_t rep = 0, tot = 0;
         for (int s = 0; s < n_seeds; ++s) {
@@ -515,6 +516,9 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
         runs = 5 * rep > 4 * tot;  // four in five (measured: at three in four the chunked loop is still ahead)
         if (o.request_loop >= 0) runs = o.request_loop != 0;
+        // (with one latency per (model, configuration) the loop over runs keeps a model's row of the table in a
+        // register, one entry per lane, whenever it produces more than the scores or the table does not fit in LDS)
+        if (uniform_stages && lat_row > kWave) runs = false;
     }
 
     phase("latency table, loop choice");
@@ -546,7 +550,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     };
     if (!batching) {
         wave_bytes = mixed_wave_bytes(nslots);  // of the largest placement
-        lat_bytes = (lat.size() * sizeof(float) + 15) & ~(size_t)15;
+        lat_bytes = runs && uniform_stages && more_than_scores ? 0 : (lat.size() * sizeof(float) + 15) & ~(size_t)15;  // (see above)
         sched_bytes = runs ? (size_t)kSchedLdsBytes : 0;
         if (lat_bytes + sched_bytes + wave_bytes > (size_t)ctx->max_lds) {
             lat_in_lds = 0;

@@ -247,8 +247,16 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         if (threadIdx.x == 0) *a.error = 1;
         return;
     }
+    // Loop over runs with one latency per (model, configuration), any output beyond the scores: a run's model row
+    // of the latency table (at most 64 entries, the host sees to that) travels in a register, one entry per lane,
+    // and the latencies of the run's listed replicas are gathered from it across the lanes once per run; the table
+    // is not needed in LDS then, and a replica scan ends with the tournament instead of a dependent read of the
+    // winner's latency (configuration 4 with per-group counts: 592 ms against 605; scores only: 536 against 534,
+    // so the scores-only kernel keeps the table in LDS).
+    constexpr bool RUNLAT = RUNS && UNIFORM && OUT != 0;
+    constexpr bool TABLE_LDS = LATLDS && !RUNLAT;
     float *lat_lds = reinterpret_cast<float *>(lds_raw);
-    const int lat_floats = LATLDS ? a.M * a.lat_row : 0;
+    const int lat_floats = TABLE_LDS ? a.M * a.lat_row : 0;
     for (int i = (int)threadIdx.x; i < lat_floats; i += (int)blockDim.x) lat_lds[i] = a.lat[i];
 
     // Which (tile, stream) pairs this wavefront simulates, and where its LDS region is.
@@ -291,7 +299,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     __syncthreads();
     if (!live) return;  // a wavefront without work: padding of the last workgroup, or no LDS region in this schedule
 
-    const float *lat_base = LATLDS ? lat_lds : a.lat;
+    const float *lat_base = TABLE_LDS ? lat_lds : a.lat;
     const double overhead = a.fixed_overhead;
 
   for (int spins = 0;;) {  // SCHED: one turn per (item, segment) this wavefront is given; otherwise a single turn
@@ -455,6 +463,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     // Loop over runs: LDS addresses of the last-stage clocks of the run's listed replicas, worked out once per run
     // (they depend on the descriptors only) and pinned there.
     uint32_t run_ca[RREG] = {};
+    float run_l[RREG] = {};  // RUNLAT: their last-stage latencies
 
     // (PLAIN: the caller has seen that the tile lists one to four replicas for the model: the scan has no case to
     // tell, reads where `sa` says, and calls `meanwhile` once its reads are under way)
@@ -489,7 +498,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     k[j].l = lds_f32(sa.l[j]);
                 } else if constexpr (RUNS) {
                     k[j].c = lds_f64(run_ca[j0 + j]);
-                    k[j].l = 0.0f;  // (the winner's latency is read after the tournament instead, one read for eight)
+                    k[j].l = RUNLAT ? run_l[j0 + j] : 0.0f;  // (otherwise the winner's latency is read after the tournament, one read for eight)
                 } else {
                     k[j].c = lds_f64(rep_addr(k[j].d) + rel_base);
                     k[j].l = lrow_m[rep_lat_last(k[j].d)];
@@ -523,7 +532,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     scan(more, Idx<4>{});
                     win = first_min(win, more);  // the final of the tournament of eight: entries 0-3 against 4-7
                     if (n > RREG) beyond_eight();
-                } else if (__builtin_expect(n > 0, 1)) {
+                } else if (OUT != 3 || n > 0) {  // (runs without a listed replica are passed over as a whole, see the loop)
                     scan(win, Idx<0>{});
                 }
             } else if constexpr (plain_scan) {
@@ -537,7 +546,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
                     if (n > RREG) beyond_eight();
                 }
             }
-            if constexpr (RUNS) win.l = lrow_m[rep_lat_last(win.d)];
+            if constexpr (RUNS && !RUNLAT) win.l = lrow_m[rep_lat_last(win.d)];
             // a clock that is infinite (a group that served a request with infinite latency) is never
             // chosen (:590-598: "tmp < min_device_clock" with min_device_clock starting at inf)
             ch_model = m;
@@ -545,11 +554,12 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             ch_best = win.c;
             ch_l_last = (double)win.l;
             // what the walk needs of the chosen group, worked out once per choice
-            const bool found = (int32_t)win.d >= 0 && win.c < 1e100;
+            // (an empty descriptor points at the +inf row, so the clock alone tells whether a group was found)
+            const bool found = win.c < 1e100;
             const int stages_m1 = (int)rep_stages_m1(win.d);
             ch_sm1 = found ? stages_m1 : -1;
             ch_last = rep_addr(win.d) + rel_base;
-            ch_first = ch_last - (uint32_t)(found ? stages_m1 : 0) * kSlotBytes;
+            ch_first = ch_last - (uint32_t)stages_m1 * kSlotBytes;  // (read by walking lanes only)
             ch_lrow = found ? (int)rep_lat_last(win.d) - stages_m1 : 0;
             if (group_regs) {  // requests handled up to here went to the group chosen before (:611, :618)
                 const uint32_t now = found ? ch_last : 0xFFFFFFFFu;
@@ -572,7 +582,9 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         double finish_time;
         bool acc = false;
         uint64_t acc_mask = 0;  // wave-uniform: lanes that accepted the request
-        constexpr bool LEAN = OUT == 0;  // scores only: nobody asks which lane accepted or when it finished
+        // Nobody asks which lane accepted or when it finished: scores only, and the counts of the loop over runs
+        // without counters in LDS (they come from the growth of n_good, per run and per choice of group).
+        constexpr bool LEAN = OUT == 0 || (OUT == 1 && RUNS);
         bool asm_walk = false;
         if constexpr (SMAX == 1) {
             // ---- single-stage groups: the clock read for the choice is the whole pipeline (:605-619)
@@ -589,26 +601,34 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             // ---- lanes that cannot make the SLO even with an otherwise idle pipeline skip the walk
             const double bound = ((vmax(tstamp, best) + l_last) + overhead) - tstamp;
             const int walk = !(bound > slo) ? sm1 : -1;  // stages - 1 of lanes that walk (no per-lane branch; -1 without a replica)
-            if constexpr (LATLDS && (SMAX == 4 || SMAX == 16)) {
+            if constexpr ((LATLDS || RUNLAT) && (SMAX == 4 || SMAX == 16)) {
                 // ---- stage walk, SLO decision and commit (:605-619) as one hand-scheduled block
                 uint64_t saved_exec, mask1, mask2, mask4, mask8;  // masks: scratch of the power-of-two walk
                 int accepted;
                 double latency;
                 const uint32_t cb_addr = first_addr;
-#define MMSIM_WALK(NAME, LATNAME, LATVAL)                                                                           \
+#define MMSIM_WALK(NAME, LATNAME, LATVAL, TSREG)                                                                    \
 asm volatile(NAME##_TEXT                                                                                        \
      : [sv] "=&s"(saved_exec), [acc] "=&v"(accepted), [fin] "=&v"(finish_time), [lat] "=&v"(latency),   \
        [ng] "+v"(n_good), [ls] "+v"(lat_sum), [m1] "=&s"(mask1), [m2] "=&s"(mask2), [m4] "=&s"(mask4),  \
        [m8] "=&s"(mask8), [am] "=&s"(acc_mask)                                                          \
-     : [walk] "v"(walk), [cb] "v"(cb_addr), [LATNAME] "v"(LATVAL), [ts] "v"(tstamp), [slo] "v"(slo),    \
+     : [walk] "v"(walk), [cb] "v"(cb_addr), [LATNAME] "v"(LATVAL), [ts] TSREG(tstamp), [slo] "v"(slo),  \
        [oh] "s"(overhead)                                                                               \
      : "vcc", "scc", "memory", NAME##_CLOBBERS)
+// (the loop over runs has the arrival time in scalar registers, read out of the block with v_readlane)
+#define MMSIM_WALK_TS(NAME, LATNAME, LATVAL)                   \
+    do {                                                       \
+        if constexpr (RUNS)                                    \
+            MMSIM_WALK(NAME, LATNAME, LATVAL, "s");            \
+        else                                                   \
+            MMSIM_WALK(NAME, LATNAME, LATVAL, "v");            \
+    } while (0)
 #define MMSIM_WALK_PICK(NAME, LATNAME, LATVAL)                 \
     do {                                                       \
         if constexpr (LEAN)                                    \
-            MMSIM_WALK(NAME##_LEAN, LATNAME, LATVAL);          \
+            MMSIM_WALK_TS(NAME##_LEAN, LATNAME, LATVAL);       \
         else                                                   \
-            MMSIM_WALK(NAME, LATNAME, LATVAL);                 \
+            MMSIM_WALK_TS(NAME, LATNAME, LATVAL);              \
     } while (0)
                 if constexpr (UNIFORM) {
                     if (pow2) {
@@ -637,6 +657,7 @@ asm volatile(NAME##_TEXT                                                        
                     }
                 }
 #undef MMSIM_WALK_PICK
+#undef MMSIM_WALK_TS
 #undef MMSIM_WALK
                 if constexpr (!LEAN) acc = accepted != 0;
                 asm_walk = true;
@@ -718,6 +739,8 @@ asm volatile(NAME##_TEXT                                                        
     if constexpr (RUNS) {
         // Descriptors of the run about to start (fetched while the run before it is simulated).
         uint4 nda = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty), ndb = nda;
+        float nlat = 0.0f;  // RUNLAT: entry `lane` of the model's row of the latency table
+        const int lat_lane = lane < a.lat_row ? lane : 0;
         // (the second half of a row, replicas 4-7, is only read by runs whose tile lists more than four replicas
         // for the model; the other runs load the first half twice -- the second load hits the line the first one
         // just brought in -- which costs no branch and no memory traffic)
@@ -725,6 +748,7 @@ asm volatile(NAME##_TEXT                                                        
             const uint4 *row = rep_tile + (size_t)(model < 0 ? 0 : model) * (2 * kWave);
             nda = row[0];
             ndb = row[more_than_four ? kWave : 0];
+            if constexpr (RUNLAT) nlat = a.lat[(size_t)(model < 0 ? 0 : model) * a.lat_row + lat_lane];
         };
         {
             const int z0 = __builtin_amdgcn_readlane(ahead.z, 0);
@@ -759,6 +783,7 @@ asm volatile(NAME##_TEXT                                                        
                 const uint64_t later = starts & (s0 >= 63 ? 0ull : (~0ull << (s0 + 1)));
                 const int s1 = later ? (int)__builtin_ctzll(later) : nblk;  // the run is requests [s0, s1)
                 const uint4 da = nda, db = ndb;
+                const float lat_row_here = nlat;
                 {   // the run after this one: of this block, or the first of the next block
                     int zn = -1;
                     if (s1 < nblk)
@@ -772,6 +797,15 @@ asm volatile(NAME##_TEXT                                                        
                 const int w = __builtin_amdgcn_readlane(r.z, s0);
                 const int m = w >= 0 ? (w & 0xFFFFFF) : -1;  // wave-uniform model id (or -1)
                 const int n = w >= 0 ? (w >> 24) : 0;        // replica bound of the tile; 0: nothing to simulate
+                if constexpr (OUT != 3) {
+                    // no lane of the tile hosts the model (or the stream names a model that does not exist): nothing
+                    // changes and nothing is counted, whatever the requests are
+                    if (n == 0) {
+                        if (group_regs) pg_req0 += (uint32_t)(s1 - s0);  // (not requests of the group the lane counts for)
+                        s0 = s1;
+                        continue;
+                    }
+                }
                 const uint64_t run = (s1 >= 64 ? ~0ull : ((1ull << s1) - 1ull)) & (~0ull << s0) & valid;
                 const int32_t good_before = n_good;  // model_per_run
                 static_while<0, RREG>([&](auto J) {
@@ -781,6 +815,16 @@ asm volatile(NAME##_TEXT                                                        
                 });
                 asm volatile("" : "+v"(run_ca[0]), "+v"(run_ca[1]), "+v"(run_ca[2]), "+v"(run_ca[3]), "+v"(run_ca[4]),
                                   "+v"(run_ca[5]), "+v"(run_ca[6]), "+v"(run_ca[7]));
+                if constexpr (RUNLAT) {
+                    auto gather = [&](auto J) {
+                        constexpr int j = decltype(J)::value;
+                        run_l[j] = __int_as_float(__builtin_amdgcn_ds_bpermute(
+                            (int)(rep_lat_last(pick_desc<j>(da, db)) << 2), __float_as_int(lat_row_here)));
+                        return true;
+                    };
+                    static_while<0, 4>(gather);
+                    if (n > 4) static_while<4, RREG>(gather);
+                }
 
                 auto request = [&](int i) {
                     return simulate(blk + i, m, n, da, db,
