@@ -490,6 +490,54 @@ def test_runs_of_one_model_with_odd_requests(eng, opts, loop, flags):
         assert 0 < ref["n_good"].sum() < len(t) * len(cfg.placements) or len(t) < 64
 
 
+@pytest.mark.parametrize("n_configs", [12, 63, 70])
+@pytest.mark.parametrize("flags", [0, _lib.WANT_MODEL_COUNTS | _lib.WANT_GROUP_COUNTS, ALL])
+def test_loop_over_runs_with_many_configurations_and_unhosted_models(eng, opts, n_configs, flags):
+    """With one latency per (model, configuration) and outputs beyond the scores, the loop over runs keeps a model's row
+    of the latency table in a register, one entry per lane, and gathers the latencies of a run's listed replicas from
+    it: rows of 13 and of 64 entries (the most that fit) take that path, 71 entries send the batch to the chunked loop
+    although the loop over runs is asked for.  Models with up to six replicas (more than the four of the usual scan),
+    models that no placement of a tile hosts (their runs are passed over) and unknown models are in the stream."""
+    from types import SimpleNamespace
+    from mms_amd.profiling import ParallelConfig, synthetic_profile
+    from mms_amd.placement_policy.base_policy import ModelPlacement
+    opts(request_loop=1)
+    rng = np.random.default_rng(7000 + n_configs)
+    M, R, B = 10, 6000, 130
+    pcs = [ParallelConfig(1 + k // 16, 1 + (k // 4) % 4, (1, 2, 4, 8)[k % 4]) for k in range(n_configs)]
+    assert len(set(pcs)) == n_configs
+    profiles = [synthetic_profile(f"m{m}", float(rng.uniform(0.05, 0.3)), pcs) for m in range(M)]
+    sols = []
+    for _ in range(B):
+        cfgs, models = [], []
+        for _g in range(int(rng.integers(3, 9))):
+            cfgs.append(pcs[int(rng.integers(0, n_configs))])
+            # models 0-1 are everywhere (up to eight replicas), 2-7 here and there, 8-9 hosted by nobody
+            models.append([0, 1][: int(rng.integers(0, 3))] + [int(x) for x in rng.choice(np.arange(2, 8), size=int(rng.integers(0, 3)), replace=False)])
+        sols.append(ModelPlacement(cfgs, models))
+    runs = rng.geometric(0.1, size=R)
+    model_ids = np.repeat(rng.integers(0, M, size=R), runs)[:R].astype(np.int32)
+    model_ids[rng.random(R) < 0.01] = -1
+    gaps = rng.exponential(0.01, size=R)
+    gaps[rng.random(R) < 0.2] = 0.0
+    st = SimpleNamespace(tstamps=np.cumsum(gaps), model_ids=model_ids, slos=rng.uniform(0.2, 1.5, R).astype(np.float32))
+    table = E.LatencyTable(profiles, [1])
+    packed = E.pack_placements(sols, table)
+    dw = E.DeviceWorkload(eng, st.tstamps, st.model_ids, st.slos, M)
+    batch = E.Batch(eng, [dw], table, packed, flags)
+    batch.run()
+    batch.sync()
+    out = batch.fetch()
+    name = batch.kernel_name()
+    assert batch.info()["max_replicas"] > 4
+    batch.close()
+    assert name.endswith(", true>") == (n_configs < 64), name       # the last template argument: loop over runs
+    traces = bool(flags & _lib.WANT_PER_REQUEST)
+    ref = oracle_batch(st, table, packed, want_per_request=traces)
+    assert_batch_matches(out, ref, 0, packed[0], per_request=traces, where=f"{n_configs} configurations, flags {flags}")
+    assert 0.02 * R * B < ref["n_good"].sum() < 0.9 * R * B
+
+
 def test_rerunning_a_batch_gives_the_same_answer(eng):
     cfg = make_config(2)
     table = E.LatencyTable(cfg.profiles, cfg.batch_sizes)
