@@ -457,9 +457,28 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     bool pow2_depths = true;  // every group has 1, 2, 4, 8 or 16 stages
     std::vector<uint8_t> slot0((size_t)B * Gmax, 0);
     std::vector<int32_t> slots_of(B, 0);  // clock slots placement p needs
+    // A placement's clock slots are laid out shallowest group first, groups that host no model before all others:
+    // the walk for power-of-two depths lets every walking lane read as many clock rows as the deepest walking lane
+    // of its wavefront, and a lane whose deepest group comes last then reads past its own slots only by what the
+    // tile's deepest group has on its own deepest (nothing, where a tile's placements are equally deep).
+    std::vector<uint8_t> group_hosts((size_t)B * Gmax, 0);
+    for (int32_t p = 0; p < B; ++p)
+        for (int64_t x = rl.off[(size_t)p * M]; x < rl.off[(size_t)(p + 1) * M]; ++x) {
+            const int32_t g = rl.grp[(size_t)x];
+            if (g >= 0 && g < rl.num_groups[p]) group_hosts[(size_t)p * Gmax + g] = 1;
+        }
     for (int32_t p = 0; p < B; ++p) {
         int s = 0;
-        for (int32_t g = 0; g < rl.num_groups[p]; ++g) {
+        int32_t by_depth[MMSIM_MAX_GROUPS];
+        const int32_t ng = rl.num_groups[p];
+        for (int32_t g = 0; g < ng; ++g) by_depth[g] = g;
+        std::stable_sort(by_depth, by_depth + ng, [&](int32_t x, int32_t y) {
+            const int kx = group_hosts[(size_t)p * Gmax + x] ? t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + x]] : 0;
+            const int ky = group_hosts[(size_t)p * Gmax + y] ? t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + y]] : 0;
+            return kx < ky;
+        });
+        for (int32_t k = 0; k < ng; ++k) {
+            const int32_t g = by_depth[k];
             const int pp = t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]];
             if (s + pp > MMSIM_MAX_SLOTS)
                 return fail(MMSIM_E_UNSUPPORTED, "placement has more than 255 pipeline stages in total");
@@ -507,7 +526,6 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
 
     // ---- which request loop: bursty streams (most requests repeat the model of the one before) get the loop over runs
     bool runs = false;
-    const bool more_than_scores = (flags & (MMSIM_WANT_PER_REQUEST | MMSIM_WANT_OP_COUNT | MMSIM_WANT_MODEL_COUNTS | MMSIM_WANT_GROUP_COUNTS)) != 0;
     if (!batching) {
         int64_t rep = 0, tot = 0;
         for (int s = 0; s < n_seeds; ++s) {
@@ -517,7 +535,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         runs = 5 * rep > 4 * tot;  // four in five (measured: at three in four the chunked loop is still ahead)
         if (o.request_loop >= 0) runs = o.request_loop != 0;
         // (with one latency per (model, configuration) the loop over runs keeps a model's row of the table in a
-        // register, one entry per lane, whenever it produces more than the scores or the table does not fit in LDS)
+        // register, one entry per lane, and no table in LDS)
         if (uniform_stages && lat_row > kWave) runs = false;
     }
 
@@ -540,17 +558,19 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         wpb_cap = (int)std::min<int64_t>(wpb_cap, std::max<int64_t>(1, (waves_total + cus - 1) / cus));
     }
     if (o.waves_per_cu > 0) wpb_cap = std::min(kMaxWavesPerBlock, o.waves_per_cu);
-    // plain simulator, per wavefront: request block | replica bounds | clocks (one extra row that stays +inf)
+    // plain simulator, per wavefront: request block | replica bounds | clocks (chunked loop: one extra row that stays
+    // +inf; loop over runs: as many rows more as the walk of the tile reads past its slots, see tile_tail)
     // | slot counters | model counters; the latency table is shared by the workgroup
     size_t model_lds_bytes = 0;  // per-model counters [M][64] in LDS (decided below)
     bool group_in_lds = false;   // a 64-bit counter per (clock slot, lane) in LDS (decided below)
-    auto mixed_wave_bytes = [&](int ns) {
-        return ((size_t)mixed_clock_offset(rmax_lds_bytes, runs) + (size_t)(ns + 1) * kSlotBytes +
-                (group_in_lds ? (size_t)ns * kSlotBytes : 0) + model_lds_bytes + 15) & ~(size_t)15;
+    auto mixed_wave_bytes = [&](int ns, int tail_rows = 0) {
+        const size_t behind = (group_in_lds ? (size_t)ns * kSlotBytes : 0) + model_lds_bytes;  // what follows the clocks
+        const size_t slack = runs ? std::max((size_t)tail_rows * kSlotBytes, behind) : (size_t)kSlotBytes + behind;
+        return ((size_t)mixed_clock_offset(rmax_lds_bytes, runs) + (size_t)ns * kSlotBytes + slack + 15) & ~(size_t)15;
     };
     if (!batching) {
         wave_bytes = mixed_wave_bytes(nslots);  // of the largest placement
-        lat_bytes = runs && uniform_stages && more_than_scores ? 0 : (lat.size() * sizeof(float) + 15) & ~(size_t)15;  // (see above)
+        lat_bytes = runs && uniform_stages ? 0 : (lat.size() * sizeof(float) + 15) & ~(size_t)15;  // (see above)
         sched_bytes = runs ? (size_t)kSchedLdsBytes : 0;
         if (lat_bytes + sched_bytes + wave_bytes > (size_t)ctx->max_lds) {
             lat_in_lds = 0;
@@ -741,7 +761,27 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     //      that all items of a workgroup finish together however many regions there are.
     std::vector<int32_t> plan;
     if (!batching && runs) {
-        const size_t cap = (size_t)ctx->max_lds - lat_bytes - sched_bytes - lds_tail;
+        // Rows the walk of a tile can read past the tile's clock slots (power-of-two walk: every walking lane reads
+        // as many rows as the deepest walking lane, from its own group's first slot on).  They are part of the
+        // item's region, so that the reads stay inside the workgroup's LDS wherever the region lies; what is read
+        // there is never used.
+        std::vector<int32_t> tile_tail(b->tiles, 0);
+        if (pow2_depths && lds_tail > 0) {
+            std::vector<int32_t> deepest_of(b->tiles, 0), reach(b->tiles, 0);
+            for (int pass = 0; pass < 2; ++pass)
+                for (int32_t p = 0; p < B; ++p) {
+                    const int tile = b->pos[p] / kWave;
+                    for (int32_t g = 0; g < rl.num_groups[p]; ++g) {
+                        if (!group_hosts[(size_t)p * Gmax + g]) continue;
+                        if (pass == 0)
+                            deepest_of[tile] = std::max(deepest_of[tile], (int32_t)t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]]);
+                        else
+                            reach[tile] = std::max(reach[tile], (int32_t)slot0[(size_t)p * Gmax + g] + deepest_of[tile]);
+                    }
+                }
+            for (int32_t t2 = 0; t2 < b->tiles; ++t2) tile_tail[t2] = std::max(0, reach[t2] - tile_nslots[t2]);
+        }
+        lds_tail = 0;  // (the chunked loop keeps one tail behind the last wavefront's region instead)
         struct Item { int32_t tile, seed, bytes; };
         const int64_t n_items = (int64_t)b->waves;
         const int64_t cus = std::max(1, ctx->prop.multiProcessorCount);
@@ -749,7 +789,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         if (o.sched_groups > 0) groups = std::min<int64_t>(n_items, o.sched_groups);
         if (n_items > groups * kMaxGroupItems) return fail(MMSIM_E_UNSUPPORTED, "too many (tile, stream) pairs for one launch; split the batch");
         std::vector<int32_t> tile_bytes(b->tiles);
-        for (int32_t t2 = 0; t2 < b->tiles; ++t2) tile_bytes[t2] = (int32_t)mixed_wave_bytes(tile_nslots[t2]);
+        for (int32_t t2 = 0; t2 < b->tiles; ++t2) tile_bytes[t2] = (int32_t)mixed_wave_bytes(tile_nslots[t2], tile_tail[t2]);
         std::vector<int32_t> torder(b->tiles);
         for (int32_t t2 = 0; t2 < b->tiles; ++t2) torder[t2] = t2;
         std::stable_sort(torder.begin(), torder.end(), [&](int32_t x, int32_t y) { return tile_bytes[x] > tile_bytes[y]; });
@@ -773,6 +813,14 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                 per_group[(size_t)mine[(size_t)at]].push_back(per_xcd[x][i]);
             }
         }
+        // The schedule state is one word per item of a workgroup (never more than the kSchedLdsBytes the budget above
+        // set aside).
+        {
+            size_t most = 1;
+            for (const auto &its : per_group) most = std::max(most, its.size());
+            sched_bytes = std::min<size_t>(kSchedLdsBytes, (most * sizeof(uint32_t) + 15) & ~(size_t)15);
+        }
+        const size_t cap = (size_t)ctx->max_lds - lat_bytes - sched_bytes;
         int max_regions = kMaxWavesPerBlock;
         if (o.waves_per_cu > 0) max_regions = std::min(kMaxWavesPerBlock, o.waves_per_cu);
         int64_t seg_requests = 16384;
@@ -794,6 +842,14 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                     used += (size_t)its[i].bytes;
                     ++regions;
                 }
+            // Wavefronts k and k + 4 of a workgroup share a SIMD.  Regions come out largest first; with more than
+            // four, the second wavefronts of the SIMDs get theirs smallest first, so that the largest items meet
+            // the smallest ones: where every item has a wavefront of its own, the wavefront of a small item ends
+            // early and leaves the SIMD to the large one, and the four SIMDs end at about the same time.
+            for (int k = 4, l = regions - 1; k < l; ++k, --l) {
+                std::swap(part_off[(size_t)w * kMaxWavesPerBlock + k], part_off[(size_t)w * kMaxWavesPerBlock + l]);
+                std::swap(part_bytes[(size_t)w * kMaxWavesPerBlock + k], part_bytes[(size_t)w * kMaxWavesPerBlock + l]);
+            }
             if ((int)its.size() > regions) shared = true;
             lds_used = std::max(lds_used, used);
             waves_max = std::max(waves_max, regions);
@@ -867,13 +923,17 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
     // slot < 0 names the lane's +inf clock.
     // The loop over runs takes addresses relative to the wavefront's clock rows (its LDS region moves from turn to
     // turn) and sizes the rows by the tile; the chunked loop takes LDS addresses, every region as large as the largest.
+    // The loop over runs has no +inf row (LDS decides how many wavefronts a CU gets there): the missing entries of a
+    // lane that lists replicas repeat its first entry, flagged empty -- a copy never beats the entry it copies, since
+    // a tie goes to the entry listed first -- and those of a lane that lists none name its first clock slot; the
+    // kernel tells by the flag that such a lane found nothing.
     auto clock_addr = [&](int ps, int slot) {
         const int tile = ps / kWave, lane = ps % kWave;
         const uint32_t base = runs ? 0u : (uint32_t)(lat_bytes + (size_t)(tile % b->waves_per_block) * b->wave_bytes + mixed_clock_offset(rmax_lds_bytes, false));
-        const int inf_slot = runs ? tile_nslots[tile] : nslots;
+        const int inf_slot = runs ? 0 : nslots;
         return base + (uint32_t)(slot < 0 ? inf_slot : slot) * kSlotBytes + (uint32_t)lane * (uint32_t)sizeof(double);
     };
-    if (!batching) {  // missing replicas: the +inf clock and the +inf latency, flagged empty
+    if (!batching) {  // missing replicas: the +inf clock (see above) and the +inf latency, flagged empty
         const uint32_t inf_lat = (uint32_t)lat_off[C] << 18;
         parallel_slices(b->tiles, 8, [&](int64_t t0, int64_t t1) {
             for (int64_t tile = t0; tile < t1; ++tile) {
@@ -907,6 +967,7 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
             uint8_t &rm = rmax[(size_t)tile * M + m];
             rm = std::max<uint8_t>(rm, (uint8_t)(hi - lo));
             uint64_t word = none8;
+            uint32_t first_desc = 0;
             for (int64_t x = lo; x < hi; ++x) {
                 const int32_t g = rl.grp[(size_t)x];
                 const int j = (int)(x - lo);
@@ -923,12 +984,20 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
                     const int pp = t->cfg_pp[c];
                     const uint32_t d = pack_rep(clock_addr(b->pos[p], slot0[(size_t)p * Gmax + g] + pp - 1), (uint32_t)pp,
                                                 (uint32_t)(lat_off[c] + (uniform_stages ? 0 : pp - 1)));
+                    if (j == 0) first_desc = d;
                     if (j < kPackedReplicas)  // word j/4 of the lane, component j%4
                         rep32[((((size_t)tile * M + m) * 2 + (size_t)(j / 4)) * kWave + lane) * 4 + (size_t)(j % 4)] = d;
                     else
                         repx32[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = d;
                 }
             }
+            if (!batching && runs && hi > lo)  // (see clock_addr)
+                for (int j = (int)(hi - lo); j < kPackedReplicas + RX; ++j) {
+                    if (j < kPackedReplicas)
+                        rep32[((((size_t)tile * M + m) * 2 + (size_t)(j / 4)) * kWave + lane) * 4 + (size_t)(j % 4)] = first_desc | kEmpty;
+                    else
+                        repx32[(((size_t)tile * M + m) * RX + (size_t)(j - kPackedReplicas)) * kWave + lane] = first_desc | kEmpty;
+                }
             if (batching && !octets) rep8[((size_t)tile * M + m) * kWave + lane] = word;
         }
     }

@@ -67,7 +67,11 @@ __host__ __device__ inline uint32_t desc_group(uint32_t d) { return (d >> 23) & 
 //   bits 18..27  index of the group's LAST-stage latency in the model's row of
 //                the compact latency table
 //   bit  31      "no such replica"; the address then names the lane's clock
-//                that is +inf forever, so it never wins the choice
+//                that is +inf forever, so it never wins the choice (chunked
+//                loop), or the entry repeats the lane's first one, which
+//                wins every tie against its copies (loop over runs, which
+//                keeps no +inf clock; a lane without any replica names its
+//                first clock slot and is told by this bit)
 constexpr uint32_t kRepAddrMask = 0x3FFF8u;
 __host__ __device__ inline uint32_t pack_rep(uint32_t last_clock_addr, uint32_t stages, uint32_t lat_last) {
     const uint32_t sm1 = stages - 1u;

@@ -16,8 +16,9 @@
 //     stage count, index of its last-stage latency), eight per (tile, model,
 //     lane) in two 16-byte words rep32[tile][model][2][lane] (two coalesced
 //     1 KiB loads, listed in the order the reference scans them).
-//     Missing replicas point at a clock that is +inf forever, so the scan
-//     needs no validity test;
+//     Missing replicas point at a clock that is +inf forever (chunked loop)
+//     or repeat the lane's first replica, which wins every tie against its
+//     copies (loop over runs), so the scan itself needs no validity test;
 //   * per-lane stage clocks live in LDS as clk[slot][lane] (8 bytes each);
 //     the slots of a lane are its groups' pipeline stages laid end to end.
 //     The bank an access hits depends on the lane only, so any per-lane
@@ -242,18 +243,17 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     constexpr bool SCHED = RUNS;
 
     // ---- LDS: [latency table][schedule state (SCHED)][per wavefront: request block (chunked loop) | replica
-    //            bounds | clocks (+inf row last) | slot counters | model counters].
+    //            bounds | clocks (chunked loop: +inf row last) | slot counters | model counters].
     if (lds_addr(lds_raw) != 0u) {  // the descriptors assume the dynamic LDS starts at address 0
         if (threadIdx.x == 0) *a.error = 1;
         return;
     }
-    // Loop over runs with one latency per (model, configuration), any output beyond the scores: a run's model row
-    // of the latency table (at most 64 entries, the host sees to that) travels in a register, one entry per lane,
-    // and the latencies of the run's listed replicas are gathered from it across the lanes once per run; the table
-    // is not needed in LDS then, and a replica scan ends with the tournament instead of a dependent read of the
-    // winner's latency (configuration 4 with per-group counts: 592 ms against 605; scores only: 536 against 534,
-    // so the scores-only kernel keeps the table in LDS).
-    constexpr bool RUNLAT = RUNS && UNIFORM && OUT != 0;
+    // Loop over runs with one latency per (model, configuration): a run's model row of the latency table (at most
+    // 64 entries, the host sees to that) travels in a register, one entry per lane, and the latencies of the run's
+    // listed replicas are gathered from it across the lanes once per run; the table is not needed in LDS then (LDS
+    // decides how many wavefronts a CU gets), and a replica scan ends with the tournament instead of a dependent
+    // read of the winner's latency.
+    constexpr bool RUNLAT = RUNS && UNIFORM;
     constexpr bool TABLE_LDS = LATLDS && !RUNLAT;
     float *lat_lds = reinterpret_cast<float *>(lds_raw);
     const int lat_floats = TABLE_LDS ? a.M * a.lat_row : 0;
@@ -364,7 +364,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     const int nslots = SCHED ? a.item_nslots[item0 + item_k] : a.nslots;
     // Slot counters (group_lds): one row per clock row, behind the clocks.  The counter of the group whose last-stage
     // clock is at LDS address x is at x + cnt_rel: requests in the low half, accepted requests in the high half.
-    const uint32_t cnt_rel = (uint32_t)(nslots + 1) * kSlotBytes;
+    // (the loop over runs has no +inf row behind its clocks)
+    const uint32_t cnt_rel = (uint32_t)(nslots + (RUNS ? 0 : 1)) * kSlotBytes;
     unsigned long long *scnt = reinterpret_cast<unsigned long long *>(lds_raw + clk_off + cnt_rel) + lane;  // [nslots][64]
     uint32_t *mcnt = reinterpret_cast<uint32_t *>(lds_raw + clk_off + cnt_rel + (group_lds ? nslots * kSlotBytes : 0)) + lane;  // [M][64] accepted requests per model
 
@@ -391,7 +392,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
     } else {
         for (int s = 0; s < nslots; ++s) clk[s * kWave] = 0.0;
     }
-    clk[nslots * kWave] = __builtin_inf();
+    if constexpr (!RUNS) clk[nslots * kWave] = __builtin_inf();
     if (group_lds)
         for (int s = 0; s < nslots; ++s) scnt[s * kWave] = 0ull;  // of this turn; added to slot_cnt when it ends
 
@@ -477,7 +478,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
         //      stage and the latency of its last stage (needed by the early-reject bound).
         // Strictly smallest clock, first listed wins ties: a tournament whose left side wins ties
         // picks the same entry as the reference's left-to-right scan, in log2 dependent steps.
-        // Entries past a lane's own replicas are empty descriptors, whose clock reads +inf.
+        // Entries past a lane's own replicas are empty descriptors, whose clock reads +inf (chunked loop) or what
+        // the lane's first entry reads (loop over runs).
         struct Cand {
             double c;
             uint32_t d;
@@ -554,8 +556,10 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void sim_mixed_kernel(con
             ch_best = win.c;
             ch_l_last = (double)win.l;
             // what the walk needs of the chosen group, worked out once per choice
-            // (an empty descriptor points at the +inf row, so the clock alone tells whether a group was found)
-            const bool found = win.c < 1e100;
+            // (chunked loop: an empty descriptor points at the +inf row, so the clock alone tells whether a group was
+            // found; loop over runs: the empty entries of a lane repeat its first entry and lose every tie to it, so
+            // an empty entry wins only where the lane lists no replica at all)
+            const bool found = win.c < 1e100 && (!RUNS || (int32_t)win.d >= 0);
             const int stages_m1 = (int)rep_stages_m1(win.d);
             ch_sm1 = found ? stages_m1 : -1;
             ch_last = rep_addr(win.d) + rel_base;
