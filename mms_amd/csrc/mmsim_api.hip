@@ -469,14 +469,20 @@ int build_batch(mmsim_ctx *ctx, const mmsim_workload *const *wls, int32_t n_seed
         }
     for (int32_t p = 0; p < B; ++p) {
         int s = 0;
-        int32_t by_depth[MMSIM_MAX_GROUPS];
+        int32_t by_depth[MMSIM_MAX_GROUPS];  // the groups by (hosts anything ? stages : 0), a counting sort
         const int32_t ng = rl.num_groups[p];
-        for (int32_t g = 0; g < ng; ++g) by_depth[g] = g;
-        std::stable_sort(by_depth, by_depth + ng, [&](int32_t x, int32_t y) {
-            const int kx = group_hosts[(size_t)p * Gmax + x] ? t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + x]] : 0;
-            const int ky = group_hosts[(size_t)p * Gmax + y] ? t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + y]] : 0;
-            return kx < ky;
-        });
+        {
+            constexpr int kKeys = 34;  // 0, 1 .. 32 stages, more (refused below)
+            uint8_t key[MMSIM_MAX_GROUPS];
+            int32_t first[kKeys + 1] = {};
+            for (int32_t g = 0; g < ng; ++g) {
+                const int pp = t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]];
+                key[g] = (uint8_t)(group_hosts[(size_t)p * Gmax + g] ? std::min(pp, kKeys - 1) : 0);
+                first[key[g] + 1] += 1;
+            }
+            for (int k = 0; k < kKeys; ++k) first[k + 1] += first[k];
+            for (int32_t g = 0; g < ng; ++g) by_depth[first[key[g]]++] = g;
+        }
         for (int32_t k = 0; k < ng; ++k) {
             const int32_t g = by_depth[k];
             const int pp = t->cfg_pp[rl.group_cfg[(size_t)p * Gmax + g]];
