@@ -88,7 +88,9 @@ typedef struct {
     int32_t struct_size;          /* sizeof(mmsim_options), set by mmsim_options_default                      */
     int32_t request_loop;         /* plain simulator: 1 = loop over runs of equal models (scheduled launch),
                                      0 = chunks of four requests; -1: runs when at least four in five requests
-                                     of the batch's streams repeat the model of the request before            */
+                                     of the batch's streams repeat the model of the request before.  A latency
+                                     table with one latency per (model, configuration) and more than 63
+                                     configurations takes the chunks whatever this says                        */
     int32_t waves_per_cu;         /* 1..8: most wavefronts per workgroup of the plain simulator; 0: as many as fit */
     int32_t counts_in_lds;        /* counts of the plain simulator: 1 = counters in LDS, 0 = in registers and
                                      global rows; -1: LDS when that does not cost a CU wavefronts              */
