@@ -247,7 +247,8 @@ COUNTS_IN_LDS = -2          # the same counts, per-group counters in LDS
 
 @pytest.mark.parametrize("flags", [0, COUNTS_IN_REGISTERS, COUNTS_IN_LDS, ALL])
 @pytest.mark.parametrize("groups,regions,segment,spin", [(1, 1, 64, None), (3, 2, 256, None), (5, 8, 512, None),
-                                                        (64, 8, 16384, None), (1, 8, 64, 0), (2, 5, 128, 1)])
+                                                        (64, 8, 16384, None), (1, 8, 64, 0), (2, 5, 128, 1),
+                                                        (2, 8, 512, None)])
 def test_scheduled_launch_with_items_taking_turns(eng, opts, flags, groups, regions, segment, spin):
     """The loop over runs is launched as a schedule: a workgroup owns several (tile, stream) items, its
     LDS is cut into regions sized by the items' clock slots, and its wavefronts simulate the items a
@@ -256,7 +257,8 @@ def test_scheduled_launch_with_items_taking_turns(eng, opts, flags, groups, regi
     different sizes x 2 streams of odd, unequal lengths), every output level.  With ``spin`` 0 or 1 a
     wavefront that finds all the items it could take in other wavefronts' hands leaves at once instead
     of waiting (normally it would look again for about 70 ms): the holders then finish the items alone,
-    and every item must still be completed."""
+    and every item must still be completed.  Two workgroups with eight regions give each of the seven items of a
+    workgroup a wavefront of its own for the whole stream (one segment), large items sharing a SIMD with small ones."""
     from types import SimpleNamespace
     from mms_amd.profiling import ParallelConfig
     from mms_amd.placement_policy.base_policy import ModelPlacement
